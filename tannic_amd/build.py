@@ -1,0 +1,86 @@
+"""Builds ``tannic_amd/csrc/libtannic_hip.so`` with hipcc for gfx950.
+
+``python -m tannic_amd.build`` compiles every translation unit (in parallel)
+and links the shared library in-tree, next to the sources.
+"""
+import concurrent.futures
+import os
+import subprocess
+import sys
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+CSRC = os.path.join(HERE, "csrc")
+OBJ = os.path.join(CSRC, "build")
+LIB = os.path.join(CSRC, "libtannic_hip.so")
+
+HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+FLAGS = [
+    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC",
+    # packed fp32 instructions are kept out of the generated code
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-Wno-unused-command-line-argument",
+]
+
+# (source, object name, extra flags)
+UNITS = [
+    ("runtime.hip", "runtime.o", []),
+    ("unary.hip", "unary.o", []),
+    ("binary.hip", "binary_add.o", ["-DTH_BINARY_ONLY=0"]),
+    ("binary.hip", "binary_sub.o", ["-DTH_BINARY_ONLY=1"]),
+    ("binary.hip", "binary_mul.o", ["-DTH_BINARY_ONLY=2"]),
+    ("binary.hip", "binary_pow.o", ["-DTH_BINARY_ONLY=3"]),
+    ("misc.hip", "misc.o", []),
+    ("reduce.hip", "reduce.o", []),
+    ("gemm.hip", "gemm.o", []),
+    ("gemm_mfma.hip", "gemm_mfma.o", []),
+    ("conv2d.hip", "conv2d.o", []),
+    ("conv2d_mfma.hip", "conv2d_mfma.o", []),
+]
+
+
+def _headers():
+    found = [os.path.join(CSRC, f) for f in os.listdir(CSRC) if f.endswith(".hpp")]
+    found.append(os.path.join(HERE, "..", "include", "tannic_hip.h"))
+    return found
+
+
+def _stale(target, sources):
+    if not os.path.exists(target):
+        return True
+    t = os.path.getmtime(target)
+    return any(os.path.getmtime(s) > t for s in sources)
+
+
+def _compile(unit, force):
+    src, obj, extra = unit
+    src_path, obj_path = os.path.join(CSRC, src), os.path.join(OBJ, obj)
+    if not force and not _stale(obj_path, [src_path] + _headers()):
+        return obj_path, ""
+    cmd = [HIPCC] + FLAGS + extra + ["-c", src_path, "-o", obj_path]
+    proc = subprocess.run(cmd, capture_output=True, text=True)
+    noise = "is not a recognized feature for this target"
+    log = "\n".join(l for l in (proc.stdout + proc.stderr).splitlines() if noise not in l)
+    if proc.returncode != 0:
+        raise RuntimeError(f"hipcc failed on {src}:\n{log}")
+    return obj_path, log
+
+
+def build(force=True, jobs=None, verbose=False):
+    """Compiles all units (``force`` recompiles even up-to-date objects) and links."""
+    os.makedirs(OBJ, exist_ok=True)
+    jobs = jobs or min(8, os.cpu_count() or 1)
+    with concurrent.futures.ThreadPoolExecutor(max_workers=jobs) as pool:
+        results = list(pool.map(lambda u: _compile(u, force), UNITS))
+    for _, log in results:
+        if verbose and log.strip():
+            print(log)
+    objects = [o for o, _ in results]
+    cmd = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB] + objects
+    proc = subprocess.run(cmd, capture_output=True, text=True)
+    if proc.returncode != 0:
+        raise RuntimeError("link failed:\n" + proc.stdout + proc.stderr)
+    return LIB
+
+
+if __name__ == "__main__":
+    print(build(force="--incremental" not in sys.argv, verbose=True))

@@ -1,0 +1,146 @@
+// Shared definitions of the gfx950 device library: element types, error
+// reporting, launch helpers.  Internal to csrc/; the public surface is
+// include/tannic_hip.h.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include <cstdint>
+#include <cstdio>
+#include <cstring>
+#include <type_traits>
+
+#include "../../include/tannic_hip.h"
+
+namespace th {
+
+// ---- error reporting ------------------------------------------------------
+// The reference terminates the process on a runtime failure
+// (src/cuda/exc.cuh:8-16).  A C ABI that is also loaded into foreign hosts
+// must not do that: failures are recorded here and surface as TANNIC_ERROR.
+void set_error(const char* what, const char* file, int line, hipError_t code);
+void set_error_text(const char* text);
+
+#define TH_TRY(expr)                                               \
+    do {                                                           \
+        hipError_t th_err_ = (expr);                               \
+        if (th_err_ != hipSuccess) {                               \
+            ::th::set_error(#expr, __FILE__, __LINE__, th_err_);   \
+            return TANNIC_ERROR;                                   \
+        }                                                          \
+    } while (0)
+
+inline hipStream_t as_stream(tannic_stream_t s) { return reinterpret_cast<hipStream_t>(s.address); }
+
+// Result of the launch that was just enqueued.
+inline int launch_status(const char* what) {
+    hipError_t err = hipGetLastError();
+    if (err != hipSuccess) {
+        set_error(what, __FILE__, __LINE__, err);
+        return TANNIC_ERROR;
+    }
+    return TANNIC_SUCCESS;
+}
+
+// ---- element types --------------------------------------------------------
+using f16 = _Float16;
+
+// bfloat16 as raw bits; conversions are explicit so that every rounding is
+// visible: widening is exact, narrowing rounds to nearest even.
+struct bf16 {
+    uint16_t bits;
+};
+
+__host__ __device__ inline float to_float(bf16 v) {
+    union { uint32_t u; float f; } c;
+    c.u = static_cast<uint32_t>(v.bits) << 16;
+    return c.f;
+}
+
+__host__ __device__ inline bf16 to_bf16(float f) {
+    union { uint32_t u; float f; } c;
+    c.f = f;
+    bf16 r;
+    if ((c.u & 0x7FFFFFFFu) > 0x7F800000u) {
+        r.bits = static_cast<uint16_t>((c.u >> 16) | 0x40u);  // quiet NaN
+    } else {
+        r.bits = static_cast<uint16_t>((c.u + 0x7FFFu + ((c.u >> 16) & 1u)) >> 16);
+    }
+    return r;
+}
+
+template <class T>
+struct cplx {
+    T re, im;
+};
+using c64 = cplx<float>;
+using c128 = cplx<double>;
+
+template <class T> struct is_16bit { static constexpr bool value = false; };
+template <> struct is_16bit<f16> { static constexpr bool value = true; };
+template <> struct is_16bit<bf16> { static constexpr bool value = true; };
+
+// widen<T>: value of a 16-bit type as float, anything else unchanged
+__host__ __device__ inline float widen(f16 v) { return static_cast<float>(v); }
+__host__ __device__ inline float widen(bf16 v) { return to_float(v); }
+template <class T> __host__ __device__ inline T widen(T v) { return v; }
+
+// narrow<D>(x): x converted to D with one rounding
+template <class D, class X> __host__ __device__ inline D narrow(X x) {
+    if constexpr (std::is_same_v<D, bf16>) return to_bf16(static_cast<float>(x));
+    else return static_cast<D>(x);
+}
+
+template <class T> struct type_tag { using type = T; };
+
+// Calls f(type_tag<T>{}) for the element type of a dtype code.
+template <class F> inline bool with_type(int dtype, F&& f) {
+    switch (dtype) {
+        case TANNIC_INT8: f(type_tag<int8_t>{}); return true;
+        case TANNIC_INT16: f(type_tag<int16_t>{}); return true;
+        case TANNIC_INT32: f(type_tag<int32_t>{}); return true;
+        case TANNIC_INT64: f(type_tag<int64_t>{}); return true;
+        case TANNIC_FLOAT16: f(type_tag<f16>{}); return true;
+        case TANNIC_BFLOAT16: f(type_tag<bf16>{}); return true;
+        case TANNIC_FLOAT32: f(type_tag<float>{}); return true;
+        case TANNIC_FLOAT64: f(type_tag<double>{}); return true;
+        case TANNIC_COMPLEX64: f(type_tag<c64>{}); return true;
+        case TANNIC_COMPLEX128: f(type_tag<c128>{}); return true;
+        default: return false;
+    }
+}
+
+inline size_t dtype_size(int dtype) {
+    switch (dtype) {
+        case TANNIC_INT8: return 1;
+        case TANNIC_INT16: case TANNIC_FLOAT16: case TANNIC_BFLOAT16: return 2;
+        case TANNIC_INT32: case TANNIC_FLOAT32: return 4;
+        case TANNIC_INT64: case TANNIC_FLOAT64: case TANNIC_COMPLEX64: return 8;
+        case TANNIC_COMPLEX128: return 16;
+        default: return 0;
+    }
+}
+
+// ---- 32-bit division by a launch-time constant ------------------------------
+// q = n / d for n < 2^31 with one multiply-high, one add and one shift.
+struct FastDiv {
+    uint32_t d, magic, shift;
+    FastDiv() : d(1), magic(1), shift(0) {}
+    explicit FastDiv(uint32_t divisor) : d(divisor) {
+        for (shift = 0; shift < 32; ++shift)
+            if ((1u << shift) >= d) break;
+        const uint64_t one = 1;
+        magic = static_cast<uint32_t>(((one << 32) * ((one << shift) - d)) / d + 1);
+    }
+    __device__ inline uint32_t div(uint32_t n) const { return (__umulhi(n, magic) + n) >> shift; }
+    __device__ inline void divmod(uint32_t n, uint32_t& q, uint32_t& r) const {
+        q = div(n);
+        r = n - q * d;
+    }
+};
+
+// Work scratch obtained stream-ordered for the duration of one call.
+int scratch_acquire(void** ptr, size_t nbytes, hipStream_t stream);
+int scratch_release(void* ptr, hipStream_t stream);
+
+}  // namespace th

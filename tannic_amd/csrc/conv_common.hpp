@@ -1,0 +1,21 @@
+// Problem description shared by the convolution kernels.
+#pragma once
+
+#include "common.hpp"
+
+namespace th {
+
+// NCHW signal, OIHW kernel, cross-correlation with zero padding
+// (src/cpu/conv2d.cpp:17-64).  Strides are element strides of each operand.
+struct ConvProblem {
+    uint32_t N, C, H, W;       // signal
+    uint32_t O, KH, KW;        // kernel: O x C x KH x KW
+    uint32_t HO, WO;           // output spatial size
+    uint32_t pad_h, pad_w, stride_h, stride_w;
+    int64_t xs[4], ws[4], ys[4];
+    bool has_bias;
+};
+
+int conv2d_mfma(const ConvProblem& p, int dtype, const void* x, const void* w, const void* bias, void* y, hipStream_t stream);
+
+}  // namespace th

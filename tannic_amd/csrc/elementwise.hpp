@@ -1,0 +1,284 @@
+// The streaming engine behind every elementwise entry point.
+//
+// HBM-bound work: the goal is 16-byte accesses per lane, every byte of every
+// operand touched once, and index arithmetic cheap enough to hide behind the
+// memory stream.  No matrix cores are involved.
+//
+// Host side: the destination's index space and the operands' element strides
+// (size-1 dims already rewritten to stride 0, operands right-aligned on the
+// destination) are collapsed: dims of extent 1 vanish and neighbours that are
+// jointly contiguous for every operand merge.  A full-size contiguous operand
+// pair thus becomes ONE dim, X[64,4096,1024] (+) Z[1,4096,1] becomes three.
+//
+// Device side: the last collapsed dim is the "row".  A thread owns VEC
+// consecutive row elements (VEC*sizeof = 16 bytes); an operand whose row
+// stride is 0 is loaded once and splat.  The row number is decoded into outer
+// coordinates with multiply-shift division by launch-time constants.  When
+// alignment or strides rule out vectors the same kernel is instantiated with
+// VEC = 1 and arbitrary row strides.
+#pragma once
+
+#include "common.hpp"
+
+namespace th {
+
+constexpr int kMaxOperands = 3;  // two sources + destination
+
+struct Plan {
+    int rank;                              // collapsed rank, >= 1
+    uint32_t extent[TANNIC_DIMENSIONS];    // collapsed extents
+    FastDiv div[TANNIC_DIMENSIONS];        // division by extent[d]
+    int64_t stride[kMaxOperands][TANNIC_DIMENSIONS];  // element strides per operand
+    uint32_t row_vectors;                  // vectors per row (set at launch)
+    FastDiv row_div;                       // division by row_vectors
+    uint32_t total_vectors;                // rows * row_vectors
+};
+
+// Collapses `rank` dims.  strides[o][d] are element strides of operand o.
+// Returns false when the index space does not fit 31 bits.
+inline bool build_plan(Plan& p, int rank, const size_t* extent, const int64_t (*strides)[TANNIC_DIMENSIONS], int operands) {
+    size_t ext[TANNIC_DIMENSIONS];
+    int64_t st[kMaxOperands][TANNIC_DIMENSIONS];
+    int r = 0;
+    for (int d = 0; d < rank; ++d) {
+        if (extent[d] == 1) continue;
+        bool merged = false;
+        if (r > 0) {
+            merged = true;
+            for (int o = 0; o < operands; ++o)
+                if (st[o][r - 1] != strides[o][d] * static_cast<int64_t>(extent[d])) merged = false;
+            if (merged) {
+                ext[r - 1] *= extent[d];
+                for (int o = 0; o < operands; ++o) st[o][r - 1] = strides[o][d];
+            }
+        }
+        if (!merged) {
+            ext[r] = extent[d];
+            for (int o = 0; o < operands; ++o) st[o][r] = strides[o][d];
+            ++r;
+        }
+    }
+    if (r == 0) {
+        ext[0] = 1;
+        for (int o = 0; o < operands; ++o) st[o][0] = 1;
+        r = 1;
+    }
+    size_t total = 1;
+    for (int d = 0; d < r; ++d) {
+        if (ext[d] >= (1ull << 31)) return false;
+        total *= ext[d];
+        if (total >= (1ull << 31)) return false;
+    }
+    p.rank = r;
+    for (int d = 0; d < TANNIC_DIMENSIONS; ++d) {
+        p.extent[d] = d < r ? static_cast<uint32_t>(ext[d]) : 1;
+        p.div[d] = FastDiv(p.extent[d]);
+        for (int o = 0; o < kMaxOperands; ++o) p.stride[o][d] = (d < r && o < operands) ? st[o][d] : 0;
+    }
+    return true;
+}
+
+template <class T, int N>
+struct alignas(sizeof(T) * N >= 16 ? 16 : sizeof(T) * N) Pack {
+    T v[N];
+};
+
+// Register image of BYTES bytes that the memory instructions understand.
+template <int BYTES> struct RawBits;
+template <> struct RawBits<16> { using type = unsigned int __attribute__((ext_vector_type(4))); };
+template <> struct RawBits<8> { using type = unsigned int __attribute__((ext_vector_type(2))); };
+template <> struct RawBits<4> { using type = unsigned int; };
+template <> struct RawBits<2> { using type = unsigned short; };
+template <> struct RawBits<1> { using type = unsigned char; };
+
+#ifndef TH_NONTEMPORAL
+#define TH_NONTEMPORAL 1
+#endif
+
+// Loads N consecutive elements with one access of sizeof(T)*N bytes.  Operand
+// streams are read once and results written once, so both bypass temporal
+// caching.
+template <class T, int N>
+__device__ inline Pack<T, N> load_pack(const T* p) {
+    static_assert(sizeof(T) * N <= 16, "a pack is at most 16 bytes");
+    using Raw = typename RawBits<sizeof(T) * N>::type;
+#if TH_NONTEMPORAL
+    const Raw raw = __builtin_nontemporal_load(reinterpret_cast<const Raw*>(p));
+#else
+    const Raw raw = *reinterpret_cast<const Raw*>(p);
+#endif
+    Pack<T, N> r;
+    __builtin_memcpy(&r, &raw, sizeof r);
+    return r;
+}
+
+template <class T, int N>
+__device__ inline void store_pack(T* p, const Pack<T, N>& v) {
+    using Raw = typename RawBits<sizeof(T) * N>::type;
+    Raw raw;
+    __builtin_memcpy(&raw, &v, sizeof raw);
+#if TH_NONTEMPORAL
+    __builtin_nontemporal_store(raw, reinterpret_cast<Raw*>(p));
+#else
+    *reinterpret_cast<Raw*>(p) = raw;
+#endif
+}
+
+template <class T, int N>
+__device__ inline Pack<T, N> load_or_splat(const T* p, bool splat) {
+    if (!splat) return load_pack<T, N>(p);
+    Pack<T, N> r;
+    const T s = *p;
+#pragma unroll
+    for (int i = 0; i < N; ++i) r.v[i] = s;
+    return r;
+}
+
+constexpr int kBlock = 256;
+constexpr int kUnroll = 4;
+
+// Element offsets of vector `v` in the three operands.
+struct Offsets {
+    int64_t o0, o1, od;
+};
+
+template <int VEC>
+__device__ inline Offsets decode(const Plan& p, uint32_t v) {
+    const int last = p.rank - 1;
+    uint32_t row, col;
+    p.row_div.divmod(v, row, col);
+    col *= VEC;
+    Offsets o;
+    o.o0 = static_cast<int64_t>(col) * p.stride[0][last];
+    o.o1 = static_cast<int64_t>(col) * p.stride[1][last];
+    o.od = static_cast<int64_t>(col) * p.stride[2][last];
+    for (int d = last - 1; d >= 0; --d) {
+        uint32_t q, c;
+        p.div[d].divmod(row, q, c);
+        row = q;
+        o.o0 += static_cast<int64_t>(c) * p.stride[0][d];
+        o.o1 += static_cast<int64_t>(c) * p.stride[1][d];
+        o.od += static_cast<int64_t>(c) * p.stride[2][d];
+    }
+    return o;
+}
+
+// F: { using S0, S1, D; static constexpr int sources; const S0* a; const S1* b; D* out;
+//      __device__ D operator()(S0, S1) const; }   (S1/b unused when sources == 1)
+template <class F, int VEC>
+__global__ __launch_bounds__(kBlock) void elementwise_kernel(F f, Plan p) {
+    using S0 = typename F::S0;
+    using S1 = typename F::S1;
+    using D = typename F::D;
+    const int last = p.rank - 1;
+    const bool splat0 = p.stride[0][last] == 0;
+    const bool splat1 = p.stride[1][last] == 0;
+    const uint32_t base = blockIdx.x * (kBlock * kUnroll) + threadIdx.x;
+    if constexpr (VEC == 1) {
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u) {
+            const uint32_t v = base + u * kBlock;
+            if (v < p.total_vectors) {
+                const Offsets o = decode<1>(p, v);
+                if constexpr (F::sources == 2) f.out[o.od] = f(f.a[o.o0], f.b[o.o1]);
+                else f.out[o.od] = f(f.a[o.o0], S1{});
+            }
+        }
+    } else {
+        // all loads of the unrolled group are issued before any store
+        Pack<S0, VEC> a[kUnroll];
+        Pack<S1, VEC> b[kUnroll];
+        Offsets o[kUnroll];
+        bool live[kUnroll];
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u) {
+            const uint32_t v = base + u * kBlock;
+            live[u] = v < p.total_vectors;
+            if (live[u]) {
+                o[u] = decode<VEC>(p, v);
+                a[u] = load_or_splat<S0, VEC>(f.a + o[u].o0, splat0);
+                if constexpr (F::sources == 2) b[u] = load_or_splat<S1, VEC>(f.b + o[u].o1, splat1);
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u) {
+            if (live[u]) {
+                Pack<D, VEC> r;
+#pragma unroll
+                for (int i = 0; i < VEC; ++i) {
+                    if constexpr (F::sources == 2) r.v[i] = f(a[u].v[i], b[u].v[i]);
+                    else r.v[i] = f(a[u].v[i], S1{});
+                }
+                store_pack<D, VEC>(f.out + o[u].od, r);
+            }
+        }
+    }
+}
+
+template <class A, class B>
+constexpr size_t max_size() { return sizeof(A) > sizeof(B) ? sizeof(A) : sizeof(B); }
+
+// Whether operand `o` allows VEC-wide access: row stride 0 or 1, every outer
+// stride and the base address multiples of the vector.
+template <class T>
+inline bool vector_ok(const Plan& p, int o, const T* ptr, int vec, bool is_dst) {
+    const int last = p.rank - 1;
+    const int64_t rs = p.stride[o][last];
+    if (is_dst ? rs != 1 : (rs != 0 && rs != 1)) return false;
+    if (rs == 0) return true;  // splat operand: scalar loads, no alignment needed
+    if (reinterpret_cast<uintptr_t>(ptr) % (sizeof(T) * vec)) return false;
+    for (int d = 0; d < last; ++d)
+        if (p.stride[o][d] % vec) return false;
+    return true;
+}
+
+// Enqueues F over the plan.  Destination operand index is 2.
+template <class F>
+int launch_elementwise(F f, Plan p, hipStream_t stream) {
+    using S0 = typename F::S0;
+    using S1 = typename F::S1;
+    using D = typename F::D;
+    constexpr size_t widest = F::sources == 2 ? (max_size<S0, S1>() > sizeof(D) ? max_size<S0, S1>() : sizeof(D))
+                                              : max_size<S0, D>();
+    constexpr int VEC = widest >= 16 ? 1 : static_cast<int>(16 / widest);
+    const int last = p.rank - 1;
+    uint32_t rows = 1;
+    for (int d = 0; d < last; ++d) rows *= p.extent[d];
+    bool vec = VEC > 1 && p.extent[last] % VEC == 0 && vector_ok(p, 0, f.a, VEC, false) &&
+               vector_ok(p, 2, f.out, VEC, true);
+    if (F::sources == 2) vec = vec && vector_ok(p, 1, f.b, VEC, false);
+    p.row_vectors = vec ? p.extent[last] / VEC : p.extent[last];
+    p.row_div = FastDiv(p.row_vectors);
+    p.total_vectors = rows * p.row_vectors;
+    if (p.total_vectors == 0) return TANNIC_SUCCESS;
+    const uint32_t grid = (p.total_vectors + kBlock * kUnroll - 1) / (kBlock * kUnroll);
+    if constexpr (VEC > 1) {
+        if (vec) {
+            hipLaunchKernelGGL((elementwise_kernel<F, VEC>), dim3(grid), dim3(kBlock), 0, stream, f, p);
+            return launch_status("elementwise_kernel");
+        }
+    }
+    hipLaunchKernelGGL((elementwise_kernel<F, 1>), dim3(grid), dim3(kBlock), 0, stream, f, p);
+    return launch_status("elementwise_kernel");
+}
+
+// Strides of `t` right-aligned on a destination of `rank` dims with `extent`;
+// size-1 dims (and missing leading dims) get stride 0
+// (src/cpu/ops-binary.cpp:89-95).
+inline void aligned_strides(const tannic_tensor_t* t, int rank, int64_t* out) {
+    const int off = rank - t->rank;
+    for (int d = 0; d < rank; ++d) {
+        if (d < off) { out[d] = 0; continue; }
+        out[d] = t->shape.sizes[d - off] == 1 ? 0 : t->strides.sizes[d - off];
+    }
+}
+
+inline void contiguous_strides(int rank, const size_t* extent, int64_t* out) {
+    int64_t run = 1;
+    for (int d = rank - 1; d >= 0; --d) {
+        out[d] = run;
+        run *= static_cast<int64_t>(extent[d]);
+    }
+}
+
+}  // namespace th

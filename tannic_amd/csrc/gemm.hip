@@ -1,0 +1,196 @@
+// gemm entry point: problem description, dtype table, generic kernel.
+//
+// Destination type per operand pair as in src/cpu/matmul.cpp:189-252.  The
+// 16-bit same-type pairs and fp32 go to the MFMA kernels (gemm_mfma.hip) when
+// their layout conditions hold; every other pair, and the leftovers, run the
+// LDS-tiled scalar kernel below, which accepts any strides.
+//
+// Differences from the reference CPU path, all documented at the ABI:
+//   - f16 x f16 and bf16 x bf16 accumulate in fp32 and round once (the CPU
+//     path accumulates in the 16-bit type);
+//   - fp32 sums are formed in a different order (tiles of K);
+//   - batch counts above 255 are handled (the CPU path narrows the batch
+//     counter to uint8_t, src/cpu/matmul.cpp:102).
+#include "gemm_common.hpp"
+
+namespace th {
+
+static bool is_transposed(const tannic_tensor_t* t) {
+    if (t->rank < 2) return false;
+    return t->strides.sizes[t->rank - 1] > t->strides.sizes[t->rank - 2];
+}
+
+int describe_gemm(const tannic_tensor_t* a, const tannic_tensor_t* b, const tannic_tensor_t* c, GemmProblem& p) {
+    if (a->rank < 2 || b->rank < 2 || c->rank < 2 || c->rank > 8) {
+        set_error_text("gemm: operands must have rank >= 2");
+        return TANNIC_ERROR;
+    }
+    const size_t M = c->shape.sizes[c->rank - 2], N = c->shape.sizes[c->rank - 1], K = a->shape.sizes[a->rank - 1];
+    if (M >= (1ull << 31) || N >= (1ull << 31) || K >= (1ull << 31)) {
+        set_error_text("gemm: dimension of 2^31 or more");
+        return TANNIC_ERROR;
+    }
+    p.M = static_cast<uint32_t>(M);
+    p.N = static_cast<uint32_t>(N);
+    p.K = static_cast<uint32_t>(K);
+    // a transposed view is recognised by its strides; its leading dimension is
+    // the larger stride and the other one is taken to be 1
+    const bool at = is_transposed(a), bt = is_transposed(b);
+    const int64_t lda = at ? a->strides.sizes[a->rank - 1] : a->strides.sizes[a->rank - 2];
+    const int64_t ldb = bt ? b->strides.sizes[b->rank - 1] : b->strides.sizes[b->rank - 2];
+    p.a_rs = at ? 1 : lda;
+    p.a_cs = at ? lda : 1;
+    p.b_rs = bt ? 1 : ldb;
+    p.b_cs = bt ? ldb : 1;
+    p.c_rs = c->strides.sizes[c->rank - 2];
+    p.batch_rank = c->rank - 2;
+    p.batches = 1;
+    for (int d = 0; d < 6; ++d) {
+        p.batch_extent[d] = 1;
+        p.a_bs[d] = p.b_bs[d] = p.c_bs[d] = 0;
+    }
+    size_t batches = 1;
+    for (int d = 0; d < p.batch_rank; ++d) {
+        p.batch_extent[d] = static_cast<uint32_t>(c->shape.sizes[d]);
+        batches *= c->shape.sizes[d];
+        p.c_bs[d] = c->strides.sizes[d];
+        // src/cpu/matmul.cpp:107-118: the coordinate of an operand is looked up
+        // right-aligned (size-1 and missing dims give 0) and multiplied by the
+        // stride stored at position d of that operand
+        auto stride_of = [&](const tannic_tensor_t* s) -> int64_t {
+            const int sd = d + (s->rank - c->rank);
+            if (sd < 0 || s->shape.sizes[sd] == 1 || d >= s->rank) return 0;
+            return s->strides.sizes[d];
+        };
+        p.a_bs[d] = stride_of(a);
+        p.b_bs[d] = stride_of(b);
+    }
+    if (batches >= (1ull << 31)) {
+        set_error_text("gemm: too many batches");
+        return TANNIC_ERROR;
+    }
+    p.batches = static_cast<uint32_t>(batches);
+    return TANNIC_SUCCESS;
+}
+
+template <class A, class B> struct GemmResult {
+    static auto pick() {
+        constexpr bool ia = std::is_integral_v<A>, ib = std::is_integral_v<B>;
+        constexpr bool ha = is_16bit<A>::value, hb = is_16bit<B>::value;
+        constexpr bool ca = std::is_same_v<A, c64> || std::is_same_v<A, c128>, cb = std::is_same_v<B, c64> || std::is_same_v<B, c128>;
+        if constexpr (ca || cb) return type_tag<void>{};
+        else if constexpr (ia && ib) {
+            if constexpr (sizeof(A) == 8 || sizeof(B) == 8 || (sizeof(A) == 4 && sizeof(B) == 4)) return type_tag<int64_t>{};
+            else return type_tag<int32_t>{};
+        } else if constexpr (ha && hb) {
+            if constexpr (std::is_same_v<A, B>) return type_tag<A>{}; else return type_tag<void>{};
+        } else if constexpr (ha || hb) {
+            using O = std::conditional_t<ha, B, A>;
+            if constexpr (std::is_same_v<O, double> || std::is_same_v<O, int64_t>) return type_tag<double>{};
+            else return type_tag<float>{};
+        } else if constexpr (ia || ib) {
+            using I = std::conditional_t<ia, A, B>;
+            using F = std::conditional_t<ia, B, A>;
+            if constexpr (std::is_same_v<I, int32_t>) return type_tag<F>{}; else return type_tag<void>{};
+        } else {
+            if constexpr (std::is_same_v<A, double> || std::is_same_v<B, double>) return type_tag<double>{};
+            else return type_tag<float>{};
+        }
+    }
+    using type = typename decltype(pick())::type;
+};
+
+// 64x64 output tile per block of 256 threads, 4x4 outputs per thread, K in
+// steps of 16 through LDS.  Products are formed in the accumulator type
+// (static_cast<D>(a) * static_cast<D>(b), src/cpu/matmul.cpp:36) — fp32 for a
+// 16-bit destination.
+template <class A, class B, class D>
+__global__ __launch_bounds__(256) void gemm_generic_kernel(const A* a, const B* b, D* c, GemmProblem p) {
+    using Acc = std::conditional_t<is_16bit<D>::value, float, D>;
+    constexpr int T = 64, KT = 16;
+    __shared__ Acc sa[KT][T + 1];
+    __shared__ Acc sb[KT][T + 1];
+    int64_t oa, ob, oc;
+    batch_offsets(p, blockIdx.z, oa, ob, oc);
+    a += oa;
+    b += ob;
+    c += oc;
+    const uint32_t m0 = blockIdx.y * T, n0 = blockIdx.x * T;
+    const int tx = threadIdx.x % 16, ty = threadIdx.x / 16;
+    Acc acc[4][4] = {};
+    for (uint32_t k0 = 0; k0 < p.K; k0 += KT) {
+        for (int i = threadIdx.x; i < T * KT; i += 256) {
+            // A tile: consecutive threads along k when k is the contiguous index, else along m
+            const int kk = p.a_cs == 1 ? i % KT : i / T, mm = p.a_cs == 1 ? i / KT : i % T;
+            const uint32_t m = m0 + mm, k = k0 + kk;
+            sa[kk][mm] = (m < p.M && k < p.K) ? static_cast<Acc>(widen(a[m * p.a_rs + k * p.a_cs])) : Acc(0);
+            const int kb = p.b_rs == 1 ? i % KT : i / T, nn = p.b_rs == 1 ? i / KT : i % T;
+            const uint32_t n = n0 + nn, k2 = k0 + kb;
+            sb[kb][nn] = (n < p.N && k2 < p.K) ? static_cast<Acc>(widen(b[k2 * p.b_rs + n * p.b_cs])) : Acc(0);
+        }
+        __syncthreads();
+#pragma unroll
+        for (int kk = 0; kk < KT; ++kk) {
+            Acc x[4], y[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) { x[i] = sa[kk][ty * 4 + i]; y[i] = sb[kk][tx * 4 + i]; }
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) acc[i][j] += x[i] * y[j];
+        }
+        __syncthreads();
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const uint32_t m = m0 + ty * 4 + i, n = n0 + tx * 4 + j;
+            if (m < p.M && n < p.N) c[m * p.c_rs + n] = narrow<D>(acc[i][j]);
+        }
+}
+
+template <class A, class B, class D>
+int run_generic(const GemmProblem& p, const void* a, const void* b, void* c, hipStream_t stream) {
+    if (p.M == 0 || p.N == 0 || p.batches == 0) return TANNIC_SUCCESS;
+    const uint32_t gx = (p.N + 63) / 64, gy = (p.M + 63) / 64;
+    if (gy > 65535 || p.batches > 65535) {
+        set_error_text("gemm: generic kernel grid limit exceeded");
+        return TANNIC_ERROR;
+    }
+    hipLaunchKernelGGL((gemm_generic_kernel<A, B, D>), dim3(gx, gy, p.batches), dim3(256), 0, stream, static_cast<const A*>(a),
+                       static_cast<const B*>(b), static_cast<D*>(c), p);
+    return launch_status("gemm_generic_kernel");
+}
+
+}  // namespace th
+
+using namespace th;
+
+extern "C" int tannic_hip_gemm(const tannic_tensor_t* a, const tannic_tensor_t* b, tannic_tensor_t* dst, tannic_stream_t stream) {
+    if (!a || !b || !dst) return TANNIC_ERROR;
+    int status = TANNIC_UNSUPPORTED_DTYPE;
+    hipStream_t s = as_stream(stream);
+    with_type(a->dtype, [&](auto ta) {
+        with_type(b->dtype, [&](auto tb) {
+            using A = typename decltype(ta)::type;
+            using B = typename decltype(tb)::type;
+            using D = typename GemmResult<A, B>::type;
+            if constexpr (!std::is_void_v<D>) {
+                GemmProblem p;
+                status = describe_gemm(a, b, dst, p);
+                if (status != TANNIC_SUCCESS) return;
+                if constexpr (std::is_same_v<A, B> && is_16bit<A>::value) {
+                    status = gemm_mfma_16bit(p, a->dtype, a->address, b->address, dst->address, s);
+                    if (status != TANNIC_UNSUPPORTED_DTYPE) return;
+                } else if constexpr (std::is_same_v<A, float> && std::is_same_v<B, float>) {
+                    status = gemm_mfma_f32(p, static_cast<const float*>(a->address), static_cast<const float*>(b->address),
+                                           static_cast<float*>(dst->address), s);
+                    if (status != TANNIC_UNSUPPORTED_DTYPE) return;
+                }
+                status = run_generic<A, B, D>(p, a->address, b->address, dst->address, s);
+            }
+        });
+    });
+    return status;
+}

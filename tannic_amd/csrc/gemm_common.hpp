@@ -1,0 +1,44 @@
+// Problem description shared by the matrix-multiply kernels.
+#pragma once
+
+#include "common.hpp"
+
+namespace th {
+
+// One batched product C[b] = A[b] * B[b].  Operands are addressed as
+// base + batch_offset + row * rs + col * cs (element strides), which covers the
+// four plain/transposed combinations the reference derives from strides
+// (src/cpu/matmul.cpp:87-94, :132-137).
+struct GemmProblem {
+    uint32_t M, N, K;
+    int64_t a_rs, a_cs;  // A[m,k]
+    int64_t b_rs, b_cs;  // B[k,n]
+    int64_t c_rs;        // C[m,n], column stride 1
+    // batch dims of the destination, outermost first
+    int batch_rank;
+    uint32_t batches;
+    uint32_t batch_extent[6];
+    int64_t a_bs[6], b_bs[6], c_bs[6];
+};
+
+__host__ __device__ inline void batch_offsets(const GemmProblem& p, uint32_t batch, int64_t& oa, int64_t& ob, int64_t& oc) {
+    oa = ob = oc = 0;
+    for (int d = p.batch_rank - 1; d >= 0; --d) {
+        const uint32_t idx = batch % p.batch_extent[d];
+        batch /= p.batch_extent[d];
+        oa += static_cast<int64_t>(idx) * p.a_bs[d];
+        ob += static_cast<int64_t>(idx) * p.b_bs[d];
+        oc += static_cast<int64_t>(idx) * p.c_bs[d];
+    }
+}
+
+// Fills `p` from the descriptors the way launchGemmKernel does
+// (src/cpu/matmul.cpp:126-176).  Returns a status.
+int describe_gemm(const tannic_tensor_t* a, const tannic_tensor_t* b, const tannic_tensor_t* c, GemmProblem& p);
+
+// MFMA paths; each returns TANNIC_UNSUPPORTED_DTYPE when the problem does not
+// meet its layout/alignment conditions so that the caller can fall back.
+int gemm_mfma_16bit(const GemmProblem& p, int dtype, const void* a, const void* b, void* c, hipStream_t stream);
+int gemm_mfma_f32(const GemmProblem& p, const float* a, const float* b, float* c, hipStream_t stream);
+
+}  // namespace th

@@ -1,0 +1,467 @@
+// Axis reductions: argsum, argmean, argmax, argmin (+ value max / min).
+//
+// HBM-bound: every source byte is read once with 16-byte accesses.  A
+// contiguous source is seen as [outer, R, inner] (src/cpu/argred.cpp:186-212):
+//   inner == 1  -> "rows":    a wavefront (or a whole block) owns a row, lanes
+//                             stride over it, partials meet in a DPP tree and,
+//                             for block-wide rows, in LDS;
+//   inner  > 1  -> "columns": a lane owns VEC adjacent columns so that a
+//                             wavefront reads contiguous bytes, the waves of
+//                             a block (and, when the output is small, several
+//                             blocks) take interleaved slices of R; partials
+//                             meet in LDS, then in a second small pass.
+// Strided sources take a one-thread-per-output walk.
+//
+// Arithmetic follows src/cpu/argred.cpp:151-181 with two documented
+// differences: partial sums are combined as a tree (fp32 results differ from
+// the sequential CPU sum within rounding), and 16-bit sums accumulate in fp32
+// and round once.  Integer sums wrap exactly as the sequential sum does.
+// argmax/argmin: strict comparison from a -inf/+inf (lowest/max) start, lowest
+// index wins ties, NaN never wins (src/cpu/argred.cpp:95-101, :317-347).
+#include "common.hpp"
+
+namespace th {
+
+constexpr int kWave = 64;
+constexpr int kThreads = 256;
+
+// ---- moving values between lanes -------------------------------------------
+template <int CTRL>
+__device__ inline uint32_t dpp32(uint32_t v) {
+    return static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, static_cast<int>(v), CTRL, 0xF, 0xF, false));
+}
+
+template <int CTRL, class T>
+__device__ inline T dpp(T v) {
+    static_assert(sizeof(T) % 4 == 0, "DPP moves 32-bit registers");
+    uint32_t w[sizeof(T) / 4];
+    __builtin_memcpy(w, &v, sizeof(T));
+#pragma unroll
+    for (size_t i = 0; i < sizeof(T) / 4; ++i) w[i] = dpp32<CTRL>(w[i]);
+    T r;
+    __builtin_memcpy(&r, w, sizeof(T));
+    return r;
+}
+
+template <class T>
+__device__ inline T read_lane(T v, int lane) {
+    uint32_t w[sizeof(T) / 4];
+    __builtin_memcpy(w, &v, sizeof(T));
+#pragma unroll
+    for (size_t i = 0; i < sizeof(T) / 4; ++i) w[i] = static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(w[i]), lane));
+    T r;
+    __builtin_memcpy(&r, w, sizeof(T));
+    return r;
+}
+
+// All 64 lanes -> one value, identical in every lane.  Four DPP steps fold
+// each row of 16 lanes (quad swaps, half-row mirror, row mirror), the four row
+// results are read out as scalars.
+template <class Op, class A>
+__device__ inline A wave_reduce(A v) {
+    v = Op::combine(v, dpp<0xB1>(v));   // quad_perm [1,0,3,2]
+    v = Op::combine(v, dpp<0x4E>(v));   // quad_perm [2,3,0,1]
+    v = Op::combine(v, dpp<0x141>(v));  // row_half_mirror
+    v = Op::combine(v, dpp<0x140>(v));  // row_mirror
+    const A r0 = read_lane(v, 0), r1 = read_lane(v, 16), r2 = read_lane(v, 32), r3 = read_lane(v, 48);
+    return Op::combine(Op::combine(r0, r1), Op::combine(r2, r3));
+}
+
+// ---- reduction policies -------------------------------------------------------
+template <class T> struct SumAcc { using type = T; };
+template <> struct SumAcc<f16> { using type = float; };
+template <> struct SumAcc<bf16> { using type = float; };
+template <> struct SumAcc<int8_t> { using type = uint32_t; };   // wraps; narrowed at the end
+template <> struct SumAcc<int16_t> { using type = uint32_t; };
+template <> struct SumAcc<int32_t> { using type = uint32_t; };
+template <> struct SumAcc<int64_t> { using type = uint64_t; };
+
+template <class T, bool MEAN>
+struct SumOp {
+    using S = T;
+    using A = typename SumAcc<T>::type;
+    using Out = T;
+    static constexpr bool needs_source = false;
+    __device__ static inline A init() { return A(0); }
+    __device__ static inline A step(A acc, T v, uint32_t) {
+        if constexpr (std::is_integral_v<T>) return acc + static_cast<A>(v);
+        else return acc + static_cast<A>(widen(v));
+    }
+    __device__ static inline A combine(A x, A y) { return x + y; }
+    __device__ static inline Out finish(A acc, uint32_t count) {
+        if constexpr (MEAN) return narrow<T>(acc / static_cast<A>(count));
+        else if constexpr (std::is_integral_v<T>) return static_cast<T>(acc);
+        else return narrow<T>(acc);
+    }
+};
+
+template <class T>
+struct Best {
+    T value;
+    uint32_t index;
+};
+template <> struct Best<f16> { f16 value; uint16_t pad; uint32_t index; };
+template <> struct Best<bf16> { bf16 value; uint16_t pad; uint32_t index; };
+template <> struct Best<int8_t> { int8_t value; int8_t pad[3]; uint32_t index; };
+template <> struct Best<int16_t> { int16_t value; int16_t pad; uint32_t index; };
+template <> struct Best<double> { double value; uint32_t index; uint32_t pad; };
+template <> struct Best<int64_t> { int64_t value; uint32_t index; uint32_t pad; };
+
+template <class T> __device__ inline bool gt(T a, T b) {
+    if constexpr (std::is_same_v<T, bf16>) return to_float(a) > to_float(b); else return a > b;
+}
+template <class T> __device__ inline bool same(T a, T b) {
+    if constexpr (std::is_same_v<T, bf16>) return to_float(a) == to_float(b); else return a == b;
+}
+
+template <class T, bool MAX> __device__ inline T arg_start() {
+    if constexpr (std::is_same_v<T, int8_t>) return MAX ? INT8_MIN : INT8_MAX;
+    else if constexpr (std::is_same_v<T, int16_t>) return MAX ? INT16_MIN : INT16_MAX;
+    else if constexpr (std::is_same_v<T, int32_t>) return MAX ? INT32_MIN : INT32_MAX;
+    else if constexpr (std::is_same_v<T, int64_t>) return MAX ? INT64_MIN : INT64_MAX;
+    else if constexpr (std::is_same_v<T, bf16>) return bf16{static_cast<uint16_t>(MAX ? 0xFF80u : 0x7F80u)};
+    else return static_cast<T>(MAX ? -__builtin_inff() : __builtin_inff());
+}
+
+// VALUE = false: int64 index out.  VALUE = true: the source element at that index.
+template <class T, bool MAX, bool VALUE>
+struct ArgOp {
+    using S = T;
+    using A = Best<T>;
+    using Out = std::conditional_t<VALUE, T, int64_t>;
+    static constexpr bool needs_source = VALUE;
+    __device__ static inline A init() {
+        A a{};
+        a.value = arg_start<T, MAX>();
+        a.index = 0;
+        return a;
+    }
+    __device__ static inline bool better(T v, uint32_t i, const A& than) {
+        const bool strictly = MAX ? gt(v, than.value) : gt(than.value, v);
+        return strictly || (same(v, than.value) && i < than.index);
+    }
+    __device__ static inline A step(A acc, T v, uint32_t r) {
+        if (better(v, r, acc)) { acc.value = v; acc.index = r; }
+        return acc;
+    }
+    __device__ static inline A combine(A x, A y) { return better(y.value, y.index, x) ? y : x; }
+    __device__ static inline int64_t finish(A acc, uint32_t) { return static_cast<int64_t>(acc.index); }
+};
+
+template <class T, int N>
+struct alignas(sizeof(T) * N >= 16 ? 16 : sizeof(T) * N) Vec {
+    T v[N];
+};
+
+template <class T, int N>
+__device__ inline Vec<T, N> load_vec(const T* p) {
+    if constexpr (N == 1) {
+        Vec<T, 1> r;
+        r.v[0] = *p;
+        return r;
+    } else {
+        using Raw = unsigned int __attribute__((ext_vector_type(sizeof(T) * N / 4)));
+        const Raw raw = __builtin_nontemporal_load(reinterpret_cast<const Raw*>(p));
+        Vec<T, N> r;
+        __builtin_memcpy(&r, &raw, sizeof r);
+        return r;
+    }
+}
+
+// Writes the result for output slot `slot`.  `first` / `step` locate the slice
+// in the source for value reductions.
+template <class Op>
+__device__ inline void emit(typename Op::A acc, uint32_t count, typename Op::Out* dst, size_t slot,
+                            const typename Op::S* src, size_t first, size_t step) {
+    if constexpr (Op::needs_source) dst[slot] = src[first + static_cast<size_t>(acc.index) * step];
+    else dst[slot] = Op::finish(acc, count);
+}
+
+// ---- rows: inner == 1 ----------------------------------------------------------
+// WAVES waves cooperate on one row; a block of 256 threads holds 4 / WAVES rows.
+template <class Op, int VEC, int WAVES>
+__global__ __launch_bounds__(kThreads) void reduce_rows_kernel(const typename Op::S* src, typename Op::Out* dst, uint32_t rows, uint32_t R) {
+    using A = typename Op::A;
+    using T = typename Op::S;
+    constexpr int ROWS_PER_BLOCK = (kThreads / kWave) / WAVES;
+    const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+    const uint32_t row = blockIdx.x * ROWS_PER_BLOCK + wave / WAVES;
+    const int part = wave % WAVES;  // which slice of the row this wave takes
+    __shared__ A shared[kThreads / kWave];
+    A acc = Op::init();
+    if (row < rows) {
+        const T* p = src + static_cast<size_t>(row) * R;
+        constexpr uint32_t STRIDE = kWave * WAVES * VEC;
+        uint32_t r = (part * kWave + lane) * VEC;
+        // two independent accumulators keep two 16-byte loads in flight per lane
+        A acc2 = Op::init();
+        for (; r + STRIDE + VEC <= R; r += 2 * STRIDE) {
+            const Vec<T, VEC> x = load_vec<T, VEC>(p + r);
+            const Vec<T, VEC> y = load_vec<T, VEC>(p + r + STRIDE);
+#pragma unroll
+            for (int i = 0; i < VEC; ++i) acc = Op::step(acc, x.v[i], r + i);
+#pragma unroll
+            for (int i = 0; i < VEC; ++i) acc2 = Op::step(acc2, y.v[i], r + STRIDE + i);
+        }
+        for (; r + VEC <= R; r += STRIDE) {
+            const Vec<T, VEC> x = load_vec<T, VEC>(p + r);
+#pragma unroll
+            for (int i = 0; i < VEC; ++i) acc = Op::step(acc, x.v[i], r + i);
+        }
+        acc = Op::combine(acc, acc2);
+    }
+    acc = wave_reduce<Op>(acc);
+    if constexpr (WAVES == 1) {
+        if (lane == 0 && row < rows) emit<Op>(acc, R, dst, row, src, static_cast<size_t>(row) * R, 1);
+    } else {
+        if (lane == 0) shared[wave] = acc;
+        __syncthreads();
+        if (threadIdx.x == 0 && row < rows) {
+            A total = shared[0];
+            for (int w = 1; w < WAVES; ++w) total = Op::combine(total, shared[w]);
+            emit<Op>(total, R, dst, row, src, static_cast<size_t>(row) * R, 1);
+        }
+    }
+}
+
+// ---- columns: inner > 1 ----------------------------------------------------------
+// Thread (tx, ty): VEC columns starting at (blockIdx.x*TX + tx)*VEC, rows
+// ty + k*TY*gridDim.z offset by blockIdx.z*TY.  LOG_TX picks the block shape.
+template <class Op, int VEC, int TX>
+__global__ __launch_bounds__(kThreads) void reduce_columns_kernel(const typename Op::S* src, typename Op::Out* dst, typename Op::A* partial,
+                                                                   uint32_t R, uint32_t inner, uint32_t slots) {
+    using A = typename Op::A;
+    using T = typename Op::S;
+    constexpr int TY = kThreads / TX;
+    const int tx = threadIdx.x % TX, ty = threadIdx.x / TX;
+    const uint32_t col = (blockIdx.x * TX + tx) * VEC;
+    const uint32_t outer = blockIdx.y;
+    const bool live = col < inner;
+    __shared__ A shared[kThreads][VEC > 4 ? 4 : VEC];  // see the loop over `pass` below
+    A acc[VEC];
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) acc[i] = Op::init();
+    if (live) {
+        const T* p = src + static_cast<size_t>(outer) * R * inner + col;
+        const uint32_t stride = TY * gridDim.z;
+        uint32_t r = blockIdx.z * TY + ty;
+        for (; r + 3 * stride < R; r += 4 * stride) {
+            Vec<T, VEC> x[4];
+#pragma unroll
+            for (int k = 0; k < 4; ++k) x[k] = load_vec<T, VEC>(p + static_cast<size_t>(r + k * stride) * inner);
+#pragma unroll
+            for (int k = 0; k < 4; ++k)
+#pragma unroll
+                for (int i = 0; i < VEC; ++i) acc[i] = Op::step(acc[i], x[k].v[i], r + k * stride);
+        }
+        for (; r < R; r += stride) {
+            const Vec<T, VEC> x = load_vec<T, VEC>(p + static_cast<size_t>(r) * inner);
+#pragma unroll
+            for (int i = 0; i < VEC; ++i) acc[i] = Op::step(acc[i], x.v[i], r);
+        }
+    }
+    // fold the TY slices through LDS, at most four columns of the vector at a time
+    constexpr int CH = VEC > 4 ? 4 : VEC;
+#pragma unroll
+    for (int pass = 0; pass < VEC / CH; ++pass) {
+        __syncthreads();
+#pragma unroll
+        for (int i = 0; i < CH; ++i) shared[threadIdx.x][i] = acc[pass * CH + i];
+        __syncthreads();
+        if (ty == 0 && live) {
+#pragma unroll
+            for (int i = 0; i < CH; ++i) {
+                A total = shared[tx][i];
+                for (int y = 1; y < TY; ++y) total = Op::combine(total, shared[y * TX + tx][i]);
+                const size_t slot = static_cast<size_t>(outer) * inner + col + pass * CH + i;
+                if (gridDim.z == 1) emit<Op>(total, R, dst, slot, src, static_cast<size_t>(outer) * R * inner + col + pass * CH + i, inner);
+                else partial[static_cast<size_t>(blockIdx.z) * slots + slot] = total;
+            }
+        }
+    }
+}
+
+// Second pass of the split-R column reduction: folds `splits` partials per slot.
+template <class Op>
+__global__ __launch_bounds__(kThreads) void reduce_finish_kernel(const typename Op::A* partial, typename Op::Out* dst, const typename Op::S* src,
+                                                                  uint32_t splits, uint32_t slots, uint32_t R, uint32_t inner) {
+    const uint32_t slot = blockIdx.x * kThreads + threadIdx.x;
+    if (slot >= slots) return;
+    typename Op::A total = partial[slot];
+    for (uint32_t s = 1; s < splits; ++s) total = Op::combine(total, partial[static_cast<size_t>(s) * slots + slot]);
+    const uint32_t outer = slot / inner, col = slot % inner;
+    emit<Op>(total, R, dst, slot, src, static_cast<size_t>(outer) * R * inner + col, inner);
+}
+
+// ---- strided sources: one thread per output slot (src/cpu/argred.cpp:44-76) -----
+struct StridedWalk {
+    int rank, axis;
+    uint32_t extent[TANNIC_DIMENSIONS];
+    int64_t stride[TANNIC_DIMENSIONS];
+};
+
+template <class Op>
+__global__ __launch_bounds__(kThreads) void reduce_strided_kernel(const typename Op::S* src, typename Op::Out* dst, StridedWalk w, uint32_t slots) {
+    const uint32_t slot = blockIdx.x * kThreads + threadIdx.x;
+    if (slot >= slots) return;
+    uint32_t rem = slot;
+    int64_t base = 0;
+    for (int d = w.rank - 1; d >= 0; --d) {
+        if (d == w.axis) continue;
+        base += static_cast<int64_t>(rem % w.extent[d]) * w.stride[d];
+        rem /= w.extent[d];
+    }
+    const uint32_t R = w.extent[w.axis];
+    const int64_t step = w.stride[w.axis];
+    typename Op::A acc = Op::init();
+    for (uint32_t r = 0; r < R; ++r) acc = Op::step(acc, src[base + static_cast<int64_t>(r) * step], r);
+    if constexpr (Op::needs_source) dst[slot] = src[base + static_cast<int64_t>(acc.index) * step];
+    else dst[slot] = Op::finish(acc, R);
+}
+
+// ---- host side -------------------------------------------------------------------
+template <class Op>
+int run_reduce(const tannic_tensor_t* src, tannic_tensor_t* dst, hipStream_t stream, uint8_t axis) {
+    using T = typename Op::S;
+    using Out = typename Op::Out;
+    using A = typename Op::A;
+    if (axis >= src->rank) {
+        set_error_text("reduce: axis out of range");
+        return TANNIC_ERROR;
+    }
+    const T* ps = static_cast<const T*>(src->address);
+    Out* pd = static_cast<Out*>(dst->address);
+    const size_t R = src->shape.sizes[axis];
+    if (R >= (1ull << 32)) {
+        set_error_text("reduce: reduced axis of 2^32 elements or more is not supported");
+        return TANNIC_ERROR;
+    }
+    if (src->layout != TANNIC_CONTIGUOUS) {
+        StridedWalk w{};
+        w.rank = src->rank;
+        w.axis = axis;
+        size_t slots = 1;
+        for (int d = 0; d < src->rank; ++d) {
+            w.extent[d] = static_cast<uint32_t>(src->shape.sizes[d]);
+            w.stride[d] = src->strides.sizes[d];
+            if (d != axis) slots *= src->shape.sizes[d];
+        }
+        if (slots == 0) return TANNIC_SUCCESS;
+        if (slots >= (1ull << 31)) { set_error_text("reduce: too many outputs"); return TANNIC_ERROR; }
+        hipLaunchKernelGGL((reduce_strided_kernel<Op>), dim3((slots + kThreads - 1) / kThreads), dim3(kThreads), 0, stream, ps, pd, w,
+                           static_cast<uint32_t>(slots));
+        return launch_status("reduce_strided_kernel");
+    }
+    size_t outer = 1, inner = 1;
+    for (int d = 0; d < src->rank; ++d) {
+        if (d < axis) outer *= src->shape.sizes[d];
+        else if (d > axis) inner *= src->shape.sizes[d];
+    }
+    const size_t slots = outer * inner;
+    if (slots == 0) return TANNIC_SUCCESS;
+    if (slots >= (1ull << 31) || outer >= (1ull << 31)) { set_error_text("reduce: too many outputs"); return TANNIC_ERROR; }
+    constexpr int VEC = sizeof(T) >= 16 ? 1 : static_cast<int>(16 / sizeof(T));
+    const bool aligned = reinterpret_cast<uintptr_t>(ps) % 16 == 0;
+
+    if (inner == 1) {
+        const uint32_t rows = static_cast<uint32_t>(outer);
+        const bool vec = VEC > 1 && aligned && R % VEC == 0;
+        // few long rows: a whole block per row
+        const bool wide = rows < 2048 && R >= 8192;
+        const uint32_t grid = wide ? rows : (rows + 3) / 4;
+        auto launch = [&](auto kernel) {
+            hipLaunchKernelGGL(kernel, dim3(grid), dim3(kThreads), 0, stream, ps, pd, rows, static_cast<uint32_t>(R));
+        };
+        if (vec && wide) launch(reduce_rows_kernel<Op, VEC, 4>);
+        else if (vec) launch(reduce_rows_kernel<Op, VEC, 1>);
+        else if (wide) launch(reduce_rows_kernel<Op, 1, 4>);
+        else launch(reduce_rows_kernel<Op, 1, 1>);
+        return launch_status("reduce_rows_kernel");
+    }
+
+    if (outer > 65535) {
+        // grid.y carries `outer`; fold the excess into a strided walk instead
+        StridedWalk w{};
+        w.rank = 3; w.axis = 1;
+        w.extent[0] = static_cast<uint32_t>(outer); w.extent[1] = static_cast<uint32_t>(R); w.extent[2] = static_cast<uint32_t>(inner);
+        w.stride[0] = static_cast<int64_t>(R * inner); w.stride[1] = static_cast<int64_t>(inner); w.stride[2] = 1;
+        hipLaunchKernelGGL((reduce_strided_kernel<Op>), dim3((slots + kThreads - 1) / kThreads), dim3(kThreads), 0, stream, ps, pd, w,
+                           static_cast<uint32_t>(slots));
+        return launch_status("reduce_strided_kernel");
+    }
+
+    const bool vec = VEC > 1 && aligned && inner % VEC == 0;
+    const uint32_t column_groups = static_cast<uint32_t>(vec ? inner / VEC : inner);
+    // block shape: TX lanes across columns, the rest of the 256 threads across R
+    const int TX = column_groups >= 64 ? 64 : column_groups >= 16 ? 16 : 4;
+    const int TY = kThreads / TX;
+    const uint32_t gx = (column_groups + TX - 1) / TX;
+    // split R over blocks until the chip has ~8 blocks per CU or slices get short
+    uint32_t splits = 1;
+    const size_t base_blocks = static_cast<size_t>(gx) * outer;
+    while (base_blocks * splits < 2048 && R / (static_cast<size_t>(TY) * splits * 2) >= 16 && splits < 64) splits *= 2;
+    A* partial = nullptr;
+    if (splits > 1) {
+        if (scratch_acquire(reinterpret_cast<void**>(&partial), sizeof(A) * splits * slots, stream) != TANNIC_SUCCESS) return TANNIC_ERROR;
+    }
+    const dim3 grid(gx, static_cast<uint32_t>(outer), splits);
+    auto launch = [&](auto kernel) {
+        hipLaunchKernelGGL(kernel, grid, dim3(kThreads), 0, stream, ps, pd, partial, static_cast<uint32_t>(R), static_cast<uint32_t>(inner),
+                           static_cast<uint32_t>(slots));
+    };
+    if (vec) {
+        if (TX == 64) launch(reduce_columns_kernel<Op, VEC, 64>);
+        else if (TX == 16) launch(reduce_columns_kernel<Op, VEC, 16>);
+        else launch(reduce_columns_kernel<Op, VEC, 4>);
+    } else {
+        if (TX == 64) launch(reduce_columns_kernel<Op, 1, 64>);
+        else if (TX == 16) launch(reduce_columns_kernel<Op, 1, 16>);
+        else launch(reduce_columns_kernel<Op, 1, 4>);
+    }
+    int status = launch_status("reduce_columns_kernel");
+    if (splits > 1) {
+        if (status == TANNIC_SUCCESS) {
+            hipLaunchKernelGGL((reduce_finish_kernel<Op>), dim3((slots + kThreads - 1) / kThreads), dim3(kThreads), 0, stream, partial, pd, ps,
+                               splits, static_cast<uint32_t>(slots), static_cast<uint32_t>(R), static_cast<uint32_t>(inner));
+            status = launch_status("reduce_finish_kernel");
+        }
+        scratch_release(partial, stream);
+    }
+    return status;
+}
+
+enum ReduceKind { R_SUM, R_MEAN, R_ARGMAX, R_ARGMIN, R_MAX, R_MIN };
+
+template <int K>
+int reduce_entry(const tannic_tensor_t* src, tannic_tensor_t* dst, tannic_stream_t stream, uint8_t axis) {
+    if (!src || !dst) return TANNIC_ERROR;
+    int status = TANNIC_UNSUPPORTED_DTYPE;
+    with_type(src->dtype, [&](auto t) {
+        using T = typename decltype(t)::type;
+        constexpr bool cplx = std::is_same_v<T, c64> || std::is_same_v<T, c128>;
+        if constexpr (!cplx) {
+            hipStream_t s = as_stream(stream);
+            // coverage: src/cpu/argred.cpp:289-347 (mean: floating types only)
+            if constexpr (K == R_SUM) status = run_reduce<SumOp<T, false>>(src, dst, s, axis);
+            else if constexpr (K == R_MEAN) { if constexpr (!std::is_integral_v<T>) status = run_reduce<SumOp<T, true>>(src, dst, s, axis); }
+            else if constexpr (K == R_ARGMAX) status = run_reduce<ArgOp<T, true, false>>(src, dst, s, axis);
+            else if constexpr (K == R_ARGMIN) status = run_reduce<ArgOp<T, false, false>>(src, dst, s, axis);
+            else if constexpr (K == R_MAX) status = run_reduce<ArgOp<T, true, true>>(src, dst, s, axis);
+            else status = run_reduce<ArgOp<T, false, true>>(src, dst, s, axis);
+        }
+    });
+    return status;
+}
+
+}  // namespace th
+
+using namespace th;
+
+extern "C" {
+int tannic_hip_argsum(const tannic_tensor_t* s, tannic_tensor_t* d, tannic_stream_t st, uint8_t ax) { return reduce_entry<R_SUM>(s, d, st, ax); }
+int tannic_hip_argmean(const tannic_tensor_t* s, tannic_tensor_t* d, tannic_stream_t st, uint8_t ax) { return reduce_entry<R_MEAN>(s, d, st, ax); }
+int tannic_hip_argmax(const tannic_tensor_t* s, tannic_tensor_t* d, tannic_stream_t st, uint8_t ax) { return reduce_entry<R_ARGMAX>(s, d, st, ax); }
+int tannic_hip_argmin(const tannic_tensor_t* s, tannic_tensor_t* d, tannic_stream_t st, uint8_t ax) { return reduce_entry<R_ARGMIN>(s, d, st, ax); }
+int tannic_hip_max(const tannic_tensor_t* s, tannic_tensor_t* d, tannic_stream_t st, uint8_t ax) { return reduce_entry<R_MAX>(s, d, st, ax); }
+int tannic_hip_min(const tannic_tensor_t* s, tannic_tensor_t* d, tannic_stream_t st, uint8_t ax) { return reduce_entry<R_MIN>(s, d, st, ax); }
+}

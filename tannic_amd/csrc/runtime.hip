@@ -1,0 +1,235 @@
+// Devices, memory, streams, host<->device copies.
+// Replaces the reference's src/cuda/mem.cu, src/cuda/streams.cu and
+// src/cuda/exc.cuh; cited per function in include/tannic_hip.h.
+#include <cstdlib>
+#include <mutex>
+#include <string>
+#include <vector>
+
+#include "common.hpp"
+
+namespace th {
+
+static thread_local std::string g_last_error;
+
+void set_error(const char* what, const char* file, int line, hipError_t code) {
+    char buf[512];
+    std::snprintf(buf, sizeof buf, "HIP error at %s:%d code=%d(%s) in '%s'", file, line, static_cast<int>(code),
+                  hipGetErrorString(code), what);
+    g_last_error = buf;
+}
+
+void set_error_text(const char* text) { g_last_error = text; }
+
+// Per-device LIFO pool of streams (src/cuda/streams.cu:23-38).  With one host
+// thread the pool hands the same stream back every time, so consecutive
+// operator calls are ordered; a mutex makes concurrent callers safe, which the
+// reference's pool is not.
+class Streams {
+   public:
+    static Streams& instance() {
+        static Streams s;
+        return s;
+    }
+    hipStream_t pop(int device) {
+        std::lock_guard<std::mutex> lock(mutex_);
+        if (device < 0) return nullptr;
+        if (static_cast<size_t>(device) >= pools_.size()) pools_.resize(device + 1);
+        auto& pool = pools_[device];
+        if (!pool.empty()) {
+            hipStream_t s = pool.back();
+            pool.pop_back();
+            return s;
+        }
+        hipStream_t s = nullptr;
+        // default flags: ordered against the legacy stream like the reference's
+        // cudaStreamCreate; default priority
+        if (hipStreamCreate(&s) != hipSuccess) return nullptr;
+        return s;
+    }
+    void put(int device, hipStream_t s) {
+        std::lock_guard<std::mutex> lock(mutex_);
+        if (device < 0) return;
+        if (static_cast<size_t>(device) >= pools_.size()) pools_.resize(device + 1);
+        pools_[device].push_back(s);
+    }
+
+   private:
+    std::mutex mutex_;
+    std::vector<std::vector<hipStream_t>> pools_;
+};
+
+// Keep freed blocks in the device's pool instead of returning them to the
+// driver: the front end allocates one temporary per operator node.
+static void retain_pool_memory(int device) {
+    static std::mutex m;
+    static std::vector<bool> done;
+    std::lock_guard<std::mutex> lock(m);
+    if (static_cast<size_t>(device) >= done.size()) done.resize(device + 1, false);
+    if (done[device]) return;
+    done[device] = true;
+    hipMemPool_t pool;
+    if (hipDeviceGetDefaultMemPool(&pool, device) == hipSuccess) {
+        uint64_t threshold = UINT64_MAX;
+        (void)hipMemPoolSetAttribute(pool, hipMemPoolAttrReleaseThreshold, &threshold);
+    }
+    (void)hipGetLastError();
+}
+
+int scratch_acquire(void** ptr, size_t nbytes, hipStream_t stream) {
+    TH_TRY(hipMallocAsync(ptr, nbytes, stream));
+    return TANNIC_SUCCESS;
+}
+
+int scratch_release(void* ptr, hipStream_t stream) {
+    TH_TRY(hipFreeAsync(ptr, stream));
+    return TANNIC_SUCCESS;
+}
+
+}  // namespace th
+
+using namespace th;
+
+extern "C" {
+
+const char* tannic_hip_last_error(void) { return g_last_error.c_str(); }
+
+const char* tannic_hip_arch(void) { return "gfx950"; }
+
+int tannic_hip_get_device_count(void) {
+    int count = 0;
+    hipError_t err = hipGetDeviceCount(&count);
+    if (err != hipSuccess) {
+        set_error("hipGetDeviceCount", __FILE__, __LINE__, err);
+        return -1;
+    }
+    return count;
+}
+
+int tannic_hip_set_device(int id) {
+    TH_TRY(hipSetDevice(id));
+    return TANNIC_SUCCESS;
+}
+
+void* tannic_hip_allocate(const tannic_device_t* device, size_t nbytes) {
+    if (!device || tannic_hip_set_device(device->id) != TANNIC_SUCCESS) return nullptr;
+    retain_pool_memory(device->id);
+    Streams& streams = Streams::instance();
+    hipStream_t stream = streams.pop(device->id);
+    void* ptr = nullptr;
+    hipError_t err = hipMallocAsync(&ptr, nbytes ? nbytes : 1, stream);
+    streams.put(device->id, stream);
+    if (err != hipSuccess) {
+        set_error("hipMallocAsync", __FILE__, __LINE__, err);
+        return nullptr;
+    }
+    return ptr;
+}
+
+void* tannic_hip_deallocate(const tannic_device_t* device, void* address) {
+    if (!device || !address) return nullptr;
+    if (tannic_hip_set_device(device->id) != TANNIC_SUCCESS) return nullptr;
+    Streams& streams = Streams::instance();
+    hipStream_t stream = streams.pop(device->id);
+    hipError_t err = hipFreeAsync(address, stream);
+    streams.put(device->id, stream);
+    if (err != hipSuccess) set_error("hipFreeAsync", __FILE__, __LINE__, err);
+    return nullptr;
+}
+
+int tannic_hip_copy_from_host(const tannic_device_t* device, const void* host, void* dev, size_t nbytes) {
+    if (!device) return TANNIC_NULL_ALLOCATOR;
+    TH_TRY(hipSetDevice(device->id));
+    Streams& streams = Streams::instance();
+    hipStream_t stream = streams.pop(device->id);
+    hipError_t err = hipMemcpyAsync(dev, host, nbytes, hipMemcpyHostToDevice, stream);
+    // callers pass temporaries (one element of an initializer list): the source
+    // must be consumed before returning
+    if (err == hipSuccess) err = hipStreamSynchronize(stream);
+    streams.put(device->id, stream);
+    TH_TRY(err);
+    return TANNIC_SUCCESS;
+}
+
+int tannic_hip_copy_device_to_host(const tannic_device_t* device, const void* dev, void* host, size_t nbytes) {
+    if (!device) return TANNIC_NULL_ALLOCATOR;
+    TH_TRY(hipSetDevice(device->id));
+    Streams& streams = Streams::instance();
+    hipStream_t stream = streams.pop(device->id);
+    hipError_t err = hipMemcpyAsync(host, dev, nbytes, hipMemcpyDeviceToHost, stream);
+    if (err == hipSuccess) err = hipStreamSynchronize(stream);
+    streams.put(device->id, stream);
+    TH_TRY(err);
+    return TANNIC_SUCCESS;
+}
+
+int tannic_hip_compare_from_host(const tannic_device_t* device, const void* host, const void* dev, size_t nbytes) {
+    if (!device) return -1;
+    void* buffer = std::malloc(nbytes ? nbytes : 1);
+    if (!buffer) return -1;
+    int rc = tannic_hip_copy_device_to_host(device, dev, buffer, nbytes);
+    int equal = rc == TANNIC_SUCCESS ? (std::memcmp(host, buffer, nbytes) == 0 ? 1 : 0) : -1;
+    std::free(buffer);
+    return equal;
+}
+
+int tannic_hip_copy(const tannic_tensor_t* src, tannic_tensor_t* dst, size_t nbytes, tannic_stream_t s) {
+    hipStream_t stream = as_stream(s);
+    const bool src_dev = src->environment.kind == TANNIC_DEVICE;
+    const bool dst_dev = dst->environment.kind == TANNIC_DEVICE;
+    if (!src_dev && dst_dev) {
+        TH_TRY(hipMemcpyAsync(dst->address, src->address, nbytes, hipMemcpyHostToDevice, stream));
+        // pageable sources behave like the reference's blocking cudaMemcpy
+        if (src->environment.resource.host.traits != TANNIC_PINNED) TH_TRY(hipStreamSynchronize(stream));
+    } else if (src_dev && !dst_dev) {
+        TH_TRY(hipMemcpyAsync(dst->address, src->address, nbytes, hipMemcpyDeviceToHost, stream));
+        if (dst->environment.resource.host.traits != TANNIC_PINNED) TH_TRY(hipStreamSynchronize(stream));
+    } else if (src_dev && dst_dev) {
+        TH_TRY(hipMemcpyAsync(dst->address, src->address, nbytes, hipMemcpyDeviceToDevice, stream));
+    }
+    return TANNIC_SUCCESS;
+}
+
+tannic_stream_t tannic_hip_pop_stream(const tannic_device_t* device) {
+    tannic_stream_t s;
+    s.address = reinterpret_cast<uintptr_t>(Streams::instance().pop(device ? device->id : 0));
+    return s;
+}
+
+void tannic_hip_put_stream(const tannic_device_t* device, tannic_stream_t stream) {
+    Streams::instance().put(device ? device->id : 0, as_stream(stream));
+}
+
+int tannic_hip_stream_synchronize(tannic_stream_t stream) {
+    TH_TRY(hipStreamSynchronize(as_stream(stream)));
+    return TANNIC_SUCCESS;
+}
+
+int tannic_hip_device_synchronize(void) {
+    TH_TRY(hipDeviceSynchronize());
+    return TANNIC_SUCCESS;
+}
+
+void* tannic_hip_event_create(void) {
+    hipEvent_t e = nullptr;
+    if (hipEventCreate(&e) != hipSuccess) return nullptr;
+    return e;
+}
+
+void tannic_hip_event_destroy(void* event) {
+    if (event) (void)hipEventDestroy(static_cast<hipEvent_t>(event));
+}
+
+int tannic_hip_event_record(void* event, tannic_stream_t stream) {
+    TH_TRY(hipEventRecord(static_cast<hipEvent_t>(event), as_stream(stream)));
+    return TANNIC_SUCCESS;
+}
+
+float tannic_hip_event_elapsed_ms(void* start, void* stop) {
+    float ms = -1.0f;
+    if (hipEventSynchronize(static_cast<hipEvent_t>(stop)) != hipSuccess) return -1.0f;
+    if (hipEventElapsedTime(&ms, static_cast<hipEvent_t>(start), static_cast<hipEvent_t>(stop)) != hipSuccess) return -1.0f;
+    return ms;
+}
+
+}  // extern "C"
