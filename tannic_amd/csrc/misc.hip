@@ -182,7 +182,7 @@ __device__ inline bool compare(T x, T y) {
 }
 
 template <class T, int K, bool FLAT>
-__global__ __launch_bounds__(kBlock) void compare_kernel(const T* a, const T* b, uint8_t* out, uint32_t ne, Plan p, bool accumulate) {
+__global__ __launch_bounds__(kBlock) void compare_kernel(const T* a, const T* b, uint8_t* out, uint32_t ne, Plan p) {
     const uint32_t byte = blockIdx.x * kBlock + threadIdx.x;
     const uint32_t first = byte * 8;
     if (first >= ne) return;
@@ -203,7 +203,6 @@ __global__ __launch_bounds__(kBlock) void compare_kernel(const T* a, const T* b,
             bits |= static_cast<uint32_t>(compare<K>(a[o.o0], b[o.o1])) << i;
         }
     }
-    if (accumulate) bits |= out[byte];
     out[byte] = static_cast<uint8_t>(bits);
 }
 
@@ -235,12 +234,13 @@ int run_compare(const tannic_tensor_t* a, const tannic_tensor_t* b, tannic_tenso
                       reinterpret_cast<uintptr_t>(pa) % 16 == 0 && reinterpret_cast<uintptr_t>(pb) % 16 == 0;
     const uint32_t bytes = (ne + 7) / 8;
     const uint32_t grid = (bytes + kBlock - 1) / kBlock;
-    // a rank-0 destination is OR-ed into, not overwritten (src/cpu/cmps.cpp:87-93)
-    const bool accumulate = rank == 0;
+    // The CPU path ORs a true result into a rank-0 destination and leaves a false
+    // one untouched (src/cpu/cmps.cpp:87-93), which reads memory nobody wrote.
+    // Here the byte is always written: 1 or 0.
     if (flat) hipLaunchKernelGGL((compare_kernel<T, K, true>), dim3(grid), dim3(kBlock), 0, stream, pa, pb,
-                                 static_cast<uint8_t*>(dst->address), ne, plan, accumulate);
+                                 static_cast<uint8_t*>(dst->address), ne, plan);
     else hipLaunchKernelGGL((compare_kernel<T, K, false>), dim3(grid), dim3(kBlock), 0, stream, pa, pb,
-                            static_cast<uint8_t*>(dst->address), ne, plan, accumulate);
+                            static_cast<uint8_t*>(dst->address), ne, plan);
     return launch_status("compare_kernel");
 }
 

@@ -150,8 +150,9 @@ def ulp_distance_f16(a, b):
 
 
 def assert_bit_exact(got, want, what=""):
-    got, want = np.asarray(got), np.asarray(want)
+    got, want = np.ascontiguousarray(got), np.ascontiguousarray(want)
     assert got.shape == want.shape, (what, got.shape, want.shape)
+    assert got.dtype == want.dtype, (what, got.dtype, want.dtype)
     if got.dtype.kind in "fc":
         same = (got.view(np.uint8) == want.view(np.uint8)).all() if got.size else True
         if not same:

@@ -1,0 +1,117 @@
+"""conv2d on the device against the CPU checker.
+
+Bars: bit-exact for integers; fp32/fp64 within 1e-5 relative plus K*eps*max|x||w|
+for summation order; fp16/bf16 (fp32 accumulation on both sides) rel 2e-3 / abs 1e-3.
+"""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+import golden_cases
+import support
+import tannic_amd as ta
+from tannic_amd import abi, ops
+
+pytestmark = pytest.mark.gpu
+SEED = 17
+CONV_GOLDEN = [c for c in golden_cases.TENSOR_CASES if c["op"] == "conv2d"]
+
+# x shape, w shape, stride, padding: scaled-down relatives of the ResNet-50 layers plus odd cases
+CASES = {
+    "stem_k7_s2_p3": ((2, 3, 40, 40), (16, 3, 7, 7), (2, 2), (3, 3)),
+    "body_k3_s1_p1": ((2, 16, 14, 14), (16, 16, 3, 3), (1, 1), (1, 1)),
+    "body_k3_64ch": ((1, 64, 12, 12), (64, 64, 3, 3), (1, 1), (1, 1)),
+    "down_k1_s2": ((2, 32, 14, 14), (48, 32, 1, 1), (2, 2), (0, 0)),
+    "rect_kernel_rect_stride": ((1, 5, 13, 9), (7, 5, 3, 2), (2, 1), (0, 2)),
+    "one_pixel_out": ((3, 4, 3, 3), (5, 4, 3, 3), (1, 1), (0, 0)),
+    "wide_padding": ((1, 2, 4, 4), (3, 2, 3, 3), (1, 1), (2, 2)),
+}
+
+
+@pytest.mark.parametrize("case", CONV_GOLDEN, ids=lambda c: c["name"])
+def test_reference_vectors_on_device(device, case):
+    got = golden_cases.run(case, device)
+    support.assert_close(got, golden_cases.expected_of(case), 1e-5, 1e-8, case["name"])
+
+
+def operands(dtype, name, device, bias):
+    xs, ws, stride, pad = CASES[name]
+    fan_in = ws[1] * ws[2] * ws[3]
+    hx, dx = support.both(support.values_for(dtype, SEED, 1, xs, -2, 2), dtype, device)
+    lim = 100 if dtype.is_integral else 2 * (2.0 / fan_in) ** 0.5
+    hw, dw = support.both(support.values_for(dtype, SEED, 2, ws, -lim, lim), dtype, device)
+    hb, db = support.both(support.values_for(dtype, SEED, 3, (ws[0],), -2, 2), dtype, device) if bias else (None, None)
+    return (hx, hw, hb), (dx, dw, db), stride, pad, fan_in
+
+
+@pytest.mark.parametrize("bias", [False, True])
+@pytest.mark.parametrize("name", list(CASES))
+@pytest.mark.parametrize("dtype", [ta.float32, ta.float64], ids=str)
+def test_float_conv(device, dtype, name, bias):
+    host, dev, stride, pad, k = operands(dtype, name, device, bias)
+    want, got = ops.convolve2d(*host, stride, pad), ops.convolve2d(*dev, stride, pad)
+    assert got.shape == want.shape
+    eps = 2.0 ** -24 if dtype is ta.float32 else 2.0 ** -53
+    support.assert_close(got.numpy(), want.numpy(), 1e-5 if dtype is ta.float32 else 1e-13, k * eps * 4, f"conv {dtype} {name}")
+
+
+@pytest.mark.parametrize("bias", [False, True])
+@pytest.mark.parametrize("name", list(CASES))
+@pytest.mark.parametrize("dtype", [ta.float16, ta.bfloat16], ids=str)
+def test_16bit_conv_fp32_accumulate(device, dtype, name, bias):
+    host, dev, stride, pad, _ = operands(dtype, name, device, bias)
+    want, got = ops.convolve2d(*host, stride, pad), ops.convolve2d(*dev, stride, pad)
+    rtol = 2e-3 if dtype is ta.float16 else 2.0 ** -7
+    support.assert_close(got.numpy(), want.numpy(), rtol, 1e-3, f"conv {dtype} {name}")
+
+
+@pytest.mark.parametrize("name", ["body_k3_s1_p1", "rect_kernel_rect_stride", "wide_padding"])
+@pytest.mark.parametrize("dtype", [ta.int8, ta.int32, ta.int64], ids=str)
+def test_integer_conv_bit_exact(device, dtype, name):
+    host, dev, stride, pad, _ = operands(dtype, name, device, True)
+    support.assert_bit_exact(ops.convolve2d(*dev, stride, pad).storage(), ops.convolve2d(*host, stride, pad).storage(), f"conv {dtype} {name}")
+
+
+def test_strided_signal_view(device):
+    hx, dx = support.both(support.values_for(ta.float32, SEED, 4, (2, 9, 10, 6)), ta.float32, device)
+    hw, dw = support.both(support.values_for(ta.float32, SEED, 5, (8, 6, 3, 3)), ta.float32, device)
+    want = ops.convolve2d(hx.permute(0, 3, 1, 2), hw, None, 1, 1).numpy()
+    got = ops.convolve2d(dx.permute(0, 3, 1, 2), dw, None, 1, 1).numpy()
+    support.assert_close(got, want, 1e-5, 54 * 2.0 ** -24 * 16, "NHWC view")
+
+
+def test_status_codes(device):
+    lib = ta.library()
+    dvc = device.structure()
+    x = ta.Tensor(ta.float32, (1, 3, 5, 5)).initialize(device)
+    w = ta.Tensor(ta.float32, (2, 4, 3, 3)).initialize(device)
+    w_ok = ta.Tensor(ta.float32, (2, 3, 3, 3)).initialize(device)
+    wi = ta.Tensor(ta.int32, (2, 3, 3, 3)).initialize(device)
+    y = ta.Tensor(ta.float32, (1, 2, 3, 3)).initialize(device)
+    y_bad = ta.Tensor(ta.float32, (1, 2, 4, 3)).initialize(device)
+    r3 = ta.Tensor(ta.float32, (3, 5, 5)).initialize(device)
+    stream = lib.pop_stream(C.byref(dvc))
+    try:
+        f = lib.kernels["conv2d"]
+        d = {k: v.descriptor() for k, v in dict(x=x, w=w, w_ok=w_ok, wi=wi, y=y, y_bad=y_bad, r3=r3).items()}
+        pad, stride = abi.SIZE2(0, 0), abi.SIZE2(1, 1)
+        assert f(C.byref(d["x"]), C.byref(d["w"]), C.byref(d["y"]), stream, pad, stride) == abi.ERROR       # channel mismatch
+        assert f(C.byref(d["x"]), C.byref(d["w_ok"]), C.byref(d["y_bad"]), stream, pad, stride) == abi.ERROR  # wrong output shape
+        assert f(C.byref(d["r3"]), C.byref(d["w_ok"]), C.byref(d["y"]), stream, pad, stride) == abi.ERROR     # rank
+        assert f(C.byref(d["x"]), C.byref(d["wi"]), C.byref(d["y"]), stream, pad, stride) == abi.UNSUPPORTED_DTYPE
+        assert f(C.byref(d["x"]), C.byref(d["w_ok"]), C.byref(d["y"]), stream, pad, stride) == abi.SUCCESS
+    finally:
+        lib.put_stream(C.byref(dvc), stream)
+
+
+def test_conv1x1_equals_gemm_on_device(device):
+    x = support.values_for(ta.float16, SEED, 6, (2, 32, 6, 6), -1, 1)
+    w = support.values_for(ta.float16, SEED, 7, (24, 32, 1, 1), -1, 1)
+    _, dx = support.both(x, ta.float16, device)
+    _, dw = support.both(w, ta.float16, device)
+    conv = ops.convolve2d(dx, dw).numpy()
+    _, pixels = support.both(np.ascontiguousarray(x.transpose(0, 2, 3, 1)).reshape(72, 32), ta.float16, device)
+    _, weights = support.both(w.reshape(24, 32), ta.float16, device)
+    gemm = ops.matmul(pixels, weights.transpose()).numpy().reshape(2, 6, 6, 24).transpose(0, 3, 1, 2)
+    support.assert_close(conv, gemm, 2e-3, 1e-3, "1x1 conv vs gemm")

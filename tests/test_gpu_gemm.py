@@ -1,0 +1,118 @@
+"""Matrix multiply on the device against the CPU checker.
+
+Bars: bit-exact for integer types; fp32 within 1e-5 relative plus an absolute
+term K*eps*max|a|*max|b| for summation order; fp16/bf16 (fp32 accumulation on
+both sides) within rel 2e-3 / abs 1e-3.
+"""
+import numpy as np
+import pytest
+
+import golden_cases
+import support
+import tannic_amd as ta
+from tannic_amd import ops
+
+pytestmark = pytest.mark.gpu
+SEED = 13
+GEMM_GOLDEN = [c for c in golden_cases.TENSOR_CASES if c["op"] == "matmul"]
+
+LAYOUTS = {
+    "nn": ((5, 7), (7, 3), [], []),
+    "nt": ((5, 7), (3, 7), [], [("transpose", (-1, -2))]),
+    "tn": ((7, 5), (7, 3), [("transpose", (-1, -2))], []),
+    "tt": ((7, 5), (3, 7), [("transpose", (-1, -2))], [("transpose", (-1, -2))]),
+    "nn_mid": ((130, 70), (70, 190), [], []),
+    "nt_mid": ((130, 72), (190, 72), [], [("transpose", (-1, -2))]),
+    "tn_mid": ((72, 130), (72, 190), [("transpose", (-1, -2))], []),
+    "tt_mid": ((72, 130), (190, 72), [("transpose", (-1, -2))], [("transpose", (-1, -2))]),
+    "nt_tiles": ((256, 128), (384, 128), [], [("transpose", (-1, -2))]),
+    "nn_tiles": ((256, 128), (128, 384), [], []),
+    "batched": ((2, 3, 33, 40), (2, 3, 40, 17), [], []),
+    "batch_broadcast": ((2, 1, 33, 40), (1, 3, 40, 17), [], []),
+    "rank4_rank2_nt": ((2, 3, 20, 64), (48, 64), [], [("transpose", (-1, -2))]),
+    "attention_scores": ((1, 4, 64, 32), (1, 4, 64, 32), [], [("transpose", (-1, -2))]),
+    "attention_values": ((1, 4, 64, 64), (1, 4, 64, 32), [], []),
+    "head_split_view": ((1, 64, 4, 32), (1, 64, 4, 32), [("transpose", (1, 2))], [("transpose", (1, 2)), ("transpose", (-1, -2))]),
+    "single_row": ((1, 256), (96, 256), [], [("transpose", (-1, -2))]),
+    "sixteen_rows": ((16, 256), (96, 256), [], [("transpose", (-1, -2))]),
+    "single_column": ((64, 96), (1, 96), [], [("transpose", (-1, -2))]),
+    "k_one": ((9, 1), (1, 11), [], []),
+}
+
+
+@pytest.mark.parametrize("case", GEMM_GOLDEN, ids=lambda c: c["name"])
+def test_reference_vectors_on_device(device, case):
+    got = golden_cases.run(case, device)
+    support.assert_close(got, golden_cases.expected_of(case), 1e-5, 1e-8, case["name"])
+
+
+def operands(pair, layout, device, low=-1, high=1):
+    sa, sb, va, vb = LAYOUTS[layout]
+    ha, da = support.both(support.values_for(pair[0], SEED, 1, sa, low, high), pair[0], device)
+    hb, db = support.both(support.values_for(pair[1], SEED, 2, sb, low, high), pair[1], device)
+    k = support.apply_view(ha, va).shape[-1]
+    return (support.apply_view(ha, va), support.apply_view(hb, vb)), (support.apply_view(da, va), support.apply_view(db, vb)), k
+
+
+@pytest.mark.parametrize("layout", list(LAYOUTS))
+@pytest.mark.parametrize("dtype", [ta.float32, ta.float64], ids=str)
+def test_float_gemm(device, dtype, layout):
+    host, dev, k = operands((dtype, dtype), layout, device)
+    want, got = ops.matmul(*host), ops.matmul(*dev)
+    assert got.shape == want.shape and got.dtype is want.dtype
+    eps = 2.0 ** -24 if dtype is ta.float32 else 2.0 ** -53
+    support.assert_close(got.numpy(), want.numpy(), 1e-5 if dtype is ta.float32 else 1e-13, k * eps, f"gemm {dtype} {layout}")
+
+
+@pytest.mark.parametrize("layout", list(LAYOUTS))
+@pytest.mark.parametrize("dtype", [ta.float16, ta.bfloat16], ids=str)
+def test_16bit_gemm_fp32_accumulate(device, dtype, layout):
+    host, dev, k = operands((dtype, dtype), layout, device)
+    want, got = ops.matmul(*host), ops.matmul(*dev)
+    assert got.shape == want.shape and got.dtype is dtype
+    rtol = 2e-3 if dtype is ta.float16 else 2.0 ** -7   # bf16 keeps 8 significant bits: one ulp is 2^-7 relative
+    support.assert_close(got.numpy(), want.numpy(), rtol, 1e-3, f"gemm {dtype} {layout}")
+
+
+@pytest.mark.parametrize("layout", ["nn", "nt_mid", "tn_mid", "batched", "batch_broadcast", "rank4_rank2_nt"])
+@pytest.mark.parametrize("pair", [(ta.int8, ta.int8), (ta.int16, ta.int32), (ta.int32, ta.int32), (ta.int64, ta.int8)], ids=lambda p: f"{p[0]}-{p[1]}")
+def test_integer_gemm_bit_exact(device, pair, layout):
+    host, dev, _ = operands(pair, layout, device, -100, 100)
+    want, got = ops.matmul(*host), ops.matmul(*dev)
+    assert got.dtype is want.dtype
+    support.assert_bit_exact(got.storage(), want.storage(), f"gemm {pair} {layout}")
+
+
+@pytest.mark.parametrize("pair", [(ta.int32, ta.float32), (ta.float64, ta.float32), (ta.float16, ta.float32), (ta.float32, ta.bfloat16)],
+                         ids=lambda p: f"{p[0]}-{p[1]}")
+def test_mixed_gemm(device, pair):
+    host, dev, k = operands(pair, "nt_mid", device, -3, 3)
+    want, got = ops.matmul(*host), ops.matmul(*dev)
+    assert got.dtype is want.dtype
+    support.assert_close(got.numpy(), want.numpy(), 1e-5, k * 9 * 2.0 ** -24, f"gemm {pair}")
+
+
+def test_integer_valued_fp16_gemm_is_exact(device):
+    """Small integers: every product and partial sum is exact in fp32, so any order of summation agrees."""
+    a = support.integers(SEED, 3, (192, 320), -4, 4)
+    b = support.integers(SEED, 4, (160, 320), -4, 4)
+    for dtype in (ta.float16, ta.bfloat16, ta.float32):
+        _, da = support.both(a, dtype, device)
+        _, db = support.both(b, dtype, device)
+        got = ops.matmul(da, db.transpose()).numpy().astype(np.int64)
+        want = a @ b.T
+        if dtype is ta.bfloat16:
+            want = support.types.bfloat16_bits_to_float32(support.types.float32_to_bfloat16_bits(want.astype(np.float32))).astype(np.int64)
+        else:
+            want = want.astype(np.float16 if dtype is ta.float16 else np.float32).astype(np.int64)
+        support.assert_bit_exact(got, want, f"integer-valued {dtype}")
+
+
+def test_fp32_matmul_512_seed0(device):
+    """C = A.B, 512^3, uniform[-1,1) from seed 0: the reference's CPU-runnable configuration."""
+    a, b = support.uniform(0, 0, (512, 512)), support.uniform(0, 1, (512, 512))
+    (ha, da), (hb, db) = support.both(a, ta.float32, device), support.both(b, ta.float32, device)
+    want, got = ops.matmul(ha, hb).numpy(), ops.matmul(da, db).numpy()
+    support.assert_close(got, want, 1e-5, 512 * 2.0 ** -24, "fp32 512^3")
+    exact = a.astype(np.float64) @ b.astype(np.float64)
+    assert np.abs(got - exact).max() <= np.abs(want - exact).max() * 1.5 + 1e-6  # no worse than the sequential sum

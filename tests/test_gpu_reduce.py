@@ -1,0 +1,141 @@
+"""Axis reductions on the device against the CPU checker.
+
+Bars: bit-exact for integer sums (wrap-around included), for argmax/argmin
+indices (ties, NaN, infinities) and for value max/min; floating sums/means
+within R*eps*sum|x| of the sequential CPU sum (the device adds partial sums as
+a tree); 16-bit sums accumulate in fp32 on both sides and differ by at most
+one rounding of the 16-bit result.
+"""
+import numpy as np
+import pytest
+
+import golden_cases
+import support
+import tannic_amd as ta
+from tannic_amd import ops
+
+pytestmark = pytest.mark.gpu
+SEED = 9
+REDUCE_GOLDEN = [c for c in golden_cases.TENSOR_CASES if c["op"] in ("sum", "mean", "argmax", "argmin", "mean_sq")]
+
+# (shape, axis): which kernel the launcher picks for a contiguous source
+SHAPES = {
+    "rows_short": ((300, 17), 1),
+    "rows_vector": ((512, 1024), 1),
+    "rows_odd": ((77, 1001), 1),
+    "rows_block_wide": ((3, 40000), 1),
+    "one_row": ((9000,), 0),
+    "columns_wide": ((4, 300, 1024), 1),
+    "columns_split": ((2, 4096, 256), 1),
+    "columns_narrow": ((5, 200, 20), 1),
+    "columns_tiny": ((7, 33, 3), 1),
+    "first_axis": ((1000, 96), 0),
+    "middle_of_4d": ((3, 50, 4, 32), 1),
+    "reduced_extent_one": ((6, 1, 40), 1),
+}
+
+
+@pytest.mark.parametrize("case", REDUCE_GOLDEN, ids=lambda c: c["name"])
+def test_reference_vectors_on_device(device, case):
+    got = golden_cases.run(case, device)
+    rtol, atol = golden_cases.tolerance(case)
+    support.assert_close(got, golden_cases.expected_of(case), rtol, atol, case["name"])
+
+
+def sum_tolerance(x, axis, dtype):
+    eps = {ta.float32: 2.0 ** -24, ta.float64: 2.0 ** -53}[dtype]
+    r = x.shape[axis]
+    return r * eps * np.abs(x.astype(np.float64)).sum(axis=axis).max()
+
+
+@pytest.mark.parametrize("name", list(SHAPES))
+@pytest.mark.parametrize("dtype", [ta.float32, ta.float64], ids=str)
+def test_float_sum_and_mean(device, dtype, name):
+    shape, axis = SHAPES[name]
+    x = support.values_for(dtype, SEED, 1, shape)
+    h, d = support.both(x, dtype, device)
+    atol = sum_tolerance(x, axis, dtype)
+    for op in ("sum", "mean"):
+        for keepdim in (False, True):
+            want, got = getattr(ops, op)(h, axis, keepdim), getattr(ops, op)(d, axis, keepdim)
+            assert got.shape == want.shape
+            support.assert_close(got.numpy(), want.numpy(), 1e-6 if dtype is ta.float32 else 1e-14, atol, f"{op} {name} {dtype}")
+
+
+@pytest.mark.parametrize("name", list(SHAPES))
+@pytest.mark.parametrize("dtype", [ta.float16, ta.bfloat16], ids=str)
+def test_16bit_sum_and_mean_accumulate_in_fp32(device, dtype, name):
+    shape, axis = SHAPES[name]
+    x = support.values_for(dtype, SEED, 2, shape, -1, 1)
+    h, d = support.both(x, dtype, device)
+    for op in ("sum", "mean"):
+        want, got = getattr(ops, op)(h, axis).numpy(), getattr(ops, op)(d, axis).numpy()
+        ulp = 2.0 ** -10 if dtype is ta.float16 else 2.0 ** -7
+        support.assert_close(got, want, ulp, ulp * 2.0 ** -3, f"{op} {name} {dtype}")
+
+
+@pytest.mark.parametrize("name", list(SHAPES))
+@pytest.mark.parametrize("dtype", [ta.int8, ta.int16, ta.int32, ta.int64], ids=str)
+def test_integer_sum_is_bit_exact_with_wrap_around(device, dtype, name):
+    shape, axis = SHAPES[name]
+    h, d = support.both(support.values_for(dtype, SEED, 3, shape, -120, 120), dtype, device)
+    support.assert_bit_exact(ops.sum(d, axis).storage(), ops.sum(h, axis).storage(), f"sum {name} {dtype}")
+
+
+@pytest.mark.parametrize("name", list(SHAPES))
+@pytest.mark.parametrize("dtype", [ta.float32, ta.float16, ta.bfloat16, ta.float64, ta.int32, ta.int8, ta.int64], ids=str)
+def test_argmax_argmin_max_min_bit_exact(device, dtype, name):
+    shape, axis = SHAPES[name]
+    # few distinct values: ties everywhere, the lowest index must win
+    x = np.round(support.values_for(dtype, SEED, 4, shape, -3, 3).astype(np.float64))
+    h, d = support.both(x, dtype, device)
+    for op in ("argmax", "argmin", "max", "min"):
+        want, got = getattr(ops, op)(h, axis), getattr(ops, op)(d, axis)
+        assert got.dtype is want.dtype and got.shape == want.shape
+        support.assert_bit_exact(got.storage(), want.storage(), f"{op} {name} {dtype}")
+
+
+def test_argmax_with_nan_and_infinities(device):
+    x = support.uniform(SEED, 5, (64, 700))
+    x[0, :] = np.nan
+    x[1, :] = -np.inf
+    x[2, 5] = np.nan
+    x[3, 10] = np.inf
+    x[3, 600] = np.inf
+    x[4, :] = np.inf
+    h, d = support.both(x, ta.float32, device)
+    for op in ("argmax", "argmin"):
+        for axis in (0, 1):
+            support.assert_bit_exact(getattr(ops, op)(d, axis).storage(), getattr(ops, op)(h, axis).storage(), f"{op} axis={axis}")
+    hi, di = support.both(np.full((5, 300), -128), ta.int8, device)
+    support.assert_bit_exact(ops.argmax(di, 1).storage(), ops.argmax(hi, 1).storage(), "int8 all lowest")
+
+
+@pytest.mark.parametrize("dtype", [ta.float32, ta.int32, ta.float16], ids=str)
+def test_strided_sources(device, dtype):
+    h, d = support.both(np.round(support.values_for(dtype, SEED, 6, (12, 30, 20)).astype(np.float64)), dtype, device)
+    for spec in ([("transpose", (0, 2))], [("index", (slice(1, 12, 2), slice(None), slice(0, 20, 3)))], [("permute", (1, 2, 0))]):
+        hv, dv = support.apply_view(h, spec), support.apply_view(d, spec)
+        for axis in range(3):
+            for op in ("sum", "argmax", "min"):
+                want, got = getattr(ops, op)(hv, axis), getattr(ops, op)(dv, axis)
+                support.assert_bit_exact(got.storage(), want.storage(), f"{op} {dtype} {spec} axis={axis}")  # integer-valued: sums exact
+
+
+def test_rms_norm_statistics(device):
+    """mean(X*X, -1, keepdim) then rsqrt: the reduction pattern of an RMSNorm row (R = 4096)."""
+    h, d = support.both(support.values_for(ta.bfloat16, SEED, 7, (1, 64, 4096)), ta.bfloat16, device)
+
+    def stat(x):
+        return ops.rsqrt(ops.mean(ops.mul(x, x), -1, True), 1e-5)
+    support.assert_close(stat(d).numpy(), stat(h).numpy(), 2.0 ** -7, 0, "rms statistics")
+
+
+def test_softmax_statistics(device):
+    """max and sum over the last axis (R = 512), as a softmax row needs them."""
+    h, d = support.both(support.values_for(ta.float32, SEED, 8, (4, 64, 512)), ta.float32, device)
+
+    def softmax_den(x):
+        m = ops.max(x, -1, True)
+        return ops.sum(ops.exp(ops.sub(x, m)), -1, True)
+    support.assert_close(softmax_den(d).numpy(), softmax_den(h).numpy(), 1e-5, 0, "softmax denominator")

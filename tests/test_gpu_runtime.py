@@ -1,0 +1,104 @@
+"""Memory, streams and copies of the device library, called through the C ABI."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+import support
+import tannic_amd as ta
+from tannic_amd import abi, ops
+
+pytestmark = pytest.mark.gpu
+
+
+def test_device_count_and_invalid_ids(device):
+    lib = ta.library()
+    assert lib.get_device_count() >= 1
+    assert lib.arch() == b"gfx950"
+    with pytest.raises(IndexError):  # std::out_of_range in the reference (src/resources.cpp:46-48)
+        ta.Device(lib.get_device_count())
+    with pytest.raises(IndexError):
+        ta.Device(-1)
+
+
+def test_stream_pool_is_lifo(device):
+    lib = ta.library()
+    dvc = device.structure()
+    s1 = lib.pop_stream(C.byref(dvc))
+    s2 = lib.pop_stream(C.byref(dvc))
+    assert s1.address != 0 and s2.address != 0 and s1.address != s2.address
+    lib.put_stream(C.byref(dvc), s2)
+    lib.put_stream(C.byref(dvc), s1)
+    again = lib.pop_stream(C.byref(dvc))
+    assert again.address == s1.address  # last put, first popped (src/cuda/streams.cu:23-38)
+    lib.put_stream(C.byref(dvc), again)
+
+
+def test_allocate_copy_compare(device):
+    lib = ta.library()
+    dvc = device.structure()
+    data = np.arange(1000, dtype=np.float32)
+    ptr = lib.allocate(C.byref(dvc), data.nbytes)
+    assert ptr
+    assert lib.copy_from_host(C.byref(dvc), data.ctypes.data, ptr, data.nbytes) == abi.SUCCESS
+    assert lib.compare_from_host(C.byref(dvc), data.ctypes.data, ptr, data.nbytes) == 1
+    other = data.copy()
+    other[500] += 1
+    assert lib.compare_from_host(C.byref(dvc), other.ctypes.data, ptr, data.nbytes) == 0
+    back = np.empty_like(data)
+    assert lib.copy_device_to_host(C.byref(dvc), ptr, back.ctypes.data, data.nbytes) == abi.SUCCESS
+    assert (back == data).all()
+    assert lib.deallocate(C.byref(dvc), ptr) is None
+
+
+def test_element_assignment_and_read_back(device):
+    """`X[i, j] = v` and `X[i, j] == v` go through copyFromHost / compareFromHost one element
+    at a time (src/tensor.cpp:34-75)."""
+    lib = ta.library()
+    dvc = device.structure()
+    x = ta.Tensor(ta.float32, (2, 3)).initialize(device)
+    for i in range(6):
+        v = C.c_float(i * 1.5)
+        assert lib.copy_from_host(C.byref(dvc), C.byref(v), x.address + 4 * i, 4) == abi.SUCCESS
+    for i in range(6):
+        v = C.c_float(i * 1.5)
+        assert lib.compare_from_host(C.byref(dvc), C.byref(v), x.address + 4 * i, 4) == 1
+    assert (x.numpy() == np.arange(6).reshape(2, 3) * 1.5).all()
+
+
+def test_tensor_copies_between_environments(device, oracle):
+    h = support.host_tensor(support.uniform(1, 1, (33, 65)), ta.float32)
+    d = h.to(device)
+    d2 = d.to(device)          # device -> device
+    back = d2.to(ta.Host())    # device -> host
+    support.assert_bit_exact(back.storage(), h.storage(), "H2D, D2D, D2H")
+    v = d.transpose()          # a view keeps its strides across the copy
+    support.assert_bit_exact(v.to(ta.Host()).storage(), h.storage().T, "view")
+
+
+def test_mixed_environments_are_rejected(device, oracle):
+    h = support.host_tensor(np.ones((2, 2)), ta.float32)
+    d = h.to(device)
+    with pytest.raises(ta.TannicError):
+        ops.add(h, d)
+
+
+def test_unsupported_dtypes_report_status(device):
+    lib = ta.library()
+    dvc = device.structure()
+    b = ta.Tensor(ta.boolean, (8,)).initialize(device)
+    c = ta.Tensor(ta.complex64, (8,)).initialize(device)
+    out = ta.Tensor(ta.float32, (8,)).initialize(device)
+    stream = lib.pop_stream(C.byref(dvc))
+    try:
+        db, dc, do = b.descriptor(), c.descriptor(), out.descriptor()
+        assert lib.kernels["log"](C.byref(db), C.byref(do), stream) == abi.UNSUPPORTED_DTYPE
+        assert lib.kernels["log"](C.byref(dc), C.byref(do), stream) == abi.UNSUPPORTED_DTYPE
+        assert lib.kernels["add"](C.byref(dc), C.byref(do), C.byref(do), stream) == abi.UNSUPPORTED_DTYPE
+        assert lib.kernels["gemm"](C.byref(dc), C.byref(dc), C.byref(do), stream) == abi.UNSUPPORTED_DTYPE
+        assert lib.kernels["argmean"](C.byref(db), C.byref(do), stream, 0) == abi.UNSUPPORTED_DTYPE
+        assert lib.kernels["allclose"](C.byref(db), C.byref(db), stream, 1e-5, 1e-8) == -1
+    finally:
+        lib.put_stream(C.byref(dvc), stream)
+    with pytest.raises(ta.TannicError):
+        ops.exp(ta.Tensor(ta.int32, (4,)).initialize(device))
