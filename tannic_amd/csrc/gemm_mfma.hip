@@ -73,29 +73,46 @@ struct Operand {
     uint32_t rows;  // M for A, N for B
 };
 
+// Calls f(std::integral_constant<int, 0>{}) ... f(std::integral_constant<int, N-1>{}).
+template <int N, class F, int I = 0>
+__device__ inline void static_for(F&& f) {
+    if constexpr (I < N) {
+        f(std::integral_constant<int, I>{});
+        static_for<N, F, I + 1>(static_cast<F&&>(f));
+    }
+}
+
 // Swizzled element offset of (row, chunk) inside a [ROWS][64] tile.
-__device__ inline uint32_t tile_offset(uint32_t row, uint32_t chunk) { return row * kBK + ((chunk ^ (row & 7u)) * kChunk); }
+// LDS serves 16 lanes of a 16-byte read per clock out of a 256-byte bank window,
+// i.e. two 128-byte rows: consecutive row PAIRS get different chunk rotations so
+// that 16 consecutive rows of one logical chunk land in 16 different slots.
+__device__ inline uint32_t tile_offset(uint32_t row, uint32_t chunk) { return row * kBK + ((chunk ^ ((row >> 1) & 7u)) * kChunk); }
 
 // ---- global -> registers -> LDS, operand contiguous along K -------------------
+// Rows past the operand's end read a clamped (valid) address: they only feed
+// rows/columns of C that are never stored.  K past the end must contribute
+// zero; that is decided when the registers are written to LDS, so that nothing
+// touches the loaded values (and waits for them) early.
+// Both loaders expose their work as single memory operations (fetch_one /
+// commit_one) so that the main loop can spread them between MFMAs.
 template <class T, int ROWS>
 struct KMajorLoader {
-    static constexpr int PASSES = ROWS / 32;
-    uint4v regs[PASSES];
-    __device__ inline void fetch(const Operand& op, uint32_t row0, uint32_t k0, uint32_t K) {
-        const uint32_t chunk = threadIdx.x % 8, r = threadIdx.x / 8;
-        const uint32_t k = k0 + chunk * kChunk;
-        const T* base = static_cast<const T*>(op.base);
-#pragma unroll
-        for (int i = 0; i < PASSES; ++i) {
-            const uint32_t row = row0 + r + 32 * i;
-            if (row < op.rows && k < K) regs[i] = *reinterpret_cast<const uint4v*>(base + static_cast<int64_t>(row) * op.row_stride + k);
-            else regs[i] = uint4v{0, 0, 0, 0};
-        }
+    static constexpr int LOADS = ROWS / 32, STORES = ROWS / 32;
+    uint4v regs[LOADS];
+    const T* base;      // operand base + this thread's k offset for the tile being fetched
+    bool k_live;
+    __device__ inline void begin_fetch(const Operand& op, uint32_t k0, uint32_t K) {
+        const uint32_t k = k0 + (threadIdx.x % 8) * kChunk;
+        k_live = k < K;
+        base = static_cast<const T*>(op.base) + (k_live ? k : 0);
     }
-    __device__ inline void commit(T* tile) const {
-        const uint32_t chunk = threadIdx.x % 8, r = threadIdx.x / 8;
-#pragma unroll
-        for (int i = 0; i < PASSES; ++i) *reinterpret_cast<uint4v*>(tile + tile_offset(r + 32 * i, chunk)) = regs[i];
+    __device__ inline void fetch_one(int i, const Operand& op, uint32_t row0) {
+        const uint32_t row = row0 + threadIdx.x / 8 + 32 * i;
+        const uint32_t srow = row < op.rows ? row : op.rows - 1;
+        regs[i] = *reinterpret_cast<const uint4v*>(base + static_cast<int64_t>(srow) * op.row_stride);
+    }
+    __device__ inline void commit_one(int i, T* tile) const {
+        *reinterpret_cast<uint4v*>(tile + tile_offset(threadIdx.x / 8 + 32 * i, threadIdx.x % 8)) = k_live ? regs[i] : uint4v{0, 0, 0, 0};
     }
 };
 
@@ -104,43 +121,39 @@ template <class T, int ROWS>
 struct RowMajorLoader {
     // ROWS/8 row-blocks x 8 k-blocks micro-blocks, 256 threads
     static constexpr int PASSES = (ROWS + 255) / 256;
+    static constexpr int LOADS = 8 * PASSES, STORES = 8 * PASSES;
     uint4v regs[PASSES][8];
-    __device__ inline void fetch(const Operand& op, uint32_t row0, uint32_t k0, uint32_t K) {
-        const T* base = static_cast<const T*>(op.base);
-#pragma unroll
-        for (int i = 0; i < PASSES; ++i) {
-            const uint32_t mb = threadIdx.x + kThreads * i;
-            const uint32_t kb = mb % 8, rb = mb / 8;
-            const uint32_t row = row0 + rb * 8;
-            const bool live = rb < ROWS / 8 && row < op.rows;
-#pragma unroll
-            for (int kk = 0; kk < 8; ++kk) {
-                const uint32_t k = k0 + kb * 8 + kk;
-                if (live && k < K) regs[i][kk] = *reinterpret_cast<const uint4v*>(base + static_cast<int64_t>(k) * op.k_stride + row);
-                else regs[i][kk] = uint4v{0, 0, 0, 0};
-            }
-        }
+    uint32_t kfirst, k_count;  // first k of this thread's micro-block; how many of its 8 k values are inside K
+    uint32_t K_;
+    __device__ inline void begin_fetch(const Operand&, uint32_t k0, uint32_t K) {
+        kfirst = k0 + (threadIdx.x % 8) * 8;
+        k_count = kfirst >= K ? 0 : (K - kfirst < 8 ? K - kfirst : 8);
+        K_ = K;
     }
-    __device__ inline void commit(T* tile) const {
+    __device__ inline void fetch_one(int idx, const Operand& op, uint32_t row0) {
+        const int i = idx / 8, kk = idx % 8;
+        const uint32_t rb = (threadIdx.x + kThreads * i) / 8;
+        const uint32_t row = row0 + rb * 8;
+        const uint32_t srow = (rb < ROWS / 8 && row < op.rows) ? row : 0;
+        const uint32_t k = kfirst + kk;
+        regs[i][kk] = *reinterpret_cast<const uint4v*>(static_cast<const T*>(op.base) + static_cast<int64_t>(k < K_ ? k : 0) * op.k_stride + srow);
+    }
+    __device__ inline void commit_one(int idx, T* tile) const {
+        const int i = idx / 8, rr = idx % 8;
+        const uint32_t mb = threadIdx.x + kThreads * i;
+        const uint32_t kb = mb % 8, rb = mb / 8;
+        if (rb >= ROWS / 8) return;
+        // row rr of the transposed micro-block: element rr of each of the 8 loaded vectors
+        uint16_t out[8];
 #pragma unroll
-        for (int i = 0; i < PASSES; ++i) {
-            const uint32_t mb = threadIdx.x + kThreads * i;
-            const uint32_t kb = mb % 8, rb = mb / 8;
-            if (rb >= ROWS / 8) continue;
-            uint16_t in[8][8], out[8][8];
-#pragma unroll
-            for (int kk = 0; kk < 8; ++kk) __builtin_memcpy(in[kk], &regs[i][kk], 16);
-#pragma unroll
-            for (int rr = 0; rr < 8; ++rr)
-#pragma unroll
-                for (int kk = 0; kk < 8; ++kk) out[rr][kk] = in[kk][rr];
-#pragma unroll
-            for (int rr = 0; rr < 8; ++rr) {
-                uint4v v;
-                __builtin_memcpy(&v, out[rr], 16);
-                *reinterpret_cast<uint4v*>(tile + tile_offset(rb * 8 + rr, kb)) = v;
-            }
+        for (int kk = 0; kk < 8; ++kk) {
+            uint16_t in[8];
+            __builtin_memcpy(in, &regs[i][kk], 16);
+            out[kk] = static_cast<uint32_t>(kk) < k_count ? in[rr] : uint16_t(0);
         }
+        uint4v v;
+        __builtin_memcpy(&v, out, 16);
+        *reinterpret_cast<uint4v*>(tile + tile_offset(rb * 8 + rr, kb)) = v;
     }
 };
 
@@ -152,9 +165,9 @@ __global__ __launch_bounds__(kThreads) void gemm16_kernel(const T* A, const T* B
     constexpr int WM = BM / 2, WN = BN / 2;   // 2 x 2 wavefronts
     constexpr int TM = WM / 32, TN = WN / 32;
     extern __shared__ __align__(16) unsigned char lds_raw[];
+    // layout: A buffer 0, A buffer 1, B buffer 0, B buffer 1 (offsets in elements)
     T* lds = reinterpret_cast<T*>(lds_raw);
-    T* sA[2] = {lds, lds + BM * kBK};
-    T* sB[2] = {lds + 2 * BM * kBK, lds + 2 * BM * kBK + BN * kBK};
+    constexpr uint32_t A_TILE = BM * kBK, B_TILE = BN * kBK, B_BASE = 2 * A_TILE;
 
     uint32_t tm, tn;
     tile_of(blockIdx.x, tiles_m, tiles_n, tm, tn);
@@ -178,39 +191,92 @@ __global__ __launch_bounds__(kThreads) void gemm16_kernel(const T* A, const T* B
 
     Loader<T, BM, A_KMAJOR> la;
     Loader<T, BN, B_KMAJOR> lb;
-    la.fetch(opA, m0, 0, p.K);
-    lb.fetch(opB, n0, 0, p.K);
-    la.commit(sA[0]);
-    lb.commit(sB[0]);
+    using LA = Loader<T, BM, A_KMAJOR>;
+    using LB = Loader<T, BN, B_KMAJOR>;
+    const uint32_t steps = (p.K + kBK - 1) / kBK;
+
+    // prologue: tile 0 into LDS buffer 0, tile 1 into registers
+    la.begin_fetch(opA, 0, p.K);
+    lb.begin_fetch(opB, 0, p.K);
+#pragma unroll
+    for (int i = 0; i < LA::LOADS; ++i) la.fetch_one(i, opA, m0);
+#pragma unroll
+    for (int i = 0; i < LB::LOADS; ++i) lb.fetch_one(i, opB, n0);
+#pragma unroll
+    for (int i = 0; i < LA::STORES; ++i) la.commit_one(i, lds);
+#pragma unroll
+    for (int i = 0; i < LB::STORES; ++i) lb.commit_one(i, lds + B_BASE);
+    if (steps > 1) {
+        la.begin_fetch(opA, kBK, p.K);
+        lb.begin_fetch(opB, kBK, p.K);
+#pragma unroll
+        for (int i = 0; i < LA::LOADS; ++i) la.fetch_one(i, opA, m0);
+#pragma unroll
+        for (int i = 0; i < LB::LOADS; ++i) lb.fetch_one(i, opB, n0);
+    }
     __syncthreads();
 
-    const uint32_t steps = (p.K + kBK - 1) / kBK;
-    for (uint32_t s = 0; s < steps; ++s) {
-        const int cur = s & 1;
-        if (s + 1 < steps) {
-            la.fetch(opA, m0, (s + 1) * kBK, p.K);
-            lb.fetch(opB, n0, (s + 1) * kBK, p.K);
+    // One K step.  The registers hold tile s+1 on entry.  The 4*TM*TN MFMAs of
+    // the step are issued in order; between them, one memory operation at a time:
+    // first the LDS writes of tile s+1 (into the buffer the previous step read),
+    // then the global loads of tile s+2 (into the registers just written out).
+    // sched_barrier pins that interleaving so that neither the load unit nor the
+    // LDS ever sees a burst while the matrix pipe idles.
+    auto step = [&](uint32_t s, auto commit_tag, auto fetch_tag) {
+        constexpr bool COMMIT = decltype(commit_tag)::value, FETCH = decltype(fetch_tag)::value;
+        constexpr int KS = kBK / 16, PER_KS = TM * TN, MFMAS = KS * PER_KS;
+        constexpr int NCA = LA::STORES, NCB = LB::STORES, NFA = LA::LOADS, NFB = LB::LOADS;
+        constexpr int OPS = NCA + NCB + NFA + NFB;
+        const uint32_t cur = s & 1;
+        const T* a_tile = lds + cur * A_TILE;
+        const T* b_tile = lds + B_BASE + cur * B_TILE;
+        T* a_next = lds + (cur ^ 1) * A_TILE;
+        T* b_next = lds + B_BASE + (cur ^ 1) * B_TILE;
+        if constexpr (FETCH) {
+            la.begin_fetch(opA, (s + 2) * kBK, p.K);
+            lb.begin_fetch(opB, (s + 2) * kBK, p.K);
         }
-        const T* a_tile = sA[cur];
-        const T* b_tile = sB[cur];
+        uint4v fa[2][TM], fb[2][TN];
 #pragma unroll
-        for (int ks = 0; ks < kBK / 16; ++ks) {
-            uint4v fa[TM], fb[TN];
+        for (int i = 0; i < TM; ++i) fa[0][i] = *reinterpret_cast<const uint4v*>(a_tile + tile_offset(wm + i * 32 + frag_row, frag_chunk));
 #pragma unroll
-            for (int i = 0; i < TM; ++i) fa[i] = *reinterpret_cast<const uint4v*>(a_tile + tile_offset(wm + i * 32 + frag_row, ks * 2 + frag_chunk));
+        for (int j = 0; j < TN; ++j) fb[0][j] = *reinterpret_cast<const uint4v*>(b_tile + tile_offset(wn + j * 32 + frag_row, frag_chunk));
+        static_for<MFMAS>([&](auto m_tag) {
+            constexpr int m = decltype(m_tag)::value;
+            constexpr int ks = m / PER_KS, i = (m % PER_KS) / TN, j = m % TN;
+            constexpr int now = ks & 1, nxt = now ^ 1;
+            if constexpr (m % PER_KS == 0) {
+                if constexpr (ks + 1 < KS) {
+                    // fragments of k-slice ks+1 are requested before the MFMAs of slice ks
 #pragma unroll
-            for (int j = 0; j < TN; ++j) fb[j] = *reinterpret_cast<const uint4v*>(b_tile + tile_offset(wn + j * 32 + frag_row, ks * 2 + frag_chunk));
+                    for (int x = 0; x < TM; ++x)
+                        fa[nxt][x] = *reinterpret_cast<const uint4v*>(a_tile + tile_offset(wm + x * 32 + frag_row, (ks + 1) * 2 + frag_chunk));
 #pragma unroll
-            for (int i = 0; i < TM; ++i)
-#pragma unroll
-                for (int j = 0; j < TN; ++j) acc[i][j] = Mfma16<T>::run(fa[i], fb[j], acc[i][j]);
-        }
-        if (s + 1 < steps) {
-            la.commit(sA[cur ^ 1]);
-            lb.commit(sB[cur ^ 1]);
-        }
+                    for (int y = 0; y < TN; ++y)
+                        fb[nxt][y] = *reinterpret_cast<const uint4v*>(b_tile + tile_offset(wn + y * 32 + frag_row, (ks + 1) * 2 + frag_chunk));
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            acc[i][j] = Mfma16<T>::run(fa[now][i], fb[now][j], acc[i][j]);
+            // memory operations [first, last) of the step go right after this MFMA
+            constexpr int first = m * OPS / MFMAS, last = (m + 1) * OPS / MFMAS;
+            static_for<last - first>([&](auto o_tag) {
+                constexpr int o = first + decltype(o_tag)::value;
+                if constexpr (o < NCA) { if constexpr (COMMIT) la.commit_one(o, a_next); }
+                else if constexpr (o < NCA + NCB) { if constexpr (COMMIT) lb.commit_one(o - NCA, b_next); }
+                else if constexpr (o < NCA + NCB + NFA) { if constexpr (FETCH) la.fetch_one(o - NCA - NCB, opA, m0); }
+                else { if constexpr (FETCH) lb.fetch_one(o - NCA - NCB - NFA, opB, n0); }
+            });
+            __builtin_amdgcn_sched_barrier(0);
+        });
         __syncthreads();
-    }
+    };
+    using Yes = std::true_type;
+    using No = std::false_type;
+    uint32_t s = 0;
+    for (; s + 2 < steps; ++s) step(s, Yes{}, Yes{});
+    if (s + 1 < steps) { step(s, Yes{}, No{}); ++s; }
+    step(s, No{}, No{});
 
     // accumulator layout of a 32x32 tile: lane -> column lane % 32; value v ->
     // row 8 * (v / 4) + 4 * (lane / 32) + v % 4
