@@ -1,0 +1,269 @@
+#!/usr/bin/env python3
+"""Benchmark of the device backend's hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--primary-only]
+
+Prints ONE JSON line.  A step is one pass of the hot path over one batch of
+synthetic input already resident in HBM: the fp16 GEMM Y = X . W^T at
+4096 x 4096 x 4096 with fp32 accumulation (the configuration the headline
+target is quoted on), evaluated the way the front end evaluates a `matmul`
+node: destination allocated, one backend call, destination released.
+
+The same line carries
+  roofline      the GEMM kernel's rate from HIP events on its stream, against
+                the published dense fp16 MFMA peak;
+  cpu_baseline  the CPU restatement of the reference's gemm (one core, as the
+                reference is single threaded) timed on a bounded sample;
+  workloads     the other configurations: GEMM sweep, conv2d layers, the
+                elementwise ops of the broadcast chain and the axis reductions,
+                each with its own roofline fraction.
+"""
+import argparse
+import ctypes as C
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+sys.path.insert(0, os.path.join(ROOT, "tests"))
+
+import numpy as np  # noqa: E402
+
+MFMA_PEAK_TFLOPS = {"f16": 2500.0, "bf16": 2500.0, "f32": 157.3}
+HBM_PEAK_GBS = 8000.0
+
+
+def parse():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--primary-only", action="store_true", help="skip the secondary workloads and the CPU baseline")
+    return ap.parse_args()
+
+
+class Bench:
+    def __init__(self):
+        import tannic_amd as ta
+        from tannic_amd import abi, ops
+        self.ta, self.abi, self.ops = ta, abi, ops
+        self.lib = ta.library()
+        self.device = ta.Device(0)
+        self.dvc = self.device.structure()
+        s = self.lib.pop_stream(C.byref(self.dvc))
+        self.lib.put_stream(C.byref(self.dvc), s)
+        self.stream = s   # the pool hands this same stream to every operator call
+        self.e0, self.e1 = self.lib.event_create(), self.lib.event_create()
+
+    def sync(self):
+        self.lib.device_synchronize()
+
+    def filled(self, dtype, shape, kind, seed, tid, scale=1.0):
+        """Device tensor with seeded values: 'normal' N(0, scale), 'uniform' U[-scale, scale)."""
+        import support
+        n = int(np.prod(shape))
+        period = min(n, 1 << 22)   # values repeat with this period: keeps host-side generation short
+        base = support.normal(seed, tid, (period,), scale) if kind == "normal" else support.uniform(seed, tid, (period,), -scale, scale)
+        if dtype.is_integral:
+            base = np.floor(base)
+        t = self.ta.Tensor(dtype, shape).initialize(self.device)
+        t.write(np.resize(base, n).reshape(shape))
+        return t
+
+    def raw_call(self, name, sources, dst, extra=(), scalar=None):
+        """Closure making one C-ABI call on pre-built descriptors (no allocation, no Python front end)."""
+        descs = [s.descriptor() for s in sources]
+        out = dst.descriptor()
+        args = [C.byref(d) for d in descs]
+        if scalar is not None:
+            args.append(C.byref(scalar))
+        args += [C.byref(out), self.stream] + list(extra)
+        fn = self.lib.kernels[name]
+
+        def run():
+            rc = fn(*args)
+            if rc != 0:
+                raise RuntimeError(f"{name}: status {rc} {self.lib.error_message()}")
+        run.keep = (descs, out, sources, dst, scalar)
+        return run
+
+    def event_time(self, run, iters, warm=2):
+        """Average milliseconds per call, from HIP events recorded on the stream the kernels run on."""
+        for _ in range(warm):
+            run()
+        self.lib.event_record(self.e0, self.stream)
+        for _ in range(iters):
+            run()
+        self.lib.event_record(self.e1, self.stream)
+        return self.lib.event_elapsed_ms(self.e0, self.e1) / iters
+
+
+def gemm_entry(b, dtype, M, N, K, iters):
+    ta = b.ta
+    x = b.filled(dtype, (M, K), "normal", 0, 1, 1.0)
+    w = b.filled(dtype, (N, K), "normal", 0, 2, 0.02)
+    y = ta.Tensor(dtype, (M, N)).initialize(b.device)
+    ms = b.event_time(b.raw_call("gemm", [x, w.transpose()], y), iters)
+    flops = 2.0 * M * N * K
+    nbytes = (M * K + N * K + M * N) * dtype.itemsize
+    tflops, gbs = flops / ms / 1e9, nbytes / ms / 1e6
+    hbm_bound = flops / nbytes < 312.0   # below the ridge of 2.5 PFLOP/s over 8 TB/s
+    return {"op": f"gemm {dtype} X[{M},{K}].W[{N},{K}]^T", "us": round(ms * 1e3, 2), "tflops": round(tflops, 2), "gbs": round(gbs, 1),
+            "bound": "hbm" if hbm_bound else "mfma",
+            "frac": round(gbs / HBM_PEAK_GBS if hbm_bound else tflops / MFMA_PEAK_TFLOPS["f16"], 4)}
+
+
+def conv_entry(b, dtype, name, xs, ws, stride, pad, iters):
+    ta = b.ta
+    fan_in = ws[1] * ws[2] * ws[3]
+    x = b.filled(dtype, xs, "normal", 0, 3, 1.0)
+    w = b.filled(dtype, ws, "normal", 0, 4, (2.0 / fan_in) ** 0.5)
+    bias = ta.Tensor(dtype, (ws[0],)).initialize(np.zeros(ws[0]), b.device)
+    ho, wo = (xs[2] + 2 * pad - ws[2]) // stride + 1, (xs[3] + 2 * pad - ws[3]) // stride + 1
+    y = ta.Tensor(dtype, (xs[0], ws[0], ho, wo)).initialize(b.device)
+    extra = (b.abi.SIZE2(pad, pad), b.abi.SIZE2(stride, stride))
+    ms = b.event_time(b.raw_call("conv2d_biased", [x, w, bias], y, extra), iters)
+    flops = 2.0 * xs[0] * ws[0] * ho * wo * fan_in
+    touched = xs[0] * xs[1] * (min(xs[2], (ho - 1) * stride + ws[2]) * min(xs[3], (wo - 1) * stride + ws[3]) if stride <= ws[2] else ho * wo)
+    nbytes = (touched + int(np.prod(ws)) + y.nelements) * dtype.itemsize
+    peak = MFMA_PEAK_TFLOPS["f32" if dtype is ta.float32 else "f16"]
+    tflops = flops / ms / 1e9
+    return {"op": f"conv2d {dtype} {name}", "us": round(ms * 1e3, 2), "tflops": round(tflops, 2), "gbs": round(nbytes / ms / 1e6, 1),
+            "mfma_frac": round(tflops / peak, 4), "hbm_frac": round(nbytes / ms / 1e6 / HBM_PEAK_GBS, 4)}
+
+
+def elementwise_entries(b, dtype, iters):
+    ta, abi, ops = b.ta, b.abi, b.ops
+    shape = (64, 4096, 1024)
+    nb = int(np.prod(shape)) * dtype.itemsize
+    x = b.filled(dtype, shape, "uniform", 0, 5, 4.0)
+    x2 = b.filled(dtype, shape, "uniform", 0, 6, 4.0)
+    z = b.filled(dtype, (1, 4096, 1), "uniform", 0, 7, 4.0)
+    one = ta.Tensor(dtype, (1,)).initialize(np.ones(1), b.device)
+    y = ta.Tensor(dtype, shape).initialize(b.device)
+    out = []
+
+    def add(label, run, traffic):
+        ms = b.event_time(run, iters)
+        out.append({"op": f"{label} {dtype}", "us": round(ms * 1e3, 1), "gbs": round(traffic / ms / 1e6, 1), "bound": "hbm",
+                    "frac": round(traffic / ms / 1e6 / HBM_PEAK_GBS, 4)})
+    if dtype.is_floating:
+        add("abs(X)", b.raw_call("abs", [x], y), 2 * nb)
+        add("X + 1 (one-element operand)", b.raw_call("add", [x, one], y), 2 * nb)
+        add("log(X)", b.raw_call("log", [x], y), 2 * nb)
+        add("exp(X)", b.raw_call("exp", [x], y), 2 * nb)
+        add("X + Z[1,4096,1] (broadcast)", b.raw_call("add", [x, z], y), 2 * nb)
+        add("X - X2 (full)", b.raw_call("sub", [x, x2], y), 3 * nb)
+        raw = C.create_string_buffer(ops.scalar_bytes(3, dtype), 16)
+        add("3 * X (scale)", b.raw_call("scale", [x], y, scalar=abi.scalar_t(C.cast(raw, C.c_void_p), dtype.code)), 2 * nb)
+    else:
+        add("X + Z[1,4096,1] (broadcast)", b.raw_call("add", [x, z], y), 2 * nb)
+        mask = ta.Tensor(ta.boolean, shape).initialize(b.device)
+        add("X > X2 (bit-packed)", b.raw_call("gt", [x, x2], mask), 2 * nb + mask.nbytes)
+    return out
+
+
+def reduction_entries(b, dtype, iters):
+    ta = b.ta
+    shape = (64, 4096, 1024)
+    nb = int(np.prod(shape)) * dtype.itemsize
+    x = b.filled(dtype, shape, "uniform", 0, 8, 4.0)
+    out = []
+    for axis in (2, 1):
+        oshape = tuple(s for d, s in enumerate(shape) if d != axis)
+        for name in ("argsum", "argmean", "max", "min", "argmax"):
+            odt = ta.int64 if name == "argmax" else dtype
+            y = ta.Tensor(odt, oshape).initialize(b.device)
+            ms = b.event_time(b.raw_call(name, [x], y, (C.c_uint8(axis),)), iters)
+            traffic = nb + y.nbytes
+            out.append({"op": f"{name[3:] if name in ('argsum', 'argmean') else name} {dtype} axis={axis}", "us": round(ms * 1e3, 1),
+                        "gbs": round(traffic / ms / 1e6, 1), "bound": "hbm", "frac": round(traffic / ms / 1e6 / HBM_PEAK_GBS, 4)})
+    return out
+
+
+def cpu_baseline(rows=64):
+    """The CPU restatement of the reference gemm on the first `rows` rows of the same problem, one core."""
+    import support
+    import tannic_amd as ta
+    from tannic_amd import ops
+    oracle = support.oracle_library()
+    ops.set_host_functions(oracle.functions)
+    K = N = 4096
+    x = support.host_tensor(support.normal(0, 1, (rows, K)).astype(np.float16), ta.float16)
+    w = support.host_tensor(np.resize(support.normal(0, 2, (1 << 22,), 0.02), N * K).reshape(N, K).astype(np.float16), ta.float16)
+    t0 = time.perf_counter()
+    ops.matmul(x, w.transpose())
+    dt = time.perf_counter() - t0
+    return {"value": round(2.0 * rows * N * K / dt / 1e12, 6), "unit": "TFLOP/s", "cores": 1, "kind": "port",
+            "sample": f"first {rows} rows of X: [{rows},4096] . [4096,4096]^T fp16, fp32 accumulate, {dt:.1f} s of {os.cpu_count()} host CPUs' one core"}
+
+
+def main():
+    args = parse()
+    if args.gpus != 1:
+        print("bench.py: this build measures one GPU; --gpus above 1 is not supported (nothing in the hot path is sharded)", file=sys.stderr)
+        sys.exit(2)
+    b = Bench()
+    ta, ops = b.ta, b.ops
+    M = N = K = 4096
+    x = b.filled(ta.float16, (M, K), "normal", 0, 1, 1.0)
+    w = b.filled(ta.float16, (N, K), "normal", 0, 2, 0.02)
+    wt = w.transpose()
+
+    def step():
+        return ops.matmul(x, wt)   # allocates the destination, one gemm call, destination released on drop
+
+    for _ in range(args.warmup):
+        step()
+    b.sync()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    b.sync()
+    wall = time.perf_counter() - t0
+    ms_per_step = wall * 1e3 / args.steps
+    flops = 2.0 * M * N * K
+    value = flops / (ms_per_step * 1e-3) / 1e12
+
+    # the kernel alone, from events on its stream
+    y = ta.Tensor(ta.float16, (M, N)).initialize(b.device)
+    kernel_ms = b.event_time(b.raw_call("gemm", [x, wt], y), max(args.steps, 10))
+    achieved = flops / kernel_ms / 1e9
+    roofline = {"bound": "mfma", "kernel": "gemm16_kernel<f16,256,256,k-major,k-major>", "achieved": round(achieved, 2),
+                "peak": MFMA_PEAK_TFLOPS["f16"], "unit": "TFLOP/s", "frac": round(achieved / MFMA_PEAK_TFLOPS["f16"], 4),
+                "avg_kernel_us": round(kernel_ms * 1e3, 2), "traffic": None}
+    del y
+
+    result = {
+        "metric": "fp16 GEMM/conv TFLOP/s + elementwise/reduce GB/s, % of MI355X roofline",
+        "value": round(value, 2), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f16 (fp32 accumulate)", "data": "synthetic",
+        "config": {"workload": "fp16 GEMM Y = X.W^T, X[4096,4096] N(0,1), W[4096,4096] N(0,0.02), seed 0 (square case of the GEMM sweep)",
+                   "step": "front-end matmul node: allocate dst, one gemm call, release dst"},
+        "roofline": roofline,
+    }
+    del x, w, wt
+
+    if not args.primary_only:
+        work = []
+        for (m, n) in [(2048, 4096), (2048, 14336), (128, 4096), (128, 14336), (16, 4096), (16, 14336), (1, 4096), (1, 14336)]:
+            work.append(gemm_entry(b, ta.float16, m, n, 4096, 20))
+        work.append(gemm_entry(b, ta.bfloat16, 4096, 4096, 4096, 20))
+        for dtype in (ta.float16, ta.float32):
+            work.append(conv_entry(b, dtype, "3->64 k7 s2 p3 @224 N=32", (32, 3, 224, 224), (64, 3, 7, 7), 2, 3, 5))
+            work.append(conv_entry(b, dtype, "64->64 k3 s1 p1 @56 N=32", (32, 64, 56, 56), (64, 64, 3, 3), 1, 1, 5))
+            work.append(conv_entry(b, dtype, "256->512 k1 s2 @56 N=32", (32, 256, 56, 56), (512, 256, 1, 1), 2, 0, 5))
+        for dtype in (ta.float32, ta.float16, ta.int32):
+            work += elementwise_entries(b, dtype, 10)
+        for dtype in (ta.float32, ta.float16):
+            work += reduction_entries(b, dtype, 10)
+        result["workloads"] = work
+        result["cpu_baseline"] = cpu_baseline()
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()
