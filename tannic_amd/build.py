@@ -39,6 +39,7 @@ UNITS = [
     ("gemm_mfma.hip", "gemm_mfma.o", []),
     ("conv2d.hip", "conv2d.o", []),
     ("conv2d_mfma.hip", "conv2d_mfma.o", []),
+    ("conv2d_patch.hip", "conv2d_patch.o", []),
 ]
 
 

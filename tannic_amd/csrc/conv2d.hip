@@ -89,7 +89,9 @@ static int conv2d_entry(const tannic_tensor_t* x, const tannic_tensor_t* w, cons
     // the bias is read as b[co]: element stride 1 (src/cpu/conv2d.cpp:90)
     const void* pb = bias ? bias->address : nullptr;
     hipStream_t s = as_stream(stream);
-    int status = conv2d_mfma(p, x->dtype, x->address, w->address, pb, y->address, s);
+    int status = conv2d_patch(p, x->dtype, x->address, w->address, pb, y->address, s);
+    if (status != TANNIC_UNSUPPORTED_DTYPE) return status;
+    status = conv2d_mfma(p, x->dtype, x->address, w->address, pb, y->address, s);
     if (status != TANNIC_UNSUPPORTED_DTYPE) return status;
     switch (x->dtype) {
         case TANNIC_INT8: return run_direct<int8_t>(p, x->address, w->address, pb, y->address, s);

@@ -26,6 +26,13 @@ CASES = {
     "rect_kernel_rect_stride": ((1, 5, 13, 9), (7, 5, 3, 2), (2, 1), (0, 2)),
     "one_pixel_out": ((3, 4, 3, 3), (5, 4, 3, 3), (1, 1), (0, 0)),
     "wide_padding": ((1, 2, 4, 4), (3, 2, 3, 3), (1, 1), (2, 2)),
+    # channel counts that are multiples of 32 with rows of 8n columns: the LDS-patch kernel
+    "patch_k3_s1_p1": ((2, 32, 8, 8), (16, 32, 3, 3), (1, 1), (1, 1)),
+    "patch_k3_64ch_rows": ((1, 64, 24, 56), (64, 64, 3, 3), (1, 1), (1, 1)),
+    "patch_k1_s2": ((2, 64, 16, 16), (96, 64, 1, 1), (2, 2), (0, 0)),
+    "patch_k5_s2_p2": ((1, 32, 24, 16), (40, 32, 5, 5), (2, 2), (2, 2)),
+    "patch_many_out_channels": ((1, 96, 8, 24), (200, 96, 3, 3), (1, 1), (1, 1)),
+    "patch_rect_stride": ((2, 32, 9, 16), (8, 32, 2, 3), (1, 2), (1, 0)),
 }
 
 
