@@ -40,6 +40,7 @@ UNITS = [
     ("conv2d.hip", "conv2d.o", []),
     ("conv2d_mfma.hip", "conv2d_mfma.o", []),
     ("conv2d_patch.hip", "conv2d_patch.o", []),
+    ("conv2d_resident.hip", "conv2d_resident.o", []),
 ]
 
 

@@ -76,12 +76,64 @@ static void retain_pool_memory(int device) {
     (void)hipGetLastError();
 }
 
+// Work scratch of the kernels (partial results, rearranged weights, flags).
+// Blocks are kept per stream and handed out again to later calls on the SAME
+// stream: stream order already separates the kernels of the earlier call from
+// those of the later one, so no allocation and no free sits on the hot path.
+struct ScratchBlock {
+    void* ptr;
+    size_t size;
+    hipStream_t stream;
+    int device;
+};
+static std::mutex g_scratch_mutex;
+static std::vector<ScratchBlock> g_scratch_free, g_scratch_live;
+static size_t g_scratch_cached = 0;
+constexpr size_t kScratchCacheLimit = size_t(2) << 30;
+
 int scratch_acquire(void** ptr, size_t nbytes, hipStream_t stream) {
-    TH_TRY(hipMallocAsync(ptr, nbytes, stream));
+    int device = 0;
+    TH_TRY(hipGetDevice(&device));
+    {
+        std::lock_guard<std::mutex> lock(g_scratch_mutex);
+        size_t best = g_scratch_free.size();
+        for (size_t i = 0; i < g_scratch_free.size(); ++i) {
+            const ScratchBlock& b = g_scratch_free[i];
+            if (b.stream == stream && b.device == device && b.size >= nbytes && (best == g_scratch_free.size() || b.size < g_scratch_free[best].size)) best = i;
+        }
+        if (best != g_scratch_free.size()) {
+            ScratchBlock b = g_scratch_free[best];
+            g_scratch_free.erase(g_scratch_free.begin() + best);
+            g_scratch_cached -= b.size;
+            g_scratch_live.push_back(b);
+            *ptr = b.ptr;
+            return TANNIC_SUCCESS;
+        }
+    }
+    const size_t size = (nbytes + 0xFFFF) & ~size_t(0xFFFF);
+    TH_TRY(hipMalloc(ptr, size ? size : 0x10000));
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    g_scratch_live.push_back(ScratchBlock{*ptr, size ? size : 0x10000, stream, device});
     return TANNIC_SUCCESS;
 }
 
 int scratch_release(void* ptr, hipStream_t stream) {
+    ScratchBlock block{nullptr, 0, stream, 0};
+    {
+        std::lock_guard<std::mutex> lock(g_scratch_mutex);
+        for (size_t i = 0; i < g_scratch_live.size(); ++i)
+            if (g_scratch_live[i].ptr == ptr) {
+                block = g_scratch_live[i];
+                g_scratch_live.erase(g_scratch_live.begin() + i);
+                break;
+            }
+        if (block.ptr && g_scratch_cached + block.size <= kScratchCacheLimit) {
+            g_scratch_free.push_back(block);
+            g_scratch_cached += block.size;
+            return TANNIC_SUCCESS;
+        }
+    }
+    // over the cache limit (or unknown pointer): give it back once the stream has passed this point
     TH_TRY(hipFreeAsync(ptr, stream));
     return TANNIC_SUCCESS;
 }
