@@ -135,7 +135,7 @@ __device__ inline Pack<T, N> load_or_splat(const T* p, bool splat) {
 }
 
 constexpr int kBlock = 256;
-constexpr int kUnroll = 4;
+constexpr int kUnroll = 1;
 
 // Element offsets of vector `v` in the three operands.
 struct Offsets {

@@ -181,29 +181,51 @@ __device__ inline bool compare(T x, T y) {
     else return x <= y;
 }
 
-template <class T, int K, bool FLAT>
+// Strided operands: a thread produces one output byte from eight consecutive elements.
+template <class T, int K>
 __global__ __launch_bounds__(kBlock) void compare_kernel(const T* a, const T* b, uint8_t* out, uint32_t ne, Plan p) {
     const uint32_t byte = blockIdx.x * kBlock + threadIdx.x;
     const uint32_t first = byte * 8;
     if (first >= ne) return;
     uint32_t bits = 0;
-    if (FLAT && first + 8 <= ne) {
-        constexpr int N = sizeof(T) >= 16 ? 1 : (16 / sizeof(T) > 8 ? 8 : 16 / sizeof(T));
-#pragma unroll
-        for (int g = 0; g < 8 / N; ++g) {
-            const Pack<T, N> x = load_pack<T, N>(a + first + g * N);
-            const Pack<T, N> y = load_pack<T, N>(b + first + g * N);
-#pragma unroll
-            for (int i = 0; i < N; ++i) bits |= static_cast<uint32_t>(compare<K>(x.v[i], y.v[i])) << (g * N + i);
-        }
-    } else {
-        const uint32_t n = ne - first < 8 ? ne - first : 8;
-        for (uint32_t i = 0; i < n; ++i) {
-            const Offsets o = decode<1>(p, first + i);
-            bits |= static_cast<uint32_t>(compare<K>(a[o.o0], b[o.o1])) << i;
-        }
+    const uint32_t n = ne - first < 8 ? ne - first : 8;
+    for (uint32_t i = 0; i < n; ++i) {
+        const Offsets o = decode<1>(p, first + i);
+        bits |= static_cast<uint32_t>(compare<K>(a[o.o0], b[o.o1])) << i;
     }
     out[byte] = static_cast<uint8_t>(bits);
+}
+
+// Contiguous operands: every lane reads ONE 16-byte vector per operand (fully coalesced) and turns it
+// into N = 16 / sizeof(T) result bits; lanes that hold less than a byte pass their bits down to the
+// first lane of their byte.
+template <class T, int K>
+__global__ __launch_bounds__(kBlock) void compare_flat_kernel(const T* a, const T* b, uint8_t* out, uint32_t ne) {
+    constexpr int N = 16 / sizeof(T);
+    const uint32_t t = blockIdx.x * kBlock + threadIdx.x;
+    const uint32_t first = t * N;
+    uint32_t bits = 0;
+    if (first + N <= ne) {
+        const Pack<T, N> x = load_pack<T, N>(a + first);
+        const Pack<T, N> y = load_pack<T, N>(b + first);
+#pragma unroll
+        for (int i = 0; i < N; ++i) bits |= static_cast<uint32_t>(compare<K>(x.v[i], y.v[i])) << i;
+    } else if (first < ne) {
+        for (uint32_t i = 0; first + i < ne; ++i) bits |= static_cast<uint32_t>(compare<K>(a[first + i], b[first + i])) << i;
+    }
+    if constexpr (N >= 8) {
+        // N = 8: one byte; N = 16: two bytes
+        if (first < ne) {
+            out[first / 8] = static_cast<uint8_t>(bits);
+            if (N == 16 && first + 8 < ne) out[first / 8 + 1] = static_cast<uint8_t>(bits >> 8);
+        }
+    } else {
+        // 8 / N consecutive lanes make one byte (a wavefront never splits a byte: 64 * N is a multiple of 8)
+        constexpr int LANES = 8 / N;
+#pragma unroll
+        for (int s = 1; s < LANES; ++s) bits |= __shfl_down(bits & ((1u << N) - 1u), s) << (s * N);
+        if (t % LANES == 0 && first < ne) out[first / 8] = static_cast<uint8_t>(bits);
+    }
 }
 
 template <class T, int K>
@@ -234,12 +256,14 @@ int run_compare(const tannic_tensor_t* a, const tannic_tensor_t* b, tannic_tenso
                       reinterpret_cast<uintptr_t>(pa) % 16 == 0 && reinterpret_cast<uintptr_t>(pb) % 16 == 0;
     const uint32_t bytes = (ne + 7) / 8;
     const uint32_t grid = (bytes + kBlock - 1) / kBlock;
+    constexpr uint32_t PER_THREAD = 16 / sizeof(T);
+    const uint32_t flat_grid = ((ne + PER_THREAD - 1) / PER_THREAD + kBlock - 1) / kBlock;
     // The CPU path ORs a true result into a rank-0 destination and leaves a false
     // one untouched (src/cpu/cmps.cpp:87-93), which reads memory nobody wrote.
     // Here the byte is always written: 1 or 0.
-    if (flat) hipLaunchKernelGGL((compare_kernel<T, K, true>), dim3(grid), dim3(kBlock), 0, stream, pa, pb,
-                                 static_cast<uint8_t*>(dst->address), ne, plan);
-    else hipLaunchKernelGGL((compare_kernel<T, K, false>), dim3(grid), dim3(kBlock), 0, stream, pa, pb,
+    if (flat) hipLaunchKernelGGL((compare_flat_kernel<T, K>), dim3(flat_grid), dim3(kBlock), 0, stream, pa, pb,
+                                 static_cast<uint8_t*>(dst->address), ne);
+    else hipLaunchKernelGGL((compare_kernel<T, K>), dim3(grid), dim3(kBlock), 0, stream, pa, pb,
                             static_cast<uint8_t*>(dst->address), ne, plan);
     return launch_status("compare_kernel");
 }

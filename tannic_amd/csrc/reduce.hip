@@ -33,11 +33,12 @@ __device__ inline uint32_t dpp32(uint32_t v) {
 
 template <int CTRL, class T>
 __device__ inline T dpp(T v) {
-    static_assert(sizeof(T) % 4 == 0, "DPP moves 32-bit registers");
-    uint32_t w[sizeof(T) / 4];
+    // DPP moves 32-bit registers: narrower values ride in one
+    constexpr size_t WORDS = (sizeof(T) + 3) / 4;
+    uint32_t w[WORDS] = {};
     __builtin_memcpy(w, &v, sizeof(T));
 #pragma unroll
-    for (size_t i = 0; i < sizeof(T) / 4; ++i) w[i] = dpp32<CTRL>(w[i]);
+    for (size_t i = 0; i < WORDS; ++i) w[i] = dpp32<CTRL>(w[i]);
     T r;
     __builtin_memcpy(&r, w, sizeof(T));
     return r;
@@ -45,10 +46,11 @@ __device__ inline T dpp(T v) {
 
 template <class T>
 __device__ inline T read_lane(T v, int lane) {
-    uint32_t w[sizeof(T) / 4];
+    constexpr size_t WORDS = (sizeof(T) + 3) / 4;
+    uint32_t w[WORDS] = {};
     __builtin_memcpy(w, &v, sizeof(T));
 #pragma unroll
-    for (size_t i = 0; i < sizeof(T) / 4; ++i) w[i] = static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(w[i]), lane));
+    for (size_t i = 0; i < WORDS; ++i) w[i] = static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(w[i]), lane));
     T r;
     __builtin_memcpy(&r, w, sizeof(T));
     return r;
@@ -140,13 +142,35 @@ struct ArgOp {
         const bool strictly = MAX ? gt(v, than.value) : gt(than.value, v);
         return strictly || (same(v, than.value) && i < than.index);
     }
+    // a lane meets its elements in increasing index order, so inside a lane "strictly better" is the whole
+    // rule; the lower-index tie-break only matters when partial results meet (combine)
     __device__ static inline A step(A acc, T v, uint32_t r) {
-        if (better(v, r, acc)) { acc.value = v; acc.index = r; }
+        const bool strictly = MAX ? gt(v, acc.value) : gt(acc.value, v);
+        acc.value = strictly ? v : acc.value;
+        acc.index = strictly ? r : acc.index;
         return acc;
     }
     __device__ static inline A combine(A x, A y) { return better(y.value, y.index, x) ? y : x; }
     __device__ static inline int64_t finish(A acc, uint32_t) { return static_cast<int64_t>(acc.index); }
 };
+
+// Value max / min = src[argmax] / src[argmin] without carrying the index: the strict maximum from the
+// -inf (lowest) start IS that element's value whenever anything beats the start; when nothing does
+// (a slice of NaN, of -inf, of the integer minimum) argmax is 0 and the answer is the slice's first element.
+template <class T, bool MAX>
+struct ValueOp {
+    using S = T;
+    using A = T;
+    using Out = T;
+    static constexpr bool needs_source = true;
+    static constexpr bool value_only = true;
+    __device__ static inline A init() { return arg_start<T, MAX>(); }
+    __device__ static inline A step(A acc, T v, uint32_t) { return (MAX ? gt(v, acc) : gt(acc, v)) ? v : acc; }
+    __device__ static inline A combine(A x, A y) { return (MAX ? gt(y, x) : gt(x, y)) ? y : x; }
+};
+
+template <class Op, class = void> struct is_value_only { static constexpr bool value = false; };
+template <class Op> struct is_value_only<Op, std::enable_if_t<Op::value_only>> { static constexpr bool value = true; };
 
 template <class T, int N>
 struct alignas(sizeof(T) * N >= 16 ? 16 : sizeof(T) * N) Vec {
@@ -173,7 +197,8 @@ __device__ inline Vec<T, N> load_vec(const T* p) {
 template <class Op>
 __device__ inline void emit(typename Op::A acc, uint32_t count, typename Op::Out* dst, size_t slot,
                             const typename Op::S* src, size_t first, size_t step) {
-    if constexpr (Op::needs_source) dst[slot] = src[first + static_cast<size_t>(acc.index) * step];
+    if constexpr (is_value_only<Op>::value) dst[slot] = same(acc, Op::init()) ? src[first] : acc;
+    else if constexpr (Op::needs_source) dst[slot] = src[first + static_cast<size_t>(acc.index) * step];
     else dst[slot] = Op::finish(acc, count);
 }
 
@@ -315,7 +340,8 @@ __global__ __launch_bounds__(kThreads) void reduce_strided_kernel(const typename
     const int64_t step = w.stride[w.axis];
     typename Op::A acc = Op::init();
     for (uint32_t r = 0; r < R; ++r) acc = Op::step(acc, src[base + static_cast<int64_t>(r) * step], r);
-    if constexpr (Op::needs_source) dst[slot] = src[base + static_cast<int64_t>(acc.index) * step];
+    if constexpr (is_value_only<Op>::value) dst[slot] = same(acc, Op::init()) ? src[base] : acc;
+    else if constexpr (Op::needs_source) dst[slot] = src[base + static_cast<int64_t>(acc.index) * step];
     else dst[slot] = Op::finish(acc, R);
 }
 
@@ -446,8 +472,8 @@ int reduce_entry(const tannic_tensor_t* src, tannic_tensor_t* dst, tannic_stream
             else if constexpr (K == R_MEAN) { if constexpr (!std::is_integral_v<T>) status = run_reduce<SumOp<T, true>>(src, dst, s, axis); }
             else if constexpr (K == R_ARGMAX) status = run_reduce<ArgOp<T, true, false>>(src, dst, s, axis);
             else if constexpr (K == R_ARGMIN) status = run_reduce<ArgOp<T, false, false>>(src, dst, s, axis);
-            else if constexpr (K == R_MAX) status = run_reduce<ArgOp<T, true, true>>(src, dst, s, axis);
-            else status = run_reduce<ArgOp<T, false, true>>(src, dst, s, axis);
+            else if constexpr (K == R_MAX) status = run_reduce<ValueOp<T, true>>(src, dst, s, axis);
+            else status = run_reduce<ValueOp<T, false>>(src, dst, s, axis);
         }
     });
     return status;
