@@ -35,12 +35,26 @@ MFMA_PEAK_TFLOPS = {"f16": 2500.0, "bf16": 2500.0, "f32": 157.3}
 HBM_PEAK_GBS = 8000.0
 
 
+def measured_traffic(name):
+    """HBM bytes per launch of a kernel, from the committed rocprofv3 counter summary under profiles/ (None if absent)."""
+    path = os.path.join(ROOT, "profiles", name)
+    try:
+        for line in open(path):
+            if line.strip().startswith("traffic_bytes_per_launch"):
+                return int(line.split("=")[1])
+    except OSError:
+        pass
+    return None
+
+
 def parse():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--primary-only", action="store_true", help="skip the secondary workloads and the CPU baseline")
+    ap.add_argument("--copy-only", action="store_true",
+                    help="run only a plain 1 GiB -> 1 GiB contiguous copy (repack): the known-size kernel that calibrates the HBM byte counters")
     return ap.parse_args()
 
 
@@ -207,6 +221,14 @@ def main():
         sys.exit(2)
     b = Bench()
     ta, ops = b.ta, b.ops
+    if args.copy_only:
+        shape = (64, 4096, 1024)
+        src = b.filled(ta.float32, shape, "uniform", 0, 9, 1.0)
+        dst = ta.Tensor(ta.float32, shape).initialize(b.device)
+        ms = b.event_time(b.raw_call("repack", [src], dst), args.steps)
+        print(json.dumps({"op": "repack float32 [64,4096,1024]", "bytes_read": src.nbytes, "bytes_written": dst.nbytes,
+                          "us": round(ms * 1e3, 1), "gbs": round(2 * src.nbytes / ms / 1e6, 1)}))
+        return
     M = N = K = 4096
     x = b.filled(ta.float16, (M, K), "normal", 0, 1, 1.0)
     w = b.filled(ta.float16, (N, K), "normal", 0, 2, 0.02)
@@ -233,7 +255,8 @@ def main():
     achieved = flops / kernel_ms / 1e9
     roofline = {"bound": "mfma", "kernel": "gemm16_kernel<f16,256,256,k-major,k-major>", "achieved": round(achieved, 2),
                 "peak": MFMA_PEAK_TFLOPS["f16"], "unit": "TFLOP/s", "frac": round(achieved / MFMA_PEAK_TFLOPS["f16"], 4),
-                "avg_kernel_us": round(kernel_ms * 1e3, 2), "traffic": None}
+                "avg_kernel_us": round(kernel_ms * 1e3, 2),
+                "traffic": measured_traffic("gemm16_fp16_4096x4096x4096_hbm_traffic.txt")}
     del y
 
     result = {
