@@ -6,9 +6,11 @@
 //   live in LDS as [row][64 k] with the eight 16-byte chunks of a row XOR-
 //   swizzled by the row number, so that the 16-byte fragment reads of a
 //   wavefront (32 rows x 2 chunks) and the tile writes are bank-conflict free.
-//   Tiles are double buffered: the global loads of step i+1 are issued before
-//   the MFMAs of step i and written to the other buffer after them; one barrier
-//   per step.  An operand that is contiguous along K is copied chunk by chunk;
+//   Tiles are double buffered in LDS and a third tile is in flight in registers:
+//   during step s every register of tile s+1 is written to the other LDS buffer
+//   and refilled from global memory with tile s+2, one memory operation between
+//   two MFMAs; one barrier per step, placed where the fragments of the next 16
+//   MFMAs are in registers already.  An operand that is contiguous along K is copied chunk by chunk;
 //   an operand that is contiguous along its row index (a transposed view of A,
 //   a plain row-major B) is read as 8x8 micro-blocks and transposed in
 //   registers on its way to LDS.
@@ -49,7 +51,6 @@ template <> struct Mfma16<bf16> {
 
 constexpr int kBK = 64;          // K elements per step (16-bit kernels)
 constexpr int kChunk = 8;        // 16-bit elements per 16-byte chunk
-constexpr int kThreads = 256;
 
 // Maps the hardware workgroup id to a tile: XCD folding, then grouped rows.
 __device__ inline void tile_of(uint32_t wg, uint32_t tiles_m, uint32_t tiles_n, uint32_t& tm, uint32_t& tn) {
@@ -95,9 +96,10 @@ __device__ inline uint32_t tile_offset(uint32_t row, uint32_t chunk) { return ro
 // touches the loaded values (and waits for them) early.
 // Both loaders expose their work as single memory operations (fetch_one /
 // commit_one) so that the main loop can spread them between MFMAs.
-template <class T, int ROWS>
+template <class T, int ROWS, int THREADS>
 struct KMajorLoader {
-    static constexpr int LOADS = ROWS / 32, STORES = ROWS / 32;
+    static constexpr int ROWS_PER_PASS = THREADS / 8;
+    static constexpr int LOADS = ROWS / ROWS_PER_PASS, STORES = ROWS / ROWS_PER_PASS;
     uint4v regs[LOADS];
     const T* base;      // operand base + this thread's k offset for the tile being fetched
     bool k_live;
@@ -107,20 +109,27 @@ struct KMajorLoader {
         base = static_cast<const T*>(op.base) + (k_live ? k : 0);
     }
     __device__ inline void fetch_one(int i, const Operand& op, uint32_t row0) {
-        const uint32_t row = row0 + threadIdx.x / 8 + 32 * i;
+        const uint32_t row = row0 + threadIdx.x / 8 + ROWS_PER_PASS * i;
         const uint32_t srow = row < op.rows ? row : op.rows - 1;
         regs[i] = *reinterpret_cast<const uint4v*>(base + static_cast<int64_t>(srow) * op.row_stride);
     }
+    template <bool MASK>
     __device__ inline void commit_one(int i, T* tile) const {
-        *reinterpret_cast<uint4v*>(tile + tile_offset(threadIdx.x / 8 + 32 * i, threadIdx.x % 8)) = k_live ? regs[i] : uint4v{0, 0, 0, 0};
+        *reinterpret_cast<uint4v*>(tile + tile_offset(threadIdx.x / 8 + ROWS_PER_PASS * i, threadIdx.x % 8)) =
+            (!MASK || k_live) ? regs[i] : uint4v{0, 0, 0, 0};
     }
+    // Order of the step's memory operations: register i is written to LDS and refilled right away, so
+    // that every load has a whole step to arrive.
+    static constexpr int OPS = STORES + LOADS;
+    static constexpr bool is_commit(int o) { return o % 2 == 0; }
+    static constexpr int index_of(int o) { return o / 2; }
 };
 
 // ---- operand contiguous along its row index: 8x8 micro-blocks, transposed --------
-template <class T, int ROWS>
+template <class T, int ROWS, int THREADS>
 struct RowMajorLoader {
-    // ROWS/8 row-blocks x 8 k-blocks micro-blocks, 256 threads
-    static constexpr int PASSES = (ROWS + 255) / 256;
+    // ROWS/8 row-blocks x 8 k-blocks micro-blocks over THREADS threads
+    static constexpr int PASSES = (ROWS + THREADS - 1) / THREADS;
     static constexpr int LOADS = 8 * PASSES, STORES = 8 * PASSES;
     uint4v regs[PASSES][8];
     uint32_t kfirst, k_count;  // first k of this thread's micro-block; how many of its 8 k values are inside K
@@ -132,15 +141,16 @@ struct RowMajorLoader {
     }
     __device__ inline void fetch_one(int idx, const Operand& op, uint32_t row0) {
         const int i = idx / 8, kk = idx % 8;
-        const uint32_t rb = (threadIdx.x + kThreads * i) / 8;
+        const uint32_t rb = (threadIdx.x + THREADS * i) / 8;
         const uint32_t row = row0 + rb * 8;
         const uint32_t srow = (rb < ROWS / 8 && row < op.rows) ? row : 0;
         const uint32_t k = kfirst + kk;
         regs[i][kk] = *reinterpret_cast<const uint4v*>(static_cast<const T*>(op.base) + static_cast<int64_t>(k < K_ ? k : 0) * op.k_stride + srow);
     }
+    template <bool MASK>
     __device__ inline void commit_one(int idx, T* tile) const {
         const int i = idx / 8, rr = idx % 8;
-        const uint32_t mb = threadIdx.x + kThreads * i;
+        const uint32_t mb = threadIdx.x + THREADS * i;
         const uint32_t kb = mb % 8, rb = mb / 8;
         if (rb >= ROWS / 8) return;
         // row rr of the transposed micro-block: element rr of each of the 8 loaded vectors
@@ -149,20 +159,28 @@ struct RowMajorLoader {
         for (int kk = 0; kk < 8; ++kk) {
             uint16_t in[8];
             __builtin_memcpy(in, &regs[i][kk], 16);
-            out[kk] = static_cast<uint32_t>(kk) < k_count ? in[rr] : uint16_t(0);
+            out[kk] = (!MASK || static_cast<uint32_t>(kk) < k_count) ? in[rr] : uint16_t(0);
         }
         uint4v v;
         __builtin_memcpy(&v, out, 16);
         *reinterpret_cast<uint4v*>(tile + tile_offset(rb * 8 + rr, kb)) = v;
     }
+    // A micro-block is transposed out of all eight of its registers: the eight writes of a pass, then its
+    // eight refills.
+    static constexpr int OPS = STORES + LOADS;
+    static constexpr bool is_commit(int o) { return o % 16 < 8; }
+    static constexpr int index_of(int o) { return (o / 16) * 8 + o % 8; }
 };
 
-template <class T, int ROWS, bool K_MAJOR>
-using Loader = std::conditional_t<K_MAJOR, KMajorLoader<T, ROWS>, RowMajorLoader<T, ROWS>>;
+template <class T, int ROWS, int THREADS, bool K_MAJOR>
+using Loader = std::conditional_t<K_MAJOR, KMajorLoader<T, ROWS, THREADS>, RowMajorLoader<T, ROWS, THREADS>>;
 
-template <class T, int BM, int BN, bool A_KMAJOR, bool B_KMAJOR>
-__global__ __launch_bounds__(kThreads) void gemm16_kernel(const T* A, const T* B, T* C, GemmProblem p, uint32_t tiles_m, uint32_t tiles_n) {
-    constexpr int WM = BM / 2, WN = BN / 2;   // 2 x 2 wavefronts
+// WAVES_N: wavefronts along N (2 -> 256 threads, one wavefront per SIMD; 4 -> 512 threads, two per SIMD, so that
+// one wavefront's waits are covered by the other's MFMAs); always two wavefronts along M.
+template <class T, int BM, int BN, int WAVES_N, bool A_KMAJOR, bool B_KMAJOR>
+__global__ __launch_bounds__(128 * WAVES_N) void gemm16_kernel(const T* A, const T* B, T* C, GemmProblem p, uint32_t tiles_m, uint32_t tiles_n) {
+    constexpr int THREADS = 128 * WAVES_N;
+    constexpr int WM = BM / 2, WN = BN / WAVES_N;
     constexpr int TM = WM / 32, TN = WN / 32;
     extern __shared__ __align__(16) unsigned char lds_raw[];
     // layout: A buffer 0, A buffer 1, B buffer 0, B buffer 1 (offsets in elements)
@@ -178,7 +196,7 @@ __global__ __launch_bounds__(kThreads) void gemm16_kernel(const T* A, const T* B
     const uint32_t m0 = tm * BM, n0 = tn * BN;
 
     const int wave = threadIdx.x / 64, lane = threadIdx.x % 64;
-    const int wm = (wave / 2) * WM, wn = (wave % 2) * WN;
+    const int wm = (wave / WAVES_N) * WM, wn = (wave % WAVES_N) * WN;
     const uint32_t frag_row = lane % 32, frag_chunk = lane / 32;
 
     float16v acc[TM][TN];
@@ -189,10 +207,10 @@ __global__ __launch_bounds__(kThreads) void gemm16_kernel(const T* A, const T* B
 #pragma unroll
             for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
 
-    Loader<T, BM, A_KMAJOR> la;
-    Loader<T, BN, B_KMAJOR> lb;
-    using LA = Loader<T, BM, A_KMAJOR>;
-    using LB = Loader<T, BN, B_KMAJOR>;
+    using LA = Loader<T, BM, THREADS, A_KMAJOR>;
+    using LB = Loader<T, BN, THREADS, B_KMAJOR>;
+    LA la;
+    LB lb;
     const uint32_t steps = (p.K + kBK - 1) / kBK;
 
     // prologue: tile 0 into LDS buffer 0, tile 1 into registers
@@ -203,9 +221,9 @@ __global__ __launch_bounds__(kThreads) void gemm16_kernel(const T* A, const T* B
 #pragma unroll
     for (int i = 0; i < LB::LOADS; ++i) lb.fetch_one(i, opB, n0);
 #pragma unroll
-    for (int i = 0; i < LA::STORES; ++i) la.commit_one(i, lds);
+    for (int i = 0; i < LA::STORES; ++i) la.template commit_one<true>(i, lds);
 #pragma unroll
-    for (int i = 0; i < LB::STORES; ++i) lb.commit_one(i, lds + B_BASE);
+    for (int i = 0; i < LB::STORES; ++i) lb.template commit_one<true>(i, lds + B_BASE);
     if (steps > 1) {
         la.begin_fetch(opA, kBK, p.K);
         lb.begin_fetch(opB, kBK, p.K);
@@ -216,17 +234,32 @@ __global__ __launch_bounds__(kThreads) void gemm16_kernel(const T* A, const T* B
     }
     __syncthreads();
 
-    // One K step.  The registers hold tile s+1 on entry.  The 4*TM*TN MFMAs of
-    // the step are issued in order; between them, one memory operation at a time:
-    // first the LDS writes of tile s+1 (into the buffer the previous step read),
-    // then the global loads of tile s+2 (into the registers just written out).
-    // sched_barrier pins that interleaving so that neither the load unit nor the
-    // LDS ever sees a burst while the matrix pipe idles.
-    auto step = [&](uint32_t s, auto commit_tag, auto fetch_tag) {
-        constexpr bool COMMIT = decltype(commit_tag)::value, FETCH = decltype(fetch_tag)::value;
-        constexpr int KS = kBK / 16, PER_KS = TM * TN, MFMAS = KS * PER_KS;
-        constexpr int NCA = LA::STORES, NCB = LB::STORES, NFA = LA::LOADS, NFB = LB::LOADS;
-        constexpr int OPS = NCA + NCB + NFA + NFB;
+    // One K step, rotated by one k-slice: the step for tile s issues the MFMAs of the LAST 16-wide k-slice of
+    // tile s-1 (its fragments are in registers already) and those of the first three slices of tile s.  The
+    // barrier thus sits where every wavefront still has 16 MFMAs to issue whose operands need no LDS, so the
+    // LDS latency of the first fragment reads of the new tile is covered.  The barrier at the end of step s-1
+    // tells that (a) all of tile s is in LDS and (b) nobody reads tile s-1 any more, so its buffer takes tile s+1.
+    // The registers hold tile s+1 on entry.  Between the MFMAs, one memory operation at a time: register i
+    // goes to LDS (tile s+1) and is refilled from global memory (tile s+2).  sched_barrier pins that
+    // interleaving so that neither the load unit nor the LDS ever sees a burst while the matrix pipe idles.
+    constexpr int KS = kBK / 16, PER_KS = TM * TN;
+    uint4v fa[2][TM], fb[2][TN];
+    auto read_fragments = [&](const T* a_tile, const T* b_tile, int ks, int into) {
+#pragma unroll
+        for (int x = 0; x < TM; ++x) fa[into][x] = *reinterpret_cast<const uint4v*>(a_tile + tile_offset(wm + x * 32 + frag_row, ks * 2 + frag_chunk));
+#pragma unroll
+        for (int y = 0; y < TN; ++y) fb[into][y] = *reinterpret_cast<const uint4v*>(b_tile + tile_offset(wn + y * 32 + frag_row, ks * 2 + frag_chunk));
+    };
+    // (for tile 0 the "previous tile's" fragments are zeros: 16 MFMAs that add nothing keep the loop free of a
+    // peeled first iteration, whose extra copy of the code costs more than it saves)
+#pragma unroll
+    for (int x = 0; x < TM; ++x) fa[(KS - 1) & 1][x] = uint4v{0, 0, 0, 0};
+#pragma unroll
+    for (int y = 0; y < TN; ++y) fb[(KS - 1) & 1][y] = uint4v{0, 0, 0, 0};
+    auto step = [&](uint32_t s, auto commit_tag, auto fetch_tag, auto mask_tag) {
+        constexpr bool COMMIT = decltype(commit_tag)::value, FETCH = decltype(fetch_tag)::value, MASK = decltype(mask_tag)::value;
+        constexpr int MFMAS = KS * PER_KS;
+        constexpr int OPS = LA::OPS + LB::OPS;
         const uint32_t cur = s & 1;
         const T* a_tile = lds + cur * A_TILE;
         const T* b_tile = lds + B_BASE + cur * B_TILE;
@@ -236,25 +269,17 @@ __global__ __launch_bounds__(kThreads) void gemm16_kernel(const T* A, const T* B
             la.begin_fetch(opA, (s + 2) * kBK, p.K);
             lb.begin_fetch(opB, (s + 2) * kBK, p.K);
         }
-        uint4v fa[2][TM], fb[2][TN];
-#pragma unroll
-        for (int i = 0; i < TM; ++i) fa[0][i] = *reinterpret_cast<const uint4v*>(a_tile + tile_offset(wm + i * 32 + frag_row, frag_chunk));
-#pragma unroll
-        for (int j = 0; j < TN; ++j) fb[0][j] = *reinterpret_cast<const uint4v*>(b_tile + tile_offset(wn + j * 32 + frag_row, frag_chunk));
+        read_fragments(a_tile, b_tile, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
         static_for<MFMAS>([&](auto m_tag) {
             constexpr int m = decltype(m_tag)::value;
-            constexpr int ks = m / PER_KS, i = (m % PER_KS) / TN, j = m % TN;
-            constexpr int now = ks & 1, nxt = now ^ 1;
-            if constexpr (m % PER_KS == 0) {
-                if constexpr (ks + 1 < KS) {
-                    // fragments of k-slice ks+1 are requested before the MFMAs of slice ks
-#pragma unroll
-                    for (int x = 0; x < TM; ++x)
-                        fa[nxt][x] = *reinterpret_cast<const uint4v*>(a_tile + tile_offset(wm + x * 32 + frag_row, (ks + 1) * 2 + frag_chunk));
-#pragma unroll
-                    for (int y = 0; y < TN; ++y)
-                        fb[nxt][y] = *reinterpret_cast<const uint4v*>(b_tile + tile_offset(wn + y * 32 + frag_row, (ks + 1) * 2 + frag_chunk));
-                }
+            constexpr int slot = m;
+            constexpr int group = slot / PER_KS;           // 0: slice 3 of the previous tile; g > 0: slice g-1 of this tile
+            constexpr int i = (slot % PER_KS) / TN, j = slot % TN;
+            constexpr int now = group == 0 ? (KS - 1) & 1 : (group - 1) & 1;
+            if constexpr (slot % PER_KS == 0 && group > 0) {
+                // fragments of slice `group` are requested before the MFMAs of slice group-1
+                read_fragments(a_tile, b_tile, group, group & 1);
                 __builtin_amdgcn_sched_barrier(0);
             }
             acc[i][j] = Mfma16<T>::run(fa[now][i], fb[now][j], acc[i][j]);
@@ -262,21 +287,32 @@ __global__ __launch_bounds__(kThreads) void gemm16_kernel(const T* A, const T* B
             constexpr int first = m * OPS / MFMAS, last = (m + 1) * OPS / MFMAS;
             static_for<last - first>([&](auto o_tag) {
                 constexpr int o = first + decltype(o_tag)::value;
-                if constexpr (o < NCA) { if constexpr (COMMIT) la.commit_one(o, a_next); }
-                else if constexpr (o < NCA + NCB) { if constexpr (COMMIT) lb.commit_one(o - NCA, b_next); }
-                else if constexpr (o < NCA + NCB + NFA) { if constexpr (FETCH) la.fetch_one(o - NCA - NCB, opA, m0); }
-                else { if constexpr (FETCH) lb.fetch_one(o - NCA - NCB - NFA, opB, n0); }
+                if constexpr (o < LA::OPS) {
+                    if constexpr (LA::is_commit(o)) { if constexpr (COMMIT) la.template commit_one<MASK>(LA::index_of(o), a_next); }
+                    else { if constexpr (FETCH) la.fetch_one(LA::index_of(o), opA, m0); }
+                } else {
+                    constexpr int ob = o - LA::OPS;
+                    if constexpr (LB::is_commit(ob)) { if constexpr (COMMIT) lb.template commit_one<MASK>(LB::index_of(ob), b_next); }
+                    else { if constexpr (FETCH) lb.fetch_one(LB::index_of(ob), opB, n0); }
+                }
             });
             __builtin_amdgcn_sched_barrier(0);
         });
         __syncthreads();
     };
+    static_assert(KS == 4, "the rotation below assumes four k-slices per tile");
     using Yes = std::true_type;
     using No = std::false_type;
+    // only the last tile can reach past K: the tiles the main loop writes to LDS need no mask
     uint32_t s = 0;
-    for (; s + 2 < steps; ++s) step(s, Yes{}, Yes{});
-    if (s + 1 < steps) { step(s, Yes{}, No{}); ++s; }
-    step(s, No{}, No{});
+    for (; s + 2 < steps; ++s) step(s, Yes{}, Yes{}, No{});
+    if (s + 1 < steps) { step(s, Yes{}, No{}, Yes{}); ++s; }
+    step(s, No{}, No{}, No{});
+    // the last slice of the last tile
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j) acc[i][j] = Mfma16<T>::run(fa[(KS - 1) & 1][i], fb[(KS - 1) & 1][j], acc[i][j]);
 
     // accumulator layout of a 32x32 tile: lane -> column lane % 32; value v ->
     // row 8 * (v / 4) + 4 * (lane / 32) + v % 4
@@ -294,27 +330,27 @@ __global__ __launch_bounds__(kThreads) void gemm16_kernel(const T* A, const T* B
         }
 }
 
-template <class T, int BM, int BN, bool AK, bool BK_>
+template <class T, int BM, int BN, int WAVES_N, bool AK, bool BK_>
 int launch16(const GemmProblem& p, const void* a, const void* b, void* c, hipStream_t stream) {
     const uint32_t tiles_m = (p.M + BM - 1) / BM, tiles_n = (p.N + BN - 1) / BN;
     constexpr size_t lds_bytes = sizeof(T) * 2 * (BM + BN) * kBK;
-    auto kernel = gemm16_kernel<T, BM, BN, AK, BK_>;
+    auto kernel = gemm16_kernel<T, BM, BN, WAVES_N, AK, BK_>;
     static bool configured = false;
     if (!configured) {
         TH_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes)));
         configured = true;
     }
-    hipLaunchKernelGGL(kernel, dim3(tiles_m * tiles_n, p.batches), dim3(kThreads), lds_bytes, stream, static_cast<const T*>(a),
+    hipLaunchKernelGGL(kernel, dim3(tiles_m * tiles_n, p.batches), dim3(128 * WAVES_N), lds_bytes, stream, static_cast<const T*>(a),
                        static_cast<const T*>(b), static_cast<T*>(c), p, tiles_m, tiles_n);
     return launch_status("gemm16_kernel");
 }
 
-template <class T, int BM, int BN>
+template <class T, int BM, int BN, int WAVES_N>
 int pick_layout16(const GemmProblem& p, bool ak, bool bk, const void* a, const void* b, void* c, hipStream_t s) {
-    if (ak && bk) return launch16<T, BM, BN, true, true>(p, a, b, c, s);
-    if (ak) return launch16<T, BM, BN, true, false>(p, a, b, c, s);
-    if (bk) return launch16<T, BM, BN, false, true>(p, a, b, c, s);
-    return launch16<T, BM, BN, false, false>(p, a, b, c, s);
+    if (ak && bk) return launch16<T, BM, BN, WAVES_N, true, true>(p, a, b, c, s);
+    if (ak) return launch16<T, BM, BN, WAVES_N, true, false>(p, a, b, c, s);
+    if (bk) return launch16<T, BM, BN, WAVES_N, false, true>(p, a, b, c, s);
+    return launch16<T, BM, BN, WAVES_N, false, false>(p, a, b, c, s);
 }
 
 template <class T>
@@ -335,10 +371,10 @@ int run16(const GemmProblem& p, const void* a, const void* b, void* c, hipStream
     if (p.batches > 65535) return TANNIC_UNSUPPORTED_DTYPE;
     // large tiles when they still give every CU work, smaller ones otherwise
     const uint64_t big = static_cast<uint64_t>((p.M + 255) / 256) * ((p.N + 255) / 256) * p.batches;
-    if (big >= 200) return pick_layout16<T, 256, 256>(p, ak, bk, a, b, c, stream);
+    if (big >= 200) return pick_layout16<T, 256, 256, 2>(p, ak, bk, a, b, c, stream);
     const uint64_t mid = static_cast<uint64_t>((p.M + 127) / 128) * ((p.N + 127) / 128) * p.batches;
-    if (mid >= 128 || p.M > 64) return pick_layout16<T, 128, 128>(p, ak, bk, a, b, c, stream);
-    return pick_layout16<T, 64, 128>(p, ak, bk, a, b, c, stream);
+    if (mid >= 128 || p.M > 64) return pick_layout16<T, 128, 128, 2>(p, ak, bk, a, b, c, stream);
+    return pick_layout16<T, 64, 128, 2>(p, ak, bk, a, b, c, stream);
 }
 
 int gemm_mfma_16bit(const GemmProblem& p, int dtype, const void* a, const void* b, void* c, hipStream_t stream) {
