@@ -282,7 +282,7 @@ __global__ __launch_bounds__(128 * WAVES_N) void gemm16_kernel(const T* A, const
                 read_fragments(a_tile, b_tile, group, group & 1);
                 __builtin_amdgcn_sched_barrier(0);
             }
-            acc[i][j] = Mfma16<T>::run(fa[now][i], fb[now][j], acc[i][j]);
+            acc[i][j] = Mfma16<T>::run(fb[now][j], fa[now][i], acc[i][j]);
             // memory operations [first, last) of the step go right after this MFMA
             constexpr int first = m * OPS / MFMAS, last = (m + 1) * OPS / MFMAS;
             static_for<last - first>([&](auto o_tag) {
@@ -312,28 +312,62 @@ __global__ __launch_bounds__(128 * WAVES_N) void gemm16_kernel(const T* A, const
 #pragma unroll
     for (int i = 0; i < TM; ++i)
 #pragma unroll
-        for (int j = 0; j < TN; ++j) acc[i][j] = Mfma16<T>::run(fa[(KS - 1) & 1][i], fb[(KS - 1) & 1][j], acc[i][j]);
+        for (int j = 0; j < TN; ++j) acc[i][j] = Mfma16<T>::run(fb[(KS - 1) & 1][j], fa[(KS - 1) & 1][i], acc[i][j]);
 
-    // accumulator layout of a 32x32 tile: lane -> column lane % 32; value v ->
-    // row 8 * (v / 4) + 4 * (lane / 32) + v % 4
+    // The B fragment is the MFMA's first operand, so a 32x32 accumulator holds C transposed: lane -> row
+    // lane % 32 of C; value v -> column 8 * (v / 4) + 4 * (lane / 32) + v % 4, i.e. runs of four consecutive
+    // columns.  Each wavefront rounds its WM x WN block into its own LDS area (nobody reads operand tiles any
+    // more after the last barrier) and writes it out as whole rows: 16 bytes per lane, WN / 8 lanes per row, so
+    // that the memory system sees full lines instead of fragments.
     T* c = C + oc;
+    const bool vector_ok = p.c_rs % 8 == 0 && p.N % 8 == 0 && reinterpret_cast<uintptr_t>(c) % 16 == 0;
+    if (vector_ok) {
+        constexpr int PITCH = WN + 8;                       // elements: rows stay 16-byte aligned and shift by four banks
+        T* stage = lds + wave * (WM * PITCH);
 #pragma unroll
-    for (int i = 0; i < TM; ++i)
+        for (int i = 0; i < TM; ++i)
 #pragma unroll
-        for (int j = 0; j < TN; ++j) {
-            const uint32_t col = n0 + wn + j * 32 + lane % 32;
+            for (int j = 0; j < TN; ++j)
 #pragma unroll
-            for (int v = 0; v < 16; ++v) {
-                const uint32_t row = m0 + wm + i * 32 + 8 * (v / 4) + 4 * (lane / 32) + v % 4;
-                if (row < p.M && col < p.N) c[static_cast<int64_t>(row) * p.c_rs + col] = narrow<T>(acc[i][j][v]);
-            }
+                for (int g = 0; g < 4; ++g) {
+                    T out[4];
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) out[e] = narrow<T>(acc[i][j][g * 4 + e]);
+                    uint2 bits;
+                    __builtin_memcpy(&bits, out, 8);
+                    *reinterpret_cast<uint2*>(stage + (i * 32 + lane % 32) * PITCH + j * 32 + g * 8 + 4 * (lane / 32)) = bits;
+                }
+        // same wavefront reads what it wrote: LDS operations of a wavefront complete in order
+        constexpr int LANES_PER_ROW = WN / 8, ROWS_PER_PASS = 64 / LANES_PER_ROW;
+        const uint32_t col = n0 + wn + (lane % LANES_PER_ROW) * 8;
+#pragma unroll
+        for (int r0 = 0; r0 < WM; r0 += ROWS_PER_PASS) {
+            const uint32_t r = r0 + lane / LANES_PER_ROW, row = m0 + wm + r;
+            const uint4v bits = *reinterpret_cast<const uint4v*>(stage + r * PITCH + (lane % LANES_PER_ROW) * 8);
+            if (row < p.M && col < p.N) *reinterpret_cast<uint4v*>(c + static_cast<int64_t>(row) * p.c_rs + col) = bits;
         }
+    } else {
+#pragma unroll
+        for (int i = 0; i < TM; ++i) {
+            const uint32_t row = m0 + wm + i * 32 + lane % 32;
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+#pragma unroll
+                for (int v = 0; v < 16; ++v) {
+                    const uint32_t col = n0 + wn + j * 32 + 8 * (v / 4) + 4 * (lane / 32) + v % 4;
+                    if (row < p.M && col < p.N) c[static_cast<int64_t>(row) * p.c_rs + col] = narrow<T>(acc[i][j][v]);
+                }
+        }
+    }
 }
 
 template <class T, int BM, int BN, int WAVES_N, bool AK, bool BK_>
 int launch16(const GemmProblem& p, const void* a, const void* b, void* c, hipStream_t stream) {
     const uint32_t tiles_m = (p.M + BM - 1) / BM, tiles_n = (p.N + BN - 1) / BN;
-    constexpr size_t lds_bytes = sizeof(T) * 2 * (BM + BN) * kBK;
+    // operand tiles (two buffers each); the same memory later stages the output, BM*BN elements in padded rows
+    constexpr size_t tile_bytes = sizeof(T) * 2 * (BM + BN) * kBK;
+    constexpr size_t stage_bytes = sizeof(T) * 2 * WAVES_N * (BM / 2) * (BN / WAVES_N + 8);
+    constexpr size_t lds_bytes = tile_bytes > stage_bytes ? tile_bytes : stage_bytes;
     auto kernel = gemm16_kernel<T, BM, BN, WAVES_N, AK, BK_>;
     static bool configured = false;
     if (!configured) {
