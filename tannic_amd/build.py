@@ -41,6 +41,8 @@ UNITS = [
     ("conv2d_mfma.hip", "conv2d_mfma.o", []),
     ("conv2d_patch.hip", "conv2d_patch.o", []),
     ("conv2d_resident.hip", "conv2d_resident.o", []),
+    ("conv2d_k3.hip", "conv2d_k3.o", []),
+    ("conv2d_pointwise.hip", "conv2d_pointwise.o", []),
 ]
 
 

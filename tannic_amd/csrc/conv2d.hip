@@ -93,6 +93,10 @@ static int conv2d_entry(const tannic_tensor_t* x, const tannic_tensor_t* w, cons
     // the gathering implicit GEMM serves it better than the LDS-patch kernels.
     int status = TANNIC_UNSUPPORTED_DTYPE;
     const bool pointwise = p.KH == 1 && p.KW == 1;
+    if (pointwise) status = conv2d_pointwise(p, x->dtype, x->address, w->address, pb, y->address, s);
+    if (status != TANNIC_UNSUPPORTED_DTYPE) return status;
+    if (!pointwise) status = conv2d_k3(p, x->dtype, x->address, w->address, pb, y->address, s);
+    if (status != TANNIC_UNSUPPORTED_DTYPE) return status;
     if (!pointwise) status = conv2d_resident(p, x->dtype, x->address, w->address, pb, y->address, s);
     if (status != TANNIC_UNSUPPORTED_DTYPE) return status;
     if (!pointwise) status = conv2d_patch(p, x->dtype, x->address, w->address, pb, y->address, s);

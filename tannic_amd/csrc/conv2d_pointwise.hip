@@ -1,0 +1,97 @@
+// conv2d with a 1x1 kernel, 16-bit signals: a matrix product per image.
+//
+// y[n] (O x HO*WO) = w (O x C) * x[n] (C x HO*WO): the kernel tensor is the
+// K-contiguous operand, an NCHW image is the row-major one (pixels contiguous for
+// each channel) and NCHW output is the plain row-major result, so the batched
+// MFMA matrix-multiply kernel runs it as it stands, with the bias as its per-row
+// start value.  With a stride the pixels the product needs are first gathered
+// into a dense [N][C][HO*WO] copy (the only extra traffic: one write and one
+// read of a quarter of the image for stride 2).
+#include "conv_common.hpp"
+#include "gemm_common.hpp"
+
+namespace th {
+
+// out[row][ow] = x[n][c][oh * stride_h][ow * stride_w], row = (n * C + c) * HO + oh; four outputs per thread
+template <class T>
+__global__ __launch_bounds__(256) void conv_subsample4_kernel(const T* x, T* out, ConvProblem p, FastDiv div_quads, FastDiv div_ho, FastDiv div_c, uint32_t total) {
+    const uint32_t idx = blockIdx.x * 256 + threadIdx.x;
+    if (idx >= total) return;
+    uint32_t row, quad, nc, oh, n, c;
+    div_quads.divmod(idx, row, quad);
+    div_ho.divmod(row, nc, oh);
+    div_c.divmod(nc, n, c);
+    const T* src = x + static_cast<int64_t>(n) * p.xs[0] + static_cast<int64_t>(c) * p.xs[1] + static_cast<int64_t>(oh * p.stride_h) * p.xs[2] +
+                   static_cast<int64_t>(quad * 4 * p.stride_w) * p.xs[3];
+    T v[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) v[e] = src[static_cast<int64_t>(e * p.stride_w) * p.xs[3]];
+    uint2 bits;
+    __builtin_memcpy(&bits, v, 8);
+    *reinterpret_cast<uint2*>(out + static_cast<int64_t>(row) * p.WO + quad * 4) = bits;
+}
+
+template <class T>
+int run_pointwise(const ConvProblem& p, int dtype, const void* x, const void* w, const void* bias, void* y, hipStream_t stream) {
+    if (p.KH != 1 || p.KW != 1 || p.pad_h != 0 || p.pad_w != 0) return TANNIC_UNSUPPORTED_DTYPE;
+    if (p.N == 0 || p.O == 0 || p.HO == 0 || p.WO == 0) return TANNIC_SUCCESS;
+    if (p.C == 0) return TANNIC_UNSUPPORTED_DTYPE;
+    // the kernel tensor as a K-contiguous O x C matrix; the result as row-major O x (HO*WO) per image
+    if (p.ws[1] != 1) return TANNIC_UNSUPPORTED_DTYPE;
+    if (p.ys[3] != 1 || p.ys[2] != static_cast<int64_t>(p.WO)) return TANNIC_UNSUPPORTED_DTYPE;
+    const uint64_t pixels = static_cast<uint64_t>(p.HO) * p.WO;
+    if (pixels >= (1ull << 31) || p.N > 65535) return TANNIC_UNSUPPORTED_DTYPE;
+    GemmProblem g{};
+    g.M = p.O;
+    g.N = static_cast<uint32_t>(pixels);
+    g.K = p.C;
+    g.a_rs = p.ws[0];
+    g.a_cs = 1;
+    g.b_cs = 1;
+    g.c_rs = p.ys[1];
+    g.batch_rank = 1;
+    g.batches = p.N;
+    for (int d = 0; d < 6; ++d) {
+        g.batch_extent[d] = 1;
+        g.a_bs[d] = g.b_bs[d] = g.c_bs[d] = 0;
+    }
+    g.batch_extent[0] = p.N;
+    g.c_bs[0] = p.ys[0];
+    g.row_bias = bias;
+    const bool dense = p.stride_h == 1 && p.stride_w == 1;
+    if (dense) {
+        if (p.xs[3] != 1 || p.xs[2] != static_cast<int64_t>(p.W)) return TANNIC_UNSUPPORTED_DTYPE;
+        g.b_rs = p.xs[1];
+        g.b_bs[0] = p.xs[0];
+        return gemm_mfma_16bit(g, dtype, w, x, y, stream);
+    }
+    // strided: gather first.  The product's own conditions are checked before any work is queued.
+    if (p.WO % 4 != 0 || pixels % 8 != 0 || p.ws[0] % 8 != 0 || p.C % 8 != 0 || reinterpret_cast<uintptr_t>(w) % 16 != 0) return TANNIC_UNSUPPORTED_DTYPE;
+    const uint64_t rows = static_cast<uint64_t>(p.N) * p.C * p.HO, quads = rows * (p.WO / 4);
+    if (quads >= (1ull << 31)) return TANNIC_UNSUPPORTED_DTYPE;
+    T* dense_x = nullptr;
+    if (scratch_acquire(reinterpret_cast<void**>(&dense_x), rows * p.WO * sizeof(T), stream) != TANNIC_SUCCESS) return TANNIC_ERROR;
+    hipLaunchKernelGGL((conv_subsample4_kernel<T>), dim3((quads + 255) / 256), dim3(256), 0, stream, static_cast<const T*>(x), dense_x, p, FastDiv(p.WO / 4),
+                       FastDiv(p.HO), FastDiv(p.C), static_cast<uint32_t>(quads));
+    int status = launch_status("conv_subsample4_kernel");
+    if (status == TANNIC_SUCCESS) {
+        g.b_rs = static_cast<int64_t>(pixels);
+        g.b_bs[0] = static_cast<int64_t>(p.C) * static_cast<int64_t>(pixels);
+        status = gemm_mfma_16bit(g, dtype, w, dense_x, y, stream);
+        // the conditions above are the product's: a refusal here would leave the result unwritten
+        if (status == TANNIC_UNSUPPORTED_DTYPE) {
+            set_error_text("conv2d: internal: the 1x1 product refused a problem its caller had checked");
+            status = TANNIC_ERROR;
+        }
+    }
+    scratch_release(dense_x, stream);
+    return status;
+}
+
+int conv2d_pointwise(const ConvProblem& p, int dtype, const void* x, const void* w, const void* bias, void* y, hipStream_t stream) {
+    if (dtype == TANNIC_FLOAT16) return run_pointwise<f16>(p, dtype, x, w, bias, y, stream);
+    if (dtype == TANNIC_BFLOAT16) return run_pointwise<bf16>(p, dtype, x, w, bias, y, stream);
+    return TANNIC_UNSUPPORTED_DTYPE;
+}
+
+}  // namespace th

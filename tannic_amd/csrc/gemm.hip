@@ -43,6 +43,7 @@ int describe_gemm(const tannic_tensor_t* a, const tannic_tensor_t* b, const tann
     p.b_rs = bt ? 1 : ldb;
     p.b_cs = bt ? ldb : 1;
     p.c_rs = c->strides.sizes[c->rank - 2];
+    p.row_bias = nullptr;
     p.batch_rank = c->rank - 2;
     p.batches = 1;
     for (int d = 0; d < 6; ++d) {

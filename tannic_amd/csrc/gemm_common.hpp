@@ -19,6 +19,8 @@ struct GemmProblem {
     uint32_t batches;
     uint32_t batch_extent[6];
     int64_t a_bs[6], b_bs[6], c_bs[6];
+    // optional (MFMA 16-bit kernels only): one value of C's type per row of C, added before rounding
+    const void* row_bias;
 };
 
 __host__ __device__ inline void batch_offsets(const GemmProblem& p, uint32_t batch, int64_t& oa, int64_t& ob, int64_t& oc) {

@@ -199,13 +199,17 @@ __global__ __launch_bounds__(128 * WAVES_N) void gemm16_kernel(const T* A, const
     const int wm = (wave / WAVES_N) * WM, wn = (wave % WAVES_N) * WN;
     const uint32_t frag_row = lane % 32, frag_chunk = lane / 32;
 
+    // an accumulator holds C transposed: the lane's row of C is lane % 32, so a per-row bias is one value per lane
     float16v acc[TM][TN];
 #pragma unroll
-    for (int i = 0; i < TM; ++i)
+    for (int i = 0; i < TM; ++i) {
+        const uint32_t row = tm * BM + (wave / WAVES_N) * WM + i * 32 + lane % 32;
+        const float start = (p.row_bias && row < p.M) ? static_cast<float>(widen(static_cast<const T*>(p.row_bias)[row])) : 0.0f;
 #pragma unroll
         for (int j = 0; j < TN; ++j)
 #pragma unroll
-            for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
+            for (int v = 0; v < 16; ++v) acc[i][j][v] = start;
+    }
 
     using LA = Loader<T, BM, THREADS, A_KMAJOR>;
     using LB = Loader<T, BN, THREADS, B_KMAJOR>;

@@ -33,6 +33,11 @@ CASES = {
     "patch_k5_s2_p2": ((1, 32, 24, 16), (40, 32, 5, 5), (2, 2), (2, 2)),
     "patch_many_out_channels": ((1, 96, 8, 24), (200, 96, 3, 3), (1, 1), (1, 1)),
     "patch_rect_stride": ((2, 32, 9, 16), (8, 32, 2, 3), (1, 2), (1, 0)),
+    # 3x3 kernels over 32-channel chunks: stride 2, no padding with four chunks, a tall tile, rectangular stride
+    "k3_s2_p1": ((2, 64, 16, 16), (64, 64, 3, 3), (2, 2), (1, 1)),
+    "k3_p0_128ch": ((1, 128, 10, 16), (32, 128, 3, 3), (1, 1), (0, 0)),
+    "k3_tall_tile": ((1, 32, 40, 16), (70, 32, 3, 3), (1, 1), (1, 1)),
+    "k3_rect_stride_pad": ((1, 96, 13, 24), (64, 96, 3, 3), (2, 1), (0, 2)),
 }
 
 
