@@ -95,6 +95,8 @@ static int conv2d_entry(const tannic_tensor_t* x, const tannic_tensor_t* w, cons
     const bool pointwise = p.KH == 1 && p.KW == 1;
     if (pointwise) status = conv2d_pointwise(p, x->dtype, x->address, w->address, pb, y->address, s);
     if (status != TANNIC_UNSUPPORTED_DTYPE) return status;
+    if (!pointwise) status = conv2d_stem(p, x->dtype, x->address, w->address, pb, y->address, s);
+    if (status != TANNIC_UNSUPPORTED_DTYPE) return status;
     if (!pointwise) status = conv2d_k3(p, x->dtype, x->address, w->address, pb, y->address, s);
     if (status != TANNIC_UNSUPPORTED_DTYPE) return status;
     if (!pointwise) status = conv2d_resident(p, x->dtype, x->address, w->address, pb, y->address, s);

@@ -37,6 +37,13 @@ CASES = {
     "k3_s2_p1": ((2, 64, 16, 16), (64, 64, 3, 3), (2, 2), (1, 1)),
     "k3_p0_128ch": ((1, 128, 10, 16), (32, 128, 3, 3), (1, 1), (0, 0)),
     "k3_tall_tile": ((1, 32, 40, 16), (70, 32, 3, 3), (1, 1), (1, 1)),
+    # few channels: rows of 8 consecutive columns as contraction slots (even horizontal stride), and shapes next to those
+    "stem_c1_k5": ((2, 1, 20, 19), (10, 1, 5, 5), (1, 1), (2, 2)),
+    "stem_c3_k3_two_tiles": ((1, 3, 12, 16), (70, 3, 3, 3), (1, 1), (1, 1)),
+    "stem_c1_k5_s2": ((2, 1, 20, 24), (10, 1, 5, 5), (2, 2), (2, 2)),
+    "stem_c3_k3_s1x2_p1": ((1, 3, 12, 16), (70, 3, 3, 3), (1, 2), (1, 1)),
+    "stem_c4_k5x8_s3x2": ((1, 4, 17, 32), (8, 4, 5, 8), (3, 2), (0, 4)),
+    "stem_c2_k7_s2_tall": ((1, 2, 64, 16), (5, 2, 7, 7), (2, 2), (3, 3)),
     "k3_rect_stride_pad": ((1, 96, 13, 24), (64, 96, 3, 3), (2, 1), (0, 2)),
 }
 
