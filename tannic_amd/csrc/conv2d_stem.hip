@@ -94,30 +94,47 @@ __global__ __launch_bounds__(kStemThreads, 2) void conv2d_stem_kernel(const T* x
         }
         __syncthreads();
     }
-    uint4s afrag[NS][2];
+    // Every (slot, channel) pair becomes one 16-byte record [slot][64 channels]: five aligned words around the slot's
+    // KW weights, moved by half a word when they start at an odd element, cleared outside the kernel row.
+    T* records = ring + ((kStemBCO * taps + 7) / 8) * 8;
     {
-        const T* raw = ring;
-        const int32_t last = static_cast<int32_t>(wrows * taps) - 1;
+        const uint32_t* raw32 = reinterpret_cast<const uint32_t*>(ring);
+        const int32_t last_word = static_cast<int32_t>((wrows * taps + 1) / 2) - 1;
+        uint32_t keep[4];
 #pragma unroll
-        for (int s = 0; s < NS; ++s)
+        for (int j = 0; j < 4; ++j) {
+            const uint32_t lo = (2u * j >= q.delta && 2u * j - q.delta < p.KW) ? 0xFFFFu : 0u;
+            const uint32_t hi = (2u * j + 1 >= q.delta && 2u * j + 1 - q.delta < p.KW) ? 0xFFFF0000u : 0u;
+            keep[j] = lo | hi;
+        }
+        for (uint32_t u = threadIdx.x; u < 2 * NS * kStemBCO; u += kStemThreads) {
+            const uint32_t cl = u % kStemBCO, slot = u / kStemBCO;
+            const bool real = cl < wrows && slot < q.slots;
+            const int32_t first = static_cast<int32_t>(cl * taps + slot * p.KW) - static_cast<int32_t>(q.delta);   // >= -1
+            const int32_t w0 = (first + 2) / 2 - 1;   // floor(first / 2)
+            const bool odd = (first & 1) != 0;
+            uint32_t word[5];
 #pragma unroll
-            for (int i = 0; i < 2; ++i) {
-                const uint32_t cl = i * 32 + lane % 32, slot = 2 * s + lane / 32;
-                const bool real = cl < wrows && slot < q.slots;
-                const int32_t first = static_cast<int32_t>(cl * taps + slot * p.KW) - static_cast<int32_t>(q.delta);
-                uint16_t e[8];
-#pragma unroll
-                for (int k = 0; k < 8; ++k) {
-                    int32_t at = first + k;
-                    at = at < 0 ? 0 : (at > last ? last : at);
-                    uint16_t v;
-                    __builtin_memcpy(&v, raw + (real ? at : 0), 2);
-                    const bool inside = real && static_cast<uint32_t>(k) >= q.delta && static_cast<uint32_t>(k) - q.delta < p.KW;
-                    e[k] = inside ? v : uint16_t(0);
-                }
-                __builtin_memcpy(&afrag[s][i], e, 16);
+            for (int j = 0; j < 5; ++j) {
+                int32_t at = w0 + j;
+                at = at < 0 ? 0 : (at > last_word ? last_word : at);
+                word[j] = raw32[real ? at : 0];
             }
+            uint4s rec;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const uint32_t v = odd ? (word[j] >> 16) | (word[j + 1] << 16) : word[j];
+                rec[j] = real ? v & keep[j] : 0u;
+            }
+            *reinterpret_cast<uint4s*>(records + u * 8) = rec;
+        }
     }
+    __syncthreads();
+    uint4s afrag[NS][2];
+#pragma unroll
+    for (int s = 0; s < NS; ++s)
+#pragma unroll
+        for (int i = 0; i < 2; ++i) afrag[s][i] = *reinterpret_cast<const uint4s*>(records + ((2 * s + lane / 32) * kStemBCO + i * 32 + lane % 32) * 8);
     float bias_v[2];
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
@@ -294,7 +311,9 @@ int run_stem(const ConvProblem& p, const void* x, const void* w, const void* bia
     const uint32_t chunks = p.W / 8;
     // the rows one step adds must fit the staging registers of the block
     if (static_cast<uint64_t>(p.C) * p.stride_h * chunks > kStemUnits * kStemThreads) return TANNIC_UNSUPPORTED_DTYPE;
-    const size_t raw_bytes = static_cast<size_t>(kStemBCO) * slots * p.KW * sizeof(T);
+    // the weights' stay in LDS: the copied rows, then 16-byte records for 2 * NS slots (NS as chosen below)
+    const uint32_t ns = (slots + 1) / 2, ns_built = ns <= 3 ? 3 : (ns <= 5 ? 5 : (ns <= 8 ? 8 : 11));
+    const size_t raw_bytes = (static_cast<size_t>(kStemBCO) * slots * p.KW + 8 + static_cast<size_t>(2 * ns_built) * kStemBCO * 8) * sizeof(T);
     size_t lds = (static_cast<size_t>(q.ring_elems) + kStemBCO * kStemOutPitch) * sizeof(T);
     if (lds < raw_bytes) lds = raw_bytes;
     if (lds > 64 * 1024) return TANNIC_UNSUPPORTED_DTYPE;
@@ -322,7 +341,6 @@ int run_stem(const ConvProblem& p, const void* x, const void* w, const void* bia
     q.div_chunks = FastDiv(chunks);
     q.div_c = FastDiv(p.C);
     q.vector_store = p.ys[3] == 1 && p.ys[2] % 8 == 0 && p.ys[1] % 8 == 0 && p.ys[0] % 8 == 0 && p.WO % 8 == 0 && reinterpret_cast<uintptr_t>(y) % 16 == 0;
-    const uint32_t ns = (slots + 1) / 2;
     const uint32_t b = static_cast<uint32_t>(blocks);
     if (ns <= 3) return launch_stem<T, 3>(p, q, b, lds, x, w, bias, y, stream);
     if (ns <= 5) return launch_stem<T, 5>(p, q, b, lds, x, w, bias, y, stream);
