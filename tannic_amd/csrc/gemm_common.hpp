@@ -40,6 +40,7 @@ int describe_gemm(const tannic_tensor_t* a, const tannic_tensor_t* b, const tann
 
 // MFMA paths; each returns TANNIC_UNSUPPORTED_DTYPE when the problem does not
 // meet its layout/alignment conditions so that the caller can fall back.
+int gemm_skinny_16bit(const GemmProblem& p, int dtype, const void* a, const void* b, void* c, hipStream_t stream);
 int gemm_mfma_16bit(const GemmProblem& p, int dtype, const void* a, const void* b, void* c, hipStream_t stream);
 int gemm_mfma_f32(const GemmProblem& p, const float* a, const float* b, float* c, hipStream_t stream);
 

@@ -177,8 +177,16 @@ using Loader = std::conditional_t<K_MAJOR, KMajorLoader<T, ROWS, THREADS>, RowMa
 
 // WAVES_N: wavefronts along N (2 -> 256 threads, one wavefront per SIMD; 4 -> 512 threads, two per SIMD, so that
 // one wavefront's waits are covered by the other's MFMAs); always two wavefronts along M.
-template <class T, int BM, int BN, int WAVES_N, bool A_KMAJOR, bool B_KMAJOR>
-__global__ __launch_bounds__(128 * WAVES_N) void gemm16_kernel(const T* A, const T* B, T* C, GemmProblem p, uint32_t tiles_m, uint32_t tiles_n) {
+// Where a block of a split product leaves its share: fp32, [split][batch][M][N].
+struct SplitK {
+    uint32_t splits, k_chunk;    // blocks per tile; K elements per block, a multiple of kBK
+    float* partials;
+};
+
+// SPLIT: several blocks share an output tile, each taking a range of K and storing its fp32 accumulators; a second
+// kernel adds the shares in split order, rounds once and writes C.
+template <class T, int BM, int BN, int WAVES_N, bool A_KMAJOR, bool B_KMAJOR, bool SPLIT = false>
+__global__ __launch_bounds__(128 * WAVES_N) void gemm16_kernel(const T* A, const T* B, T* C, GemmProblem p, uint32_t tiles_m, uint32_t tiles_n, SplitK sk) {
     constexpr int THREADS = 128 * WAVES_N;
     constexpr int WM = BM / 2, WN = BN / WAVES_N;
     constexpr int TM = WM / 32, TN = WN / 32;
@@ -188,11 +196,15 @@ __global__ __launch_bounds__(128 * WAVES_N) void gemm16_kernel(const T* A, const
     constexpr uint32_t A_TILE = BM * kBK, B_TILE = BN * kBK, B_BASE = 2 * A_TILE;
 
     uint32_t tm, tn;
-    tile_of(blockIdx.x, tiles_m, tiles_n, tm, tn);
+    const uint32_t tile_id = SPLIT ? blockIdx.x / sk.splits : blockIdx.x, split = SPLIT ? blockIdx.x % sk.splits : 0;
+    tile_of(tile_id, tiles_m, tiles_n, tm, tn);
     int64_t oa, ob, oc;
     batch_offsets(p, blockIdx.y, oa, ob, oc);
-    const Operand opA{A + oa, p.a_rs, p.a_cs, p.M};
-    const Operand opB{B + ob, p.b_cs, p.b_rs, p.N};   // rows of B's operand are the columns n
+    // this block's range of K: all of it, or its share
+    const uint32_t k_first = SPLIT ? split * sk.k_chunk : 0;
+    const uint32_t K = SPLIT ? (p.K - k_first < sk.k_chunk ? p.K - k_first : sk.k_chunk) : p.K;
+    const Operand opA{A + oa + static_cast<int64_t>(k_first) * p.a_cs, p.a_rs, p.a_cs, p.M};
+    const Operand opB{B + ob + static_cast<int64_t>(k_first) * p.b_rs, p.b_cs, p.b_rs, p.N};   // rows of B's operand are the columns n
     const uint32_t m0 = tm * BM, n0 = tn * BN;
 
     const int wave = threadIdx.x / 64, lane = threadIdx.x % 64;
@@ -215,11 +227,11 @@ __global__ __launch_bounds__(128 * WAVES_N) void gemm16_kernel(const T* A, const
     using LB = Loader<T, BN, THREADS, B_KMAJOR>;
     LA la;
     LB lb;
-    const uint32_t steps = (p.K + kBK - 1) / kBK;
+    const uint32_t steps = (K + kBK - 1) / kBK;
 
     // prologue: tile 0 into LDS buffer 0, tile 1 into registers
-    la.begin_fetch(opA, 0, p.K);
-    lb.begin_fetch(opB, 0, p.K);
+    la.begin_fetch(opA, 0, K);
+    lb.begin_fetch(opB, 0, K);
 #pragma unroll
     for (int i = 0; i < LA::LOADS; ++i) la.fetch_one(i, opA, m0);
 #pragma unroll
@@ -229,8 +241,8 @@ __global__ __launch_bounds__(128 * WAVES_N) void gemm16_kernel(const T* A, const
 #pragma unroll
     for (int i = 0; i < LB::STORES; ++i) lb.template commit_one<true>(i, lds + B_BASE);
     if (steps > 1) {
-        la.begin_fetch(opA, kBK, p.K);
-        lb.begin_fetch(opB, kBK, p.K);
+        la.begin_fetch(opA, kBK, K);
+        lb.begin_fetch(opB, kBK, K);
 #pragma unroll
         for (int i = 0; i < LA::LOADS; ++i) la.fetch_one(i, opA, m0);
 #pragma unroll
@@ -270,8 +282,8 @@ __global__ __launch_bounds__(128 * WAVES_N) void gemm16_kernel(const T* A, const
         T* a_next = lds + (cur ^ 1) * A_TILE;
         T* b_next = lds + B_BASE + (cur ^ 1) * B_TILE;
         if constexpr (FETCH) {
-            la.begin_fetch(opA, (s + 2) * kBK, p.K);
-            lb.begin_fetch(opB, (s + 2) * kBK, p.K);
+            la.begin_fetch(opA, (s + 2) * kBK, K);
+            lb.begin_fetch(opB, (s + 2) * kBK, K);
         }
         read_fragments(a_tile, b_tile, 0, 0);
         __builtin_amdgcn_sched_barrier(0);
@@ -323,6 +335,31 @@ __global__ __launch_bounds__(128 * WAVES_N) void gemm16_kernel(const T* A, const
     // columns.  Each wavefront rounds its WM x WN block into its own LDS area (nobody reads operand tiles any
     // more after the last barrier) and writes it out as whole rows: 16 bytes per lane, WN / 8 lanes per row, so
     // that the memory system sees full lines instead of fragments.
+    if constexpr (SPLIT) {
+        // lane: row lane % 32 of each 32x32 block, runs of four consecutive columns
+        float* mine = sk.partials + (static_cast<size_t>(split) * p.batches + blockIdx.y) * p.M * p.N;
+        const bool quads = p.N % 4 == 0;
+#pragma unroll
+        for (int i = 0; i < TM; ++i) {
+            const uint32_t row = m0 + wm + i * 32 + lane % 32;
+            if (row >= p.M) continue;
+            float* rp = mine + static_cast<size_t>(row) * p.N;
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+#pragma unroll
+                for (int g = 0; g < 4; ++g) {
+                    const uint32_t col = n0 + wn + j * 32 + g * 8 + 4 * (lane / 32);
+                    if (quads) {
+                        if (col < p.N) *reinterpret_cast<float4*>(rp + col) = float4{acc[i][j][g * 4], acc[i][j][g * 4 + 1], acc[i][j][g * 4 + 2], acc[i][j][g * 4 + 3]};
+                    } else {
+#pragma unroll
+                        for (int e = 0; e < 4; ++e)
+                            if (col + e < p.N) rp[col + e] = acc[i][j][g * 4 + e];
+                    }
+                }
+        }
+        return;
+    }
     T* c = C + oc;
     const bool vector_ok = p.c_rs % 8 == 0 && p.N % 8 == 0 && reinterpret_cast<uintptr_t>(c) % 16 == 0;
     if (vector_ok) {
@@ -365,21 +402,21 @@ __global__ __launch_bounds__(128 * WAVES_N) void gemm16_kernel(const T* A, const
     }
 }
 
-template <class T, int BM, int BN, int WAVES_N, bool AK, bool BK_>
-int launch16(const GemmProblem& p, const void* a, const void* b, void* c, hipStream_t stream) {
+template <class T, int BM, int BN, int WAVES_N, bool AK, bool BK_, bool SPLIT = false>
+int launch16(const GemmProblem& p, const void* a, const void* b, void* c, hipStream_t stream, SplitK sk = SplitK{1, 0, nullptr}) {
     const uint32_t tiles_m = (p.M + BM - 1) / BM, tiles_n = (p.N + BN - 1) / BN;
     // operand tiles (two buffers each); the same memory later stages the output, BM*BN elements in padded rows
     constexpr size_t tile_bytes = sizeof(T) * 2 * (BM + BN) * kBK;
     constexpr size_t stage_bytes = sizeof(T) * 2 * WAVES_N * (BM / 2) * (BN / WAVES_N + 8);
     constexpr size_t lds_bytes = tile_bytes > stage_bytes ? tile_bytes : stage_bytes;
-    auto kernel = gemm16_kernel<T, BM, BN, WAVES_N, AK, BK_>;
+    auto kernel = gemm16_kernel<T, BM, BN, WAVES_N, AK, BK_, SPLIT>;
     static bool configured = false;
     if (!configured) {
         TH_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes)));
         configured = true;
     }
-    hipLaunchKernelGGL(kernel, dim3(tiles_m * tiles_n, p.batches), dim3(128 * WAVES_N), lds_bytes, stream, static_cast<const T*>(a),
-                       static_cast<const T*>(b), static_cast<T*>(c), p, tiles_m, tiles_n);
+    hipLaunchKernelGGL(kernel, dim3(tiles_m * tiles_n * sk.splits, p.batches), dim3(128 * WAVES_N), lds_bytes, stream, static_cast<const T*>(a),
+                       static_cast<const T*>(b), static_cast<T*>(c), p, tiles_m, tiles_n, sk);
     return launch_status("gemm16_kernel");
 }
 
@@ -389,6 +426,52 @@ int pick_layout16(const GemmProblem& p, bool ak, bool bk, const void* a, const v
     if (ak) return launch16<T, BM, BN, WAVES_N, true, false>(p, a, b, c, s);
     if (bk) return launch16<T, BM, BN, WAVES_N, false, true>(p, a, b, c, s);
     return launch16<T, BM, BN, WAVES_N, false, false>(p, a, b, c, s);
+}
+
+// C[batch][m][n] = sum over splits of partials[split][batch][m][n], four columns per thread
+template <class T>
+__global__ __launch_bounds__(256) void gemm_split_reduce_kernel(const float* partials, T* C, GemmProblem p, uint32_t splits, uint32_t quads_per_row, uint32_t total) {
+    const uint32_t idx = blockIdx.x * 256 + threadIdx.x;
+    if (idx >= total) return;
+    const uint32_t r = idx / quads_per_row, col = (idx % quads_per_row) * 4;
+    const uint32_t batch = r / p.M, m = r % p.M;
+    const size_t share = static_cast<size_t>(p.batches) * p.M * p.N;
+    const float* src = partials + static_cast<size_t>(r) * p.N + col;
+    float sum[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+    const uint32_t live = p.N - col < 4 ? p.N - col : 4;
+    for (uint32_t sp = 0; sp < splits; ++sp)
+        for (uint32_t e = 0; e < live; ++e) sum[e] += src[sp * share + e];
+    int64_t oa, ob, oc;
+    batch_offsets(p, batch, oa, ob, oc);
+    T* dst = C + oc + static_cast<int64_t>(m) * p.c_rs + col;
+    for (uint32_t e = 0; e < live; ++e) dst[e] = narrow<T>(sum[e]);
+}
+
+// Few tiles and a long K: each tile is shared by `splits` blocks.
+template <class T, int BM>
+int run16_split(const GemmProblem& p, bool ak, bool bk, uint32_t splits, const void* a, const void* b, void* c, hipStream_t stream) {
+    constexpr int BN = 128;
+    const uint32_t steps = (p.K + kBK - 1) / kBK;
+    SplitK sk{};
+    sk.k_chunk = (steps + splits - 1) / splits * kBK;
+    sk.splits = (p.K + sk.k_chunk - 1) / sk.k_chunk;   // no block without a step
+    const uint64_t rows = static_cast<uint64_t>(p.batches) * p.M, quads_per_row = (p.N + 3) / 4;
+    if (rows * quads_per_row >= (1ull << 31)) return TANNIC_UNSUPPORTED_DTYPE;
+    const size_t bytes = static_cast<size_t>(sk.splits) * rows * p.N * sizeof(float);
+    if (scratch_acquire(reinterpret_cast<void**>(&sk.partials), bytes, stream) != TANNIC_SUCCESS) return TANNIC_ERROR;
+    int status;
+    if (ak && bk) status = launch16<T, BM, BN, 2, true, true, true>(p, a, b, c, stream, sk);
+    else if (ak) status = launch16<T, BM, BN, 2, true, false, true>(p, a, b, c, stream, sk);
+    else if (bk) status = launch16<T, BM, BN, 2, false, true, true>(p, a, b, c, stream, sk);
+    else status = launch16<T, BM, BN, 2, false, false, true>(p, a, b, c, stream, sk);
+    if (status == TANNIC_SUCCESS) {
+        const uint32_t total = static_cast<uint32_t>(rows * quads_per_row);
+        hipLaunchKernelGGL((gemm_split_reduce_kernel<T>), dim3((total + 255) / 256), dim3(256), 0, stream, sk.partials, static_cast<T*>(c), p, sk.splits,
+                           static_cast<uint32_t>(quads_per_row), total);
+        status = launch_status("gemm_split_reduce_kernel");
+    }
+    scratch_release(sk.partials, stream);
+    return status;
 }
 
 template <class T>
@@ -411,11 +494,25 @@ int run16(const GemmProblem& p, const void* a, const void* b, void* c, hipStream
     const uint64_t big = static_cast<uint64_t>((p.M + 255) / 256) * ((p.N + 255) / 256) * p.batches;
     if (big >= 200) return pick_layout16<T, 256, 256, 2>(p, ak, bk, a, b, c, stream);
     const uint64_t mid = static_cast<uint64_t>((p.M + 127) / 128) * ((p.N + 127) / 128) * p.batches;
-    if (mid >= 128 || p.M > 64) return pick_layout16<T, 128, 128, 2>(p, ak, bk, a, b, c, stream);
+    if (mid >= 200) return pick_layout16<T, 128, 128, 2>(p, ak, bk, a, b, c, stream);
+    // too few tiles for the chip: a share of K per block while a block keeps four steps.  Tiles as tall as M allows,
+    // so that the other operand is read once.
+    const bool tall = p.M > 64;
+    const uint64_t few = tall ? mid : static_cast<uint64_t>((p.M + 63) / 64) * ((p.N + 127) / 128) * p.batches;
+    uint64_t splits = few < 256 ? 256 / few : 1;
+    if (splits > p.K / 256) splits = p.K / 256;
+    if (splits > 1 && !p.row_bias) {
+        if (tall) return run16_split<T, 128>(p, ak, bk, static_cast<uint32_t>(splits), a, b, c, stream);
+        return run16_split<T, 64>(p, ak, bk, static_cast<uint32_t>(splits), a, b, c, stream);
+    }
+    if (tall) return pick_layout16<T, 128, 128, 2>(p, ak, bk, a, b, c, stream);
     return pick_layout16<T, 64, 128, 2>(p, ak, bk, a, b, c, stream);
 }
 
 int gemm_mfma_16bit(const GemmProblem& p, int dtype, const void* a, const void* b, void* c, hipStream_t stream) {
+    // a handful of rows: stream the other operand once, no tiles
+    const int skinny = gemm_skinny_16bit(p, dtype, a, b, c, stream);
+    if (skinny != TANNIC_UNSUPPORTED_DTYPE) return skinny;
     if (dtype == TANNIC_FLOAT16) return run16<f16>(p, a, b, c, stream);
     if (dtype == TANNIC_BFLOAT16) return run16<bf16>(p, a, b, c, stream);
     return TANNIC_UNSUPPORTED_DTYPE;

@@ -1,0 +1,142 @@
+// Matrix product with very few rows (M <= 32), 16-bit types: y = x * W^T as the
+// decoding step of a transformer runs it.  The work is reading W once; there is
+// nothing to reuse, so nothing goes through LDS on the way in.
+//
+// v_mfma_f32_16x16x32: a block of 512 threads owns 16 columns of the result (16
+// rows of W, which is K-contiguous); its eight wavefronts split K.  A lane loads
+// its operand fragments straight from global memory — 16 bytes of a row of W
+// (row lane % 16, k chunk lane / 16: four lanes cover 64 contiguous bytes of a
+// row) and 16 bytes of a row of x — eight steps at a time, so that 8 KB per
+// wavefront are in flight.  The eight partial 16x16 tiles meet in LDS, the
+// first wavefront adds them, rounds once and stores four consecutive columns
+// per lane.
+#include "gemm_common.hpp"
+
+namespace th {
+
+typedef _Float16 half8y __attribute__((ext_vector_type(8)));
+typedef __bf16 bfloat8y __attribute__((ext_vector_type(8)));
+typedef float float4y __attribute__((ext_vector_type(4)));
+typedef unsigned int uint4y __attribute__((ext_vector_type(4)));
+
+template <class T> __device__ inline float4y skinny_mfma(uint4y a, uint4y b, float4y c) {
+    if constexpr (std::is_same_v<T, f16>) {
+        half8y x, y;
+        __builtin_memcpy(&x, &a, 16);
+        __builtin_memcpy(&y, &b, 16);
+        return __builtin_amdgcn_mfma_f32_16x16x32_f16(x, y, c, 0, 0, 0);
+    } else {
+        bfloat8y x, y;
+        __builtin_memcpy(&x, &a, 16);
+        __builtin_memcpy(&y, &b, 16);
+        return __builtin_amdgcn_mfma_f32_16x16x32_bf16(x, y, c, 0, 0, 0);
+    }
+}
+
+constexpr int kSkinnyWaves = 8;
+constexpr int kSkinnyUnroll = 8;   // K steps of 32 whose loads are issued together
+
+// what a chunk past the end of K reads instead: both operands, so that the product is an exact zero
+__device__ const uint4y skinny_zeros = {0, 0, 0, 0};
+
+// MB: blocks of 16 rows of x
+template <class T, int MB>
+__global__ __launch_bounds__(64 * kSkinnyWaves) void gemm_skinny_kernel(const T* x, const T* w, T* c, GemmProblem p, uint32_t k_per_wave) {
+    __shared__ float4y partial[kSkinnyWaves][MB][64];
+    int64_t ox, ow, oc;
+    batch_offsets(p, blockIdx.y, ox, ow, oc);
+    const int wave = threadIdx.x / 64, lane = threadIdx.x % 64;
+    const uint32_t r = lane % 16, kc = lane / 16;
+    const uint32_t n0 = blockIdx.x * 16;
+    // rows past the end are read from the last row: they only feed results that are never stored
+    const uint32_t n = n0 + r < p.N ? n0 + r : p.N - 1;
+    const T* wrow = w + ow + static_cast<int64_t>(n) * p.b_cs + kc * 8;
+    const T* xrow[MB];
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb) {
+        const uint32_t m = mb * 16 + r < p.M ? mb * 16 + r : p.M - 1;
+        xrow[mb] = x + ox + static_cast<int64_t>(m) * p.a_rs + kc * 8;
+    }
+    const uint32_t k_begin = wave * k_per_wave;
+    const uint32_t k_end = k_begin + k_per_wave < p.K ? k_begin + k_per_wave : p.K;
+    const T* zeros = reinterpret_cast<const T*>(&skinny_zeros) - kc * 8;
+
+    float4y acc[MB];
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb) acc[mb] = float4y{0.0f, 0.0f, 0.0f, 0.0f};
+    for (uint32_t k0 = k_begin; k0 < k_end; k0 += 32 * kSkinnyUnroll) {
+        uint4y fw[kSkinnyUnroll], fx[kSkinnyUnroll][MB];
+#pragma unroll
+        for (int u = 0; u < kSkinnyUnroll; ++u) {
+            const uint32_t k = k0 + 32 * u;
+            const bool live = k + kc * 8 < k_end;   // K and the ranges are multiples of 8: a chunk is inside or outside
+            fw[u] = *reinterpret_cast<const uint4y*>(live ? wrow + k : zeros + kc * 8);
+#pragma unroll
+            for (int mb = 0; mb < MB; ++mb) fx[u][mb] = *reinterpret_cast<const uint4y*>(live ? xrow[mb] + k : zeros + kc * 8);
+        }
+#pragma unroll
+        for (int u = 0; u < kSkinnyUnroll; ++u)
+#pragma unroll
+            for (int mb = 0; mb < MB; ++mb) acc[mb] = skinny_mfma<T>(fw[u], fx[u][mb], acc[mb]);
+    }
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb) partial[wave][mb][lane] = acc[mb];
+    __syncthreads();
+    if (wave != 0) return;
+    // accumulator: lane -> row of x (m) lane % 16; value v -> column n0 + 4 * (lane / 16) + v
+    T* cb = c + oc;
+    const bool vector_ok = p.c_rs % 4 == 0 && p.N % 4 == 0 && reinterpret_cast<uintptr_t>(cb) % 8 == 0;
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb) {
+        float4y sum = partial[0][mb][lane];
+#pragma unroll
+        for (int v = 1; v < kSkinnyWaves; ++v) sum += partial[v][mb][lane];
+        const uint32_t m = mb * 16 + r, col = n0 + 4 * kc;
+        if (m >= p.M) continue;
+        T out[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) out[e] = narrow<T>(sum[e]);
+        T* dst = cb + static_cast<int64_t>(m) * p.c_rs + col;
+        if (vector_ok) {
+            if (col < p.N) {
+                uint2 bits;
+                __builtin_memcpy(&bits, out, 8);
+                *reinterpret_cast<uint2*>(dst) = bits;
+            }
+        } else {
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+                if (col + e < p.N) dst[e] = out[e];
+        }
+    }
+}
+
+template <class T>
+int run_skinny(const GemmProblem& p, const void* a, const void* b, void* c, hipStream_t stream) {
+    if (p.M == 0 || p.M > 32 || p.N == 0 || p.K == 0 || p.batches == 0 || p.batches > 65535 || p.row_bias) return TANNIC_UNSUPPORTED_DTYPE;
+    // both operands K-contiguous; 16-byte chunks along K
+    if (p.a_cs != 1 || p.b_rs != 1) return TANNIC_UNSUPPORTED_DTYPE;
+    auto mult8 = [](int64_t v) { return v % 8 == 0; };
+    if (!mult8(p.K) || !mult8(p.a_rs) || !mult8(p.b_cs)) return TANNIC_UNSUPPORTED_DTYPE;
+    if (reinterpret_cast<uintptr_t>(a) % 16 || reinterpret_cast<uintptr_t>(b) % 16) return TANNIC_UNSUPPORTED_DTYPE;
+    for (int d = 0; d < p.batch_rank; ++d)
+        if (!mult8(p.a_bs[d]) || !mult8(p.b_bs[d])) return TANNIC_UNSUPPORTED_DTYPE;
+    // K is split evenly over the wavefronts, in whole steps of 32
+    const uint32_t steps = (p.K + 31) / 32, per_wave = (steps + kSkinnyWaves - 1) / kSkinnyWaves;
+    const uint32_t k_per_wave = per_wave * 32;
+    const uint32_t blocks = (p.N + 15) / 16;
+    const dim3 grid(blocks, p.batches), block(64 * kSkinnyWaves);
+    if (p.M <= 16)
+        hipLaunchKernelGGL((gemm_skinny_kernel<T, 1>), grid, block, 0, stream, static_cast<const T*>(a), static_cast<const T*>(b), static_cast<T*>(c), p, k_per_wave);
+    else
+        hipLaunchKernelGGL((gemm_skinny_kernel<T, 2>), grid, block, 0, stream, static_cast<const T*>(a), static_cast<const T*>(b), static_cast<T*>(c), p, k_per_wave);
+    return launch_status("gemm_skinny_kernel");
+}
+
+int gemm_skinny_16bit(const GemmProblem& p, int dtype, const void* a, const void* b, void* c, hipStream_t stream) {
+    if (dtype == TANNIC_FLOAT16) return run_skinny<f16>(p, a, b, c, stream);
+    if (dtype == TANNIC_BFLOAT16) return run_skinny<bf16>(p, a, b, c, stream);
+    return TANNIC_UNSUPPORTED_DTYPE;
+}
+
+}  // namespace th

@@ -37,6 +37,11 @@ LAYOUTS = {
     "sixteen_rows": ((16, 256), (96, 256), [], [("transpose", (-1, -2))]),
     "single_column": ((64, 96), (1, 96), [], [("transpose", (-1, -2))]),
     "k_one": ((9, 1), (1, 11), [], []),
+    # few rows: ragged K steps and columns, two row blocks, batches; a long K shared between blocks
+    "skinny_17_rows_ragged": ((17, 72), (40, 72), [], [("transpose", (-1, -2))]),
+    "skinny_batched": ((3, 5, 64), (3, 24, 64), [], [("transpose", (-1, -2))]),
+    "split_k_nt": ((128, 1096), (136, 1096), [], [("transpose", (-1, -2))]),
+    "split_k_nn": ((72, 2048), (2048, 64), [], []),
 }
 
 
