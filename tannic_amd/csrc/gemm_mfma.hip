@@ -15,8 +15,10 @@
 //   a plain row-major B) is read as 8x8 micro-blocks and transposed in
 //   registers on its way to LDS.
 //
-// fp32 operands: v_mfma_f32_32x32x2f32 (true fp32), same tiling with K steps
-//   of 16; fragments are single LDS words.
+// fp32 operands: v_mfma_f32_32x32x2f32 (true fp32), the same kernel with K steps
+//   of 32 (rows of a tile stay 128 bytes): a 16-byte fragment feeds four MFMAs,
+//   one per element; which k an element stands for is the same permutation for
+//   both operands.  The result is written from the accumulators as 16 bytes per lane.
 //
 // Workgroup ids are dealt round-robin to the 8 XCDs, each with its own L2, so
 // the id is first folded (id % 8 selects the XCD's contiguous share of tiles)
@@ -49,8 +51,22 @@ template <> struct Mfma16<bf16> {
     }
 };
 
-constexpr int kBK = 64;          // K elements per step (16-bit kernels)
-constexpr int kChunk = 8;        // 16-bit elements per 16-byte chunk
+// A tile row is 128 bytes = eight 16-byte chunks for every element type.
+template <class T> constexpr int kBKof = 128 / sizeof(T);      // K elements per step: 64 (16-bit), 32 (fp32)
+template <class T> constexpr int kChunkOf = 16 / sizeof(T);    // elements per 16-byte chunk
+template <> struct Mfma16<float> {
+    // element e of both fragments is one k: four 32x32x2 MFMAs (lanes 0-31 hold one k of the pair, lanes 32-63 the other)
+    __device__ static inline float16v run(uint4v a, uint4v b, float16v c) {
+        float x[4], y[4];
+        __builtin_memcpy(x, &a, 16);
+        __builtin_memcpy(y, &b, 16);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) c = __builtin_amdgcn_mfma_f32_32x32x2f32(x[e], y[e], c, 0, 0, 0);
+        return c;
+    }
+};
+
+constexpr int kBK = 64;          // K granule the host splits by (a multiple of every type's step)
 
 // Maps the hardware workgroup id to a tile: XCD folding, then grouped rows.
 __device__ inline void tile_of(uint32_t wg, uint32_t tiles_m, uint32_t tiles_n, uint32_t& tm, uint32_t& tn) {
@@ -83,11 +99,11 @@ __device__ inline void static_for(F&& f) {
     }
 }
 
-// Swizzled element offset of (row, chunk) inside a [ROWS][64] tile.
+// Swizzled element offset of (row, chunk) inside a [ROWS][128 bytes] tile.
 // LDS serves 16 lanes of a 16-byte read per clock out of a 256-byte bank window,
 // i.e. two 128-byte rows: consecutive row PAIRS get different chunk rotations so
 // that 16 consecutive rows of one logical chunk land in 16 different slots.
-__device__ inline uint32_t tile_offset(uint32_t row, uint32_t chunk) { return row * kBK + ((chunk ^ ((row >> 1) & 7u)) * kChunk); }
+template <class T> __device__ inline uint32_t tile_offset(uint32_t row, uint32_t chunk) { return row * kBKof<T> + ((chunk ^ ((row >> 1) & 7u)) * kChunkOf<T>); }
 
 // ---- global -> registers -> LDS, operand contiguous along K -------------------
 // Rows past the operand's end read a clamped (valid) address: they only feed
@@ -104,7 +120,7 @@ struct KMajorLoader {
     const T* base;      // operand base + this thread's k offset for the tile being fetched
     bool k_live;
     __device__ inline void begin_fetch(const Operand& op, uint32_t k0, uint32_t K) {
-        const uint32_t k = k0 + (threadIdx.x % 8) * kChunk;
+        const uint32_t k = k0 + (threadIdx.x % 8) * kChunkOf<T>;
         k_live = k < K;
         base = static_cast<const T*>(op.base) + (k_live ? k : 0);
     }
@@ -115,7 +131,7 @@ struct KMajorLoader {
     }
     template <bool MASK>
     __device__ inline void commit_one(int i, T* tile) const {
-        *reinterpret_cast<uint4v*>(tile + tile_offset(threadIdx.x / 8 + ROWS_PER_PASS * i, threadIdx.x % 8)) =
+        *reinterpret_cast<uint4v*>(tile + tile_offset<T>(threadIdx.x / 8 + ROWS_PER_PASS * i, threadIdx.x % 8)) =
             (!MASK || k_live) ? regs[i] : uint4v{0, 0, 0, 0};
     }
     // Order of the step's memory operations: register i is written to LDS and refilled right away, so
@@ -125,51 +141,53 @@ struct KMajorLoader {
     static constexpr int index_of(int o) { return o / 2; }
 };
 
-// ---- operand contiguous along its row index: 8x8 micro-blocks, transposed --------
+// ---- operand contiguous along its row index: E x E micro-blocks (E elements per 16 bytes), transposed --------
 template <class T, int ROWS, int THREADS>
 struct RowMajorLoader {
-    // ROWS/8 row-blocks x 8 k-blocks micro-blocks over THREADS threads
-    static constexpr int PASSES = (ROWS + THREADS - 1) / THREADS;
-    static constexpr int LOADS = 8 * PASSES, STORES = 8 * PASSES;
-    uint4v regs[PASSES][8];
-    uint32_t kfirst, k_count;  // first k of this thread's micro-block; how many of its 8 k values are inside K
+    static constexpr int E = kChunkOf<T>;
+    using U = std::conditional_t<sizeof(T) == 2, uint16_t, uint32_t>;
+    // ROWS/E row-blocks x 8 k-blocks micro-blocks over THREADS threads
+    static constexpr int BLOCKS = ROWS / E * 8;
+    static constexpr int PASSES = (BLOCKS + THREADS - 1) / THREADS;
+    static constexpr int LOADS = E * PASSES, STORES = E * PASSES;
+    uint4v regs[PASSES][E];
+    uint32_t kfirst, k_count;  // first k of this thread's micro-block; how many of its E k values are inside K
     uint32_t K_;
     __device__ inline void begin_fetch(const Operand&, uint32_t k0, uint32_t K) {
-        kfirst = k0 + (threadIdx.x % 8) * 8;
-        k_count = kfirst >= K ? 0 : (K - kfirst < 8 ? K - kfirst : 8);
+        kfirst = k0 + (threadIdx.x % 8) * E;
+        k_count = kfirst >= K ? 0 : (K - kfirst < E ? K - kfirst : E);
         K_ = K;
     }
     __device__ inline void fetch_one(int idx, const Operand& op, uint32_t row0) {
-        const int i = idx / 8, kk = idx % 8;
+        const int i = idx / E, kk = idx % E;
         const uint32_t rb = (threadIdx.x + THREADS * i) / 8;
-        const uint32_t row = row0 + rb * 8;
-        const uint32_t srow = (rb < ROWS / 8 && row < op.rows) ? row : 0;
+        const uint32_t row = row0 + rb * E;
+        const uint32_t srow = (rb < ROWS / E && row < op.rows) ? row : 0;
         const uint32_t k = kfirst + kk;
         regs[i][kk] = *reinterpret_cast<const uint4v*>(static_cast<const T*>(op.base) + static_cast<int64_t>(k < K_ ? k : 0) * op.k_stride + srow);
     }
     template <bool MASK>
     __device__ inline void commit_one(int idx, T* tile) const {
-        const int i = idx / 8, rr = idx % 8;
+        const int i = idx / E, rr = idx % E;
         const uint32_t mb = threadIdx.x + THREADS * i;
         const uint32_t kb = mb % 8, rb = mb / 8;
-        if (rb >= ROWS / 8) return;
-        // row rr of the transposed micro-block: element rr of each of the 8 loaded vectors
-        uint16_t out[8];
+        if (rb >= ROWS / E) return;
+        // row rr of the transposed micro-block: element rr of each of the E loaded vectors
+        U out[E];
 #pragma unroll
-        for (int kk = 0; kk < 8; ++kk) {
-            uint16_t in[8];
+        for (int kk = 0; kk < E; ++kk) {
+            U in[E];
             __builtin_memcpy(in, &regs[i][kk], 16);
-            out[kk] = (!MASK || static_cast<uint32_t>(kk) < k_count) ? in[rr] : uint16_t(0);
+            out[kk] = (!MASK || static_cast<uint32_t>(kk) < k_count) ? in[rr] : U(0);
         }
         uint4v v;
         __builtin_memcpy(&v, out, 16);
-        *reinterpret_cast<uint4v*>(tile + tile_offset(rb * 8 + rr, kb)) = v;
+        *reinterpret_cast<uint4v*>(tile + tile_offset<T>(rb * E + rr, kb)) = v;
     }
-    // A micro-block is transposed out of all eight of its registers: the eight writes of a pass, then its
-    // eight refills.
+    // A micro-block is transposed out of all of its registers: the E writes of a pass, then its E refills.
     static constexpr int OPS = STORES + LOADS;
-    static constexpr bool is_commit(int o) { return o % 16 < 8; }
-    static constexpr int index_of(int o) { return (o / 16) * 8 + o % 8; }
+    static constexpr bool is_commit(int o) { return o % (2 * E) < E; }
+    static constexpr int index_of(int o) { return (o / (2 * E)) * E + o % E; }
 };
 
 template <class T, int ROWS, int THREADS, bool K_MAJOR>
@@ -193,6 +211,7 @@ __global__ __launch_bounds__(128 * WAVES_N) void gemm16_kernel(const T* A, const
     extern __shared__ __align__(16) unsigned char lds_raw[];
     // layout: A buffer 0, A buffer 1, B buffer 0, B buffer 1 (offsets in elements)
     T* lds = reinterpret_cast<T*>(lds_raw);
+    constexpr int kBK = kBKof<T>;   // K elements per step
     constexpr uint32_t A_TILE = BM * kBK, B_TILE = BN * kBK, B_BASE = 2 * A_TILE;
 
     uint32_t tm, tn;
@@ -258,13 +277,13 @@ __global__ __launch_bounds__(128 * WAVES_N) void gemm16_kernel(const T* A, const
     // The registers hold tile s+1 on entry.  Between the MFMAs, one memory operation at a time: register i
     // goes to LDS (tile s+1) and is refilled from global memory (tile s+2).  sched_barrier pins that
     // interleaving so that neither the load unit nor the LDS ever sees a burst while the matrix pipe idles.
-    constexpr int KS = kBK / 16, PER_KS = TM * TN;
+    constexpr int KS = 4, PER_KS = TM * TN;   // a k-slice is two chunks: one per half of the wavefront
     uint4v fa[2][TM], fb[2][TN];
     auto read_fragments = [&](const T* a_tile, const T* b_tile, int ks, int into) {
 #pragma unroll
-        for (int x = 0; x < TM; ++x) fa[into][x] = *reinterpret_cast<const uint4v*>(a_tile + tile_offset(wm + x * 32 + frag_row, ks * 2 + frag_chunk));
+        for (int x = 0; x < TM; ++x) fa[into][x] = *reinterpret_cast<const uint4v*>(a_tile + tile_offset<T>(wm + x * 32 + frag_row, ks * 2 + frag_chunk));
 #pragma unroll
-        for (int y = 0; y < TN; ++y) fb[into][y] = *reinterpret_cast<const uint4v*>(b_tile + tile_offset(wn + y * 32 + frag_row, ks * 2 + frag_chunk));
+        for (int y = 0; y < TN; ++y) fb[into][y] = *reinterpret_cast<const uint4v*>(b_tile + tile_offset<T>(wn + y * 32 + frag_row, ks * 2 + frag_chunk));
     };
     // (for tile 0 the "previous tile's" fragments are zeros: 16 MFMAs that add nothing keep the loop free of a
     // peeled first iteration, whose extra copy of the code costs more than it saves)
@@ -361,6 +380,30 @@ __global__ __launch_bounds__(128 * WAVES_N) void gemm16_kernel(const T* A, const
         return;
     }
     T* c = C + oc;
+    if constexpr (sizeof(T) == 4) {
+        // four consecutive columns per lane are 16 bytes already
+        const bool quads = p.c_rs % 4 == 0 && p.N % 4 == 0 && reinterpret_cast<uintptr_t>(c) % 16 == 0;
+#pragma unroll
+        for (int i = 0; i < TM; ++i) {
+            const uint32_t row = m0 + wm + i * 32 + lane % 32;
+            if (row >= p.M) continue;
+            T* rp = c + static_cast<int64_t>(row) * p.c_rs;
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+#pragma unroll
+                for (int g = 0; g < 4; ++g) {
+                    const uint32_t col = n0 + wn + j * 32 + g * 8 + 4 * (lane / 32);
+                    if (quads) {
+                        if (col < p.N) *reinterpret_cast<float4*>(rp + col) = float4{acc[i][j][g * 4], acc[i][j][g * 4 + 1], acc[i][j][g * 4 + 2], acc[i][j][g * 4 + 3]};
+                    } else {
+#pragma unroll
+                        for (int e = 0; e < 4; ++e)
+                            if (col + e < p.N) rp[col + e] = acc[i][j][g * 4 + e];
+                    }
+                }
+        }
+        return;
+    }
     const bool vector_ok = p.c_rs % 8 == 0 && p.N % 8 == 0 && reinterpret_cast<uintptr_t>(c) % 16 == 0;
     if (vector_ok) {
         constexpr int PITCH = WN + 8;                       // elements: rows stay 16-byte aligned and shift by four banks
@@ -406,9 +449,9 @@ template <class T, int BM, int BN, int WAVES_N, bool AK, bool BK_, bool SPLIT = 
 int launch16(const GemmProblem& p, const void* a, const void* b, void* c, hipStream_t stream, SplitK sk = SplitK{1, 0, nullptr}) {
     const uint32_t tiles_m = (p.M + BM - 1) / BM, tiles_n = (p.N + BN - 1) / BN;
     // operand tiles (two buffers each); the same memory later stages the output, BM*BN elements in padded rows
-    constexpr size_t tile_bytes = sizeof(T) * 2 * (BM + BN) * kBK;
+    constexpr size_t tile_bytes = sizeof(T) * 2 * (BM + BN) * kBKof<T>;
     constexpr size_t stage_bytes = sizeof(T) * 2 * WAVES_N * (BM / 2) * (BN / WAVES_N + 8);
-    constexpr size_t lds_bytes = tile_bytes > stage_bytes ? tile_bytes : stage_bytes;
+    constexpr size_t lds_bytes = (sizeof(T) == 2 && stage_bytes > tile_bytes) ? stage_bytes : tile_bytes;   // fp32 results are not staged
     auto kernel = gemm16_kernel<T, BM, BN, WAVES_N, AK, BK_, SPLIT>;
     static bool configured = false;
     if (!configured) {
@@ -482,8 +525,8 @@ int run16(const GemmProblem& p, const void* a, const void* b, void* c, hipStream
     if (!ak && p.a_rs != 1) return TANNIC_UNSUPPORTED_DTYPE;
     if (!bk && p.b_cs != 1) return TANNIC_UNSUPPORTED_DTYPE;
     // 16-byte accesses: addresses, leading dimensions, batch strides and the
-    // contiguous extent must be multiples of 8 elements
-    auto mult8 = [](int64_t v) { return v % 8 == 0; };
+    // contiguous extent must be multiples of a chunk (8 elements of 16 bits, 4 of 32)
+    auto mult8 = [](int64_t v) { return v % kChunkOf<T> == 0; };
     if (reinterpret_cast<uintptr_t>(a) % 16 || reinterpret_cast<uintptr_t>(b) % 16) return TANNIC_UNSUPPORTED_DTYPE;
     if (!mult8(ak ? p.a_rs : p.a_cs) || !mult8(bk ? p.b_cs : p.b_rs)) return TANNIC_UNSUPPORTED_DTYPE;
     if (!mult8(ak ? p.K : p.M) || !mult8(bk ? p.K : p.N)) return TANNIC_UNSUPPORTED_DTYPE;
@@ -518,6 +561,6 @@ int gemm_mfma_16bit(const GemmProblem& p, int dtype, const void* a, const void* 
     return TANNIC_UNSUPPORTED_DTYPE;
 }
 
-int gemm_mfma_f32(const GemmProblem&, const float*, const float*, float*, hipStream_t) { return TANNIC_UNSUPPORTED_DTYPE; }
+int gemm_mfma_f32(const GemmProblem& p, const float* a, const float* b, float* c, hipStream_t stream) { return run16<float>(p, a, b, c, stream); }
 
 }  // namespace th
