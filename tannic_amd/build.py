@@ -45,6 +45,7 @@ UNITS = [
     ("conv2d_k3.hip", "conv2d_k3.o", []),
     ("conv2d_pointwise.hip", "conv2d_pointwise.o", []),
     ("conv2d_stem.hip", "conv2d_stem.o", []),
+    ("conv2d_unfold.hip", "conv2d_unfold.o", []),
 ]
 
 

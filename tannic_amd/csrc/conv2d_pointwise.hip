@@ -1,4 +1,4 @@
-// conv2d with a 1x1 kernel, 16-bit signals: a matrix product per image.
+// conv2d with a 1x1 kernel, fp16 / bf16 / fp32 signals: a matrix product per image.
 //
 // y[n] (O x HO*WO) = w (O x C) * x[n] (C x HO*WO): the kernel tensor is the
 // K-contiguous operand, an NCHW image is the row-major one (pixels contiguous for
@@ -26,9 +26,16 @@ __global__ __launch_bounds__(256) void conv_subsample4_kernel(const T* x, T* out
     T v[4];
 #pragma unroll
     for (int e = 0; e < 4; ++e) v[e] = src[static_cast<int64_t>(e * p.stride_w) * p.xs[3]];
-    uint2 bits;
-    __builtin_memcpy(&bits, v, 8);
-    *reinterpret_cast<uint2*>(out + static_cast<int64_t>(row) * p.WO + quad * 4) = bits;
+    using Quad = std::conditional_t<sizeof(T) == 2, uint2, uint4>;
+    Quad bits;
+    __builtin_memcpy(&bits, v, sizeof(Quad));
+    *reinterpret_cast<Quad*>(out + static_cast<int64_t>(row) * p.WO + quad * 4) = bits;
+}
+
+template <class T>
+int product(const GemmProblem& g, int dtype, const void* a, const void* b, void* c, hipStream_t stream) {
+    if constexpr (std::is_same_v<T, float>) return gemm_mfma_f32(g, static_cast<const float*>(a), static_cast<const float*>(b), static_cast<float*>(c), stream);
+    else return gemm_mfma_16bit(g, dtype, a, b, c, stream);
 }
 
 template <class T>
@@ -63,10 +70,11 @@ int run_pointwise(const ConvProblem& p, int dtype, const void* x, const void* w,
         if (p.xs[3] != 1 || p.xs[2] != static_cast<int64_t>(p.W)) return TANNIC_UNSUPPORTED_DTYPE;
         g.b_rs = p.xs[1];
         g.b_bs[0] = p.xs[0];
-        return gemm_mfma_16bit(g, dtype, w, x, y, stream);
+        return product<T>(g, dtype, w, x, y, stream);
     }
     // strided: gather first.  The product's own conditions are checked before any work is queued.
-    if (p.WO % 4 != 0 || pixels % 8 != 0 || p.ws[0] % 8 != 0 || p.C % 8 != 0 || reinterpret_cast<uintptr_t>(w) % 16 != 0) return TANNIC_UNSUPPORTED_DTYPE;
+    constexpr int E = 16 / sizeof(T);   // elements per 16 bytes
+    if (p.WO % 4 != 0 || pixels % E != 0 || p.ws[0] % E != 0 || p.C % E != 0 || reinterpret_cast<uintptr_t>(w) % 16 != 0) return TANNIC_UNSUPPORTED_DTYPE;
     const uint64_t rows = static_cast<uint64_t>(p.N) * p.C * p.HO, quads = rows * (p.WO / 4);
     if (quads >= (1ull << 31)) return TANNIC_UNSUPPORTED_DTYPE;
     T* dense_x = nullptr;
@@ -77,7 +85,7 @@ int run_pointwise(const ConvProblem& p, int dtype, const void* x, const void* w,
     if (status == TANNIC_SUCCESS) {
         g.b_rs = static_cast<int64_t>(pixels);
         g.b_bs[0] = static_cast<int64_t>(p.C) * static_cast<int64_t>(pixels);
-        status = gemm_mfma_16bit(g, dtype, w, dense_x, y, stream);
+        status = product<T>(g, dtype, w, dense_x, y, stream);
         // the conditions above are the product's: a refusal here would leave the result unwritten
         if (status == TANNIC_UNSUPPORTED_DTYPE) {
             set_error_text("conv2d: internal: the 1x1 product refused a problem its caller had checked");
@@ -91,6 +99,7 @@ int run_pointwise(const ConvProblem& p, int dtype, const void* x, const void* w,
 int conv2d_pointwise(const ConvProblem& p, int dtype, const void* x, const void* w, const void* bias, void* y, hipStream_t stream) {
     if (dtype == TANNIC_FLOAT16) return run_pointwise<f16>(p, dtype, x, w, bias, y, stream);
     if (dtype == TANNIC_BFLOAT16) return run_pointwise<bf16>(p, dtype, x, w, bias, y, stream);
+    if (dtype == TANNIC_FLOAT32) return run_pointwise<float>(p, dtype, x, w, bias, y, stream);
     return TANNIC_UNSUPPORTED_DTYPE;
 }
 

@@ -533,16 +533,14 @@ int run16(const GemmProblem& p, const void* a, const void* b, void* c, hipStream
     for (int d = 0; d < p.batch_rank; ++d)
         if (!mult8(p.a_bs[d]) || !mult8(p.b_bs[d])) return TANNIC_UNSUPPORTED_DTYPE;
     if (p.batches > 65535) return TANNIC_UNSUPPORTED_DTYPE;
-    // large tiles when they still give every CU work, smaller ones otherwise
+    // Tile height by M (a tile taller than M multiplies padding), large tiles only when they still give every CU work.
     const uint64_t big = static_cast<uint64_t>((p.M + 255) / 256) * ((p.N + 255) / 256) * p.batches;
-    if (big >= 200) return pick_layout16<T, 256, 256, 2>(p, ak, bk, a, b, c, stream);
-    const uint64_t mid = static_cast<uint64_t>((p.M + 127) / 128) * ((p.N + 127) / 128) * p.batches;
-    if (mid >= 200) return pick_layout16<T, 128, 128, 2>(p, ak, bk, a, b, c, stream);
-    // too few tiles for the chip: a share of K per block while a block keeps four steps.  Tiles as tall as M allows,
-    // so that the other operand is read once.
+    if (p.M > 192 && big >= 200) return pick_layout16<T, 256, 256, 2>(p, ak, bk, a, b, c, stream);
     const bool tall = p.M > 64;
-    const uint64_t few = tall ? mid : static_cast<uint64_t>((p.M + 63) / 64) * ((p.N + 127) / 128) * p.batches;
-    uint64_t splits = few < 256 ? 256 / few : 1;
+    const uint64_t tiles = tall ? static_cast<uint64_t>((p.M + 127) / 128) * ((p.N + 127) / 128) * p.batches
+                                : static_cast<uint64_t>((p.M + 63) / 64) * ((p.N + 127) / 128) * p.batches;
+    // too few tiles for the chip: a share of K per block while a block keeps four steps
+    uint64_t splits = tiles < 256 ? 256 / tiles : 1;
     if (splits > p.K / 256) splits = p.K / 256;
     if (splits > 1 && !p.row_bias) {
         if (tall) return run16_split<T, 128>(p, ak, bk, static_cast<uint32_t>(splits), a, b, c, stream);
