@@ -241,6 +241,17 @@ int tannic_hip_view_as_cartesian(const tannic_tensor_t* re, const tannic_tensor_
 int tannic_hip_view_as_polar(const tannic_tensor_t* rho, const tannic_tensor_t* theta, tannic_tensor_t* dst, tannic_stream_t stream);
 
 /* ------------------------------------------------------------------ *
+ * Shape-changing copies     replaces src/cuda/reps.cuh:11, src/cuda/triang.cuh:11-12
+ * ------------------------------------------------------------------ */
+/* cuda::repeat(src, dst, axis, reps, stream): every index along `axis` repeated `reps` times in place
+ * (dst[.., j*reps + r, ..] = src[.., j, ..]); src strided, dst contiguous (CPU: src/cpu/reps.cpp:18-99) */
+int tannic_hip_repeat(const tannic_tensor_t* src, tannic_tensor_t* dst, tannic_stream_t stream, int axis, int reps);
+/* cuda::triu / cuda::tril: rank 2; keeps j >= i + k (upper) or j <= i + k (lower) with the sum formed in
+ * unsigned 64-bit as the CPU path forms it (src/cpu/triang.cpp:8-22, 24-105); other ranks: UNSUPPORTED_DTYPE */
+int tannic_hip_triu(const tannic_tensor_t* src, tannic_tensor_t* dst, tannic_stream_t stream, int k);
+int tannic_hip_tril(const tannic_tensor_t* src, tannic_tensor_t* dst, tannic_stream_t stream, int k);
+
+/* ------------------------------------------------------------------ *
  * Copies and checks                 replaces src/cuda/cpy.cuh:9, src/cuda/val.cuh:11
  * ------------------------------------------------------------------ */
 /* cuda::cpy: strided -> strided, size-1 dims broadcast (CPU: src/cpu/cpy.cpp:18-80) */

@@ -655,6 +655,62 @@ template <class T> int cpy_run(const tannic_tensor_t* src, tannic_tensor_t* dst)
 }
 
 /* ------------------------------------------------------------------ *
+ * repeat: interleaved repetition along one axis     src/cpu/reps.cpp:18-99
+ * dst is written in order: for every outer index, every index j of the axis, `reps` copies of the inner block
+ * ------------------------------------------------------------------ */
+template <class T> int repeat_run(const tannic_tensor_t* src, tannic_tensor_t* dst, int axis, int reps) {
+    const T* ps = static_cast<const T*>(src->address);
+    T* pd = static_cast<T*>(dst->address);
+    size_t outer = 1, inner = 1;
+    for (int d = 0; d < src->rank; ++d) {
+        if (d < axis) outer *= src->shape.sizes[d];
+        else if (d > axis) inner *= src->shape.sizes[d];
+    }
+    const size_t along = src->shape.sizes[axis];
+    for (size_t o = 0; o < outer; ++o) {
+        int64_t base = 0;
+        size_t t = o;
+        for (int d = axis - 1; d >= 0; --d) {
+            base += static_cast<int64_t>(t % src->shape.sizes[d]) * src->strides.sizes[d];
+            t /= src->shape.sizes[d];
+        }
+        for (size_t j = 0; j < along; ++j)
+            for (int r = 0; r < reps; ++r)
+                for (size_t k = 0; k < inner; ++k) {
+                    int64_t off = base + static_cast<int64_t>(j) * src->strides.sizes[axis];
+                    size_t u = k;
+                    for (int d = src->rank - 1; d > axis; --d) {
+                        off += static_cast<int64_t>(u % src->shape.sizes[d]) * src->strides.sizes[d];
+                        u /= src->shape.sizes[d];
+                    }
+                    *pd++ = ps[off];
+                }
+    }
+    return TANNIC_SUCCESS;
+}
+
+/* ------------------------------------------------------------------ *
+ * triu / tril, rank 2                      src/cpu/triang.cpp:8-105
+ * `i + k` is size_t + int: k is converted to unsigned 64-bit, so it wraps for i < -k
+ * ------------------------------------------------------------------ */
+template <class T, bool UPPER> int triangular_run(const tannic_tensor_t* src, tannic_tensor_t* dst, int k) {
+    if (src->rank != 2) return TANNIC_UNSUPPORTED_DTYPE;
+    const T* ps = static_cast<const T*>(src->address);
+    T* pd = static_cast<T*>(dst->address);
+    const size_t rows = src->shape.sizes[0], cols = src->shape.sizes[1];
+    const bool plain = src->layout == TANNIC_CONTIGUOUS;
+    for (size_t i = 0; i < rows; ++i)
+        for (size_t j = 0; j < cols; ++j) {
+            const size_t edge = i + static_cast<size_t>(static_cast<int64_t>(k));
+            const bool keep = UPPER ? j >= edge : j <= edge;
+            const int64_t os = plain ? static_cast<int64_t>(i * cols + j) : static_cast<int64_t>(i) * src->strides.sizes[0] + static_cast<int64_t>(j) * src->strides.sizes[1];
+            const int64_t od = plain ? static_cast<int64_t>(i * cols + j) : static_cast<int64_t>(i) * dst->strides.sizes[0] + static_cast<int64_t>(j) * dst->strides.sizes[1];
+            pd[od] = keep ? ps[os] : T{};
+        }
+    return TANNIC_SUCCESS;
+}
+
+/* ------------------------------------------------------------------ *
  * allclose                                src/cpu/val.cpp:17-83
  * ------------------------------------------------------------------ */
 template <class T> int allclose_run(const tannic_tensor_t* a, const tannic_tensor_t* b, double rtol, double atol) {
@@ -788,6 +844,34 @@ int oracle_cpy(const tannic_tensor_t* s, tannic_tensor_t* d) {
     int st = TANNIC_UNSUPPORTED_DTYPE;
     with_type(s->dtype, [&](auto t) { using T = typename decltype(t)::type; st = cpy_run<T>(s, d); });
     return st;
+}
+
+/* src/cpu/reps.cpp:82-97: dispatch on the destination dtype; no boolean, no complex */
+int oracle_repeat(const tannic_tensor_t* s, tannic_tensor_t* d, int axis, int reps) {
+    switch (d->dtype) {
+        case TANNIC_INT8: return repeat_run<int8_t>(s, d, axis, reps);
+        case TANNIC_INT16: case TANNIC_FLOAT16: case TANNIC_BFLOAT16: return repeat_run<uint16_t>(s, d, axis, reps);
+        case TANNIC_INT32: case TANNIC_FLOAT32: return repeat_run<uint32_t>(s, d, axis, reps);
+        case TANNIC_INT64: case TANNIC_FLOAT64: return repeat_run<uint64_t>(s, d, axis, reps);
+        default: return TANNIC_UNSUPPORTED_DTYPE;
+    }
+}
+/* src/cpu/triang.cpp:75-103: int32, int64 and the float types */
+int oracle_triu(const tannic_tensor_t* s, tannic_tensor_t* d, int k) {
+    switch (s->dtype) {
+        case TANNIC_FLOAT16: case TANNIC_BFLOAT16: return triangular_run<uint16_t, true>(s, d, k);
+        case TANNIC_INT32: case TANNIC_FLOAT32: return triangular_run<uint32_t, true>(s, d, k);
+        case TANNIC_INT64: case TANNIC_FLOAT64: return triangular_run<uint64_t, true>(s, d, k);
+        default: return TANNIC_UNSUPPORTED_DTYPE;
+    }
+}
+int oracle_tril(const tannic_tensor_t* s, tannic_tensor_t* d, int k) {
+    switch (s->dtype) {
+        case TANNIC_FLOAT16: case TANNIC_BFLOAT16: return triangular_run<uint16_t, false>(s, d, k);
+        case TANNIC_INT32: case TANNIC_FLOAT32: return triangular_run<uint32_t, false>(s, d, k);
+        case TANNIC_INT64: case TANNIC_FLOAT64: return triangular_run<uint64_t, false>(s, d, k);
+        default: return TANNIC_UNSUPPORTED_DTYPE;
+    }
 }
 
 /* 1 close, 0 not close, -1 unsupported dtype (the reference throws, src/cpu/val.cpp:81) */

@@ -19,6 +19,8 @@
 #include "cpu/cmps.hpp"
 #include "cpu/complex.hpp"
 #include "cpu/cpy.hpp"
+#include "cpu/reps.hpp"
+#include "cpu/triang.hpp"
 #include "cpu/val.hpp"
 
 static_assert(sizeof(tensor_t) == 176 && offsetof(tensor_t, rank) == 8 && offsetof(tensor_t, shape) == 16 &&
@@ -50,6 +52,9 @@ int ref_conv2d_biased(const tensor_t* x, const tensor_t* w, const tensor_t* b, t
     return cpu::conv2d(x, w, b, y, pad, stride);
 }
 int ref_cpy(const tensor_t* s, tensor_t* d) { return cpu::cpy(s, d); }
+int ref_repeat(const tensor_t* s, tensor_t* d, int axis, int reps) { return cpu::repeat(s, d, axis, reps); }
+int ref_triu(const tensor_t* s, tensor_t* d, int k) { return cpu::triu(s, d, k); }
+int ref_tril(const tensor_t* s, tensor_t* d, int k) { return cpu::tril(s, d, k); }
 int ref_allclose(const tensor_t* a, const tensor_t* b, double rtol, double atol) {
     try { return cpu::allclose(a, b, rtol, atol) ? 1 : 0; } catch (...) { return -1; }
 }

@@ -109,6 +109,9 @@ def kernel_signatures(with_stream):
     for n in REDUCE_OPS:
         sig[n] = (C.c_int, [TP, TP] + s + [C.c_uint8])
     sig["cpy"] = (C.c_int, [TP, TP] + s)
+    sig["repeat"] = (C.c_int, [TP, TP] + s + [C.c_int, C.c_int])
+    sig["triu"] = (C.c_int, [TP, TP] + s + [C.c_int])
+    sig["tril"] = (C.c_int, [TP, TP] + s + [C.c_int])
     sig["allclose"] = (C.c_int, [TP, TP] + s + [C.c_double, C.c_double])
     sig["conv2d"] = (C.c_int, [TP, TP, TP] + s + [SIZE2, SIZE2])
     sig["conv2d_biased"] = (C.c_int, [TP, TP, TP, TP] + s + [SIZE2, SIZE2])

@@ -35,6 +35,7 @@ UNITS = [
     ("binary.hip", "binary_pow.o", EXACT + ["-DTH_BINARY_ONLY=3"]),
     ("misc.hip", "misc.o", EXACT),
     ("reduce.hip", "reduce.o", []),
+    ("shape_ops.hip", "shape_ops.o", []),
     ("gemm.hip", "gemm.o", []),
     ("gemm_mfma.hip", "gemm_mfma.o", []),
     ("gemm_skinny.hip", "gemm_skinny.o", []),

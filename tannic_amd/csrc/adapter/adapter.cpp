@@ -106,10 +106,10 @@ bool allclose(const tensor_t* a, const tensor_t* b, stream_t q, double rtol, dou
 
 status conv1d(const tensor_t*, const tensor_t*, tensor_t*, stream_t, const size_t, const size_t) { return UNSUPPORTED_DTYPE; }
 status outer(const tensor_t*, const tensor_t*, tensor_t*, stream_t) { return UNSUPPORTED_DTYPE; }
-status repeat(const tensor_t*, tensor_t*, int, int, stream_t) { return UNSUPPORTED_DTYPE; }
+status repeat(const tensor_t* s, tensor_t* d, int axis, int reps, stream_t q) { return static_cast<status>(tannic_hip_repeat(in(s), out(d), st(q), axis, reps)); }
 status concat(const tensor_t*, const tensor_t*, tensor_t*, stream_t, int) { return UNSUPPORTED_DTYPE; }
-status triu(const tensor_t*, tensor_t*, stream_t, int) { return UNSUPPORTED_DTYPE; }
-status tril(const tensor_t*, tensor_t*, stream_t, int) { return UNSUPPORTED_DTYPE; }
+status triu(const tensor_t* s, tensor_t* d, stream_t q, int k) { return static_cast<status>(tannic_hip_triu(in(s), out(d), st(q), k)); }
+status tril(const tensor_t* s, tensor_t* d, stream_t q, int k) { return static_cast<status>(tannic_hip_tril(in(s), out(d), st(q), k)); }
 
 }  // namespace cuda
 

@@ -347,6 +347,37 @@ def convolve2d(signal, kernel, bias=None, stride=1, padding=0):
 
 
 # ---- copies and checks ---------------------------------------------------
+def repeat(x, repeats, axis=0):
+    """``repeat(source, repeats, axis)``: every index along ``axis`` ``repeats`` times in place
+    (``include/tannic/transformations.hpp:221-240, 325-329``; kernel ``src/cpu/reps.cpp:18-54``)."""
+    axis = axis + x.rank if axis < 0 else axis
+    if not 0 <= axis < x.rank:
+        raise TannicError("repeat: axis out of range")
+    shape = list(x.shape)
+    shape[axis] *= repeats
+    env = _resolve(x)
+    dst = Tensor(x.dtype, tuple(shape)).initialize(env)
+    _call("repeat", env, [x], dst, (C.c_int(axis), C.c_int(repeats)))
+    return dst
+
+
+def _triangular(name, x, k):
+    env = _resolve(x)
+    dst = Tensor(x.dtype, x.shape).initialize(env)
+    _call(name, env, [x], dst, (C.c_int(k),))
+    return dst
+
+
+def triu(x, k=0):
+    """``triangular(x, Position::Upper, k)`` (``include/tannic/filter.hpp:63-76``, ``src/filter.cpp:20-37``)."""
+    return _triangular("triu", x, k)
+
+
+def tril(x, k=0):
+    """``triangular(x, Position::Lower, k)`` (``include/tannic/filter.hpp:63-76``, ``src/filter.cpp:20-37``)."""
+    return _triangular("tril", x, k)
+
+
 def copy_into(dst, src):
     """``slice = expr``: strided copy into an existing view (``include/tannic/tensor.hpp:447-456``)."""
     return _call("cpy", _resolve(dst, src), [src], dst)

@@ -24,6 +24,8 @@ def build(spec, env):
     t = ta.tensor(np.array(spec["data"], dtype=np.float64).reshape(spec["shape"]), dtype, env)
     if "transpose" in spec:
         t = t.transpose(*spec["transpose"])
+    if "permute" in spec:
+        t = t.permute(*spec["permute"])
     return t
 
 
@@ -64,6 +66,8 @@ def run(case, env):
         out = getattr(ops, op)(ins[0], case["axis"], case.get("keepdim", False))
     elif op == "mean_sq":
         out = ops.mean(ops.mul(ins[0], ins[0]), case["axis"])
+    elif op == "repeat":
+        out = ops.repeat(ins[0], case["repeats"], case["axis"])
     elif op == "polar":
         out = ops.realify(ops.polar(ins[0], ins[1]))
     else:

@@ -192,3 +192,35 @@ def test_polar_has_the_radius_as_modulus(oracle):
     z0 = ops.polar(support.host_tensor(rho, ta.float32), support.host_tensor(np.zeros((6, 5)), ta.float32)).numpy()
     support.assert_bit_exact(z0.real, rho, "theta = 0")
     assert (z0.imag == 0).all()
+
+
+# ---- repeat, triu, tril against numpy ---------------------------------------------------------------------------
+@pytest.mark.parametrize("axis", [0, 1, 2])
+def test_repeat_is_numpy_repeat(oracle, axis):
+    x = support.values_for(ta.float32, 5, 41, (3, 4, 5), -2, 2)
+    with support.use_functions(oracle):
+        got = ops.repeat(support.host_tensor(x, ta.float32).transpose(0, 2).transpose(0, 2), 3, axis).numpy()
+    np.testing.assert_array_equal(got, np.repeat(x, 3, axis=axis))
+
+
+@pytest.mark.parametrize("k", [0, 1, 2, 5])
+def test_triangular_is_numpy_for_non_negative_offsets(oracle, k):
+    x = support.values_for(ta.float64, 5, 42, (6, 4), 1, 2)
+    with support.use_functions(oracle):
+        up = ops.triu(support.host_tensor(x, ta.float64), k).numpy()
+        lo = ops.tril(support.host_tensor(x, ta.float64), k).numpy()
+    np.testing.assert_array_equal(up, np.triu(x, k))
+    np.testing.assert_array_equal(lo, np.tril(x, k))
+
+
+def test_triangular_negative_offset_wraps_for_the_first_rows(oracle):
+    # i + k is formed in unsigned arithmetic (src/cpu/triang.cpp:12,20): for i < -k the edge is huge,
+    # so triu clears those rows and tril keeps them whole; from row -k on both agree with numpy
+    x = support.values_for(ta.float32, 5, 43, (5, 5), 1, 2)
+    with support.use_functions(oracle):
+        up = ops.triu(support.host_tensor(x, ta.float32), -2).numpy()
+        lo = ops.tril(support.host_tensor(x, ta.float32), -2).numpy()
+    assert not up[:2].any()
+    np.testing.assert_array_equal(up[2:], np.triu(x, -2)[2:])
+    np.testing.assert_array_equal(lo[:2], x[:2])
+    np.testing.assert_array_equal(lo[2:], np.tril(x, -2)[2:])

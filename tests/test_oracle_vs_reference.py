@@ -251,3 +251,44 @@ def test_allclose(oracle, reference):
             assert ops.allclose(a, n) is True  # NaN differences never trip the test
             with pytest.raises(ta.TannicError):
                 ops.allclose(make(ta.int32, 28, (2,)), make(ta.int32, 28, (2,)))
+
+
+REPEAT_VIEWS = {
+    "plain": ((2, 3, 4), []),
+    "permuted": ((2, 3, 4), [("permute", (2, 0, 1))]),
+    "sliced": ((4, 6, 5), [("index", (slice(0, 4, 2), slice(1, 6, 2), slice(0, 5, 1)))]),
+    "expanded": ((1, 3, 1), [("expand", (2, 3, 4))]),
+    "vector": ((5,), []),
+}
+
+
+@pytest.mark.parametrize("axis", [0, 1, 2, -1])
+@pytest.mark.parametrize("view", list(REPEAT_VIEWS))
+@pytest.mark.parametrize("dtype", INTS + REALS, ids=str)
+def test_repeat(oracle, reference, dtype, view, axis):
+    shape, spec = REPEAT_VIEWS[view]
+    x = support.apply_view(make(dtype, 31, shape), spec)
+    if axis >= x.rank:
+        pytest.skip("axis beyond the rank")
+    check(oracle, reference, lambda: ops.repeat(x, 3, axis), f"repeat {dtype} {view} axis {axis}")
+
+
+@pytest.mark.parametrize("k", [0, 1, 3, -1, -2, 7, -7])
+@pytest.mark.parametrize("view", ["plain", "transposed", "sliced"])
+@pytest.mark.parametrize("op", ["triu", "tril"])
+@pytest.mark.parametrize("dtype", [ta.int32, ta.int64] + REALS, ids=str)
+def test_triangular(oracle, reference, dtype, op, view, k):
+    x = make(dtype, 32, (5, 6))
+    if view == "transposed":
+        x = x.transpose(0, 1)
+    elif view == "sliced":
+        x = x[1:5, 0:6:2]
+    check(oracle, reference, lambda: getattr(ops, op)(x, k), f"{op} {dtype} {view} k={k}")
+
+
+def test_triangular_rejects_other_ranks(oracle, reference):
+    x = make(ta.float32, 33, (2, 3, 4))
+    for lib in (oracle, reference):
+        with support.use_functions(lib):
+            with pytest.raises(ops.TannicError):
+                ops.triu(x, 0)
