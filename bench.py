@@ -15,8 +15,9 @@ The same line carries
   cpu_baseline  the CPU restatement of the reference's gemm (one core, as the
                 reference is single threaded) timed on a bounded sample;
   workloads     the other configurations: GEMM sweep, conv2d layers, the
-                elementwise ops of the broadcast chain and the axis reductions,
-                each with its own roofline fraction.
+                elementwise ops of the broadcast chain, the axis reductions and
+                the decoder layer composed from the operators, each with its own
+                roofline fraction.
 """
 import argparse
 import ctypes as C
@@ -55,6 +56,8 @@ def parse():
     ap.add_argument("--primary-only", action="store_true", help="skip the secondary workloads and the CPU baseline")
     ap.add_argument("--copy-only", action="store_true",
                     help="run only a plain 1 GiB -> 1 GiB contiguous copy (repack): the known-size kernel that calibrates the HBM byte counters")
+    ap.add_argument("--only", choices=["gemm", "conv", "elementwise", "reduce", "layer"],
+                    help="run one group of the secondary workloads alone and print its entries (for profiling that group)")
     return ap.parse_args()
 
 
@@ -123,10 +126,53 @@ def gemm_entry(b, dtype, M, N, K, iters):
     flops = 2.0 * M * N * K
     nbytes = (M * K + N * K + M * N) * dtype.itemsize
     tflops, gbs = flops / ms / 1e9, nbytes / ms / 1e6
-    hbm_bound = flops / nbytes < 312.0   # below the ridge of 2.5 PFLOP/s over 8 TB/s
+    peak = MFMA_PEAK_TFLOPS["f32" if dtype is ta.float32 else "f16"]
+    hbm_bound = flops / nbytes < peak * 1e3 / HBM_PEAK_GBS   # below the ridge of the matrix peak over 8 TB/s
     return {"op": f"gemm {dtype} X[{M},{K}].W[{N},{K}]^T", "us": round(ms * 1e3, 2), "tflops": round(tflops, 2), "gbs": round(gbs, 1),
             "bound": "hbm" if hbm_bound else "mfma",
-            "frac": round(gbs / HBM_PEAK_GBS if hbm_bound else tflops / MFMA_PEAK_TFLOPS["f16"], 4)}
+            "frac": round(gbs / HBM_PEAK_GBS if hbm_bound else tflops / peak, 4)}
+
+
+def measured_value(name, key):
+    """A number recorded in a committed profile summary under profiles/ (None if absent)."""
+    try:
+        for line in open(os.path.join(ROOT, "profiles", name)):
+            if line.strip().startswith(key):
+                return float(line.split("=")[1])
+    except OSError:
+        pass
+    return None
+
+
+def decoder_layer_entry(b, iters):
+    """One Llama-3-8B decoder layer, seq 512, bf16, written with the operators (about 65 backend calls).
+    The time is wall-clock through this Python front end, which is what bounds it; the device-busy time of the
+    same calls comes from the committed kernel trace."""
+    from tannic_amd import decoder_layer as dl
+    import support
+    ta = b.ta
+    s, seq, dtype = dl.LayerShape(), 512, ta.bfloat16
+    w = {}
+    for i, (name, shape) in enumerate(dl.weight_shapes(s).items()):
+        w[name] = ta.tensor(np.ones(shape), dtype, b.device) if name.startswith("g") else b.filled(dtype, shape, "normal", 0, 40 + i, 0.02)
+    x = b.filled(dtype, (1, seq, s.hidden), "normal", 0, 39, 1.0)
+    cos, sin = dl.rotary_tables(s, seq, dtype, b.device)
+    mask, one = dl.causal_mask(seq, dtype, b.device), ta.tensor(np.ones(1), dtype, b.device)
+    for _ in range(2):
+        dl.forward(s, w, x, cos, sin, mask, one)
+    b.sync()
+    t0 = time.perf_counter()
+    for _ in range(iters):
+        out = dl.forward(s, w, x, cos, sin, mask, one)
+    b.sync()
+    us = (time.perf_counter() - t0) / iters * 1e6
+    flops = dl.flop_count(s, seq)
+    busy = measured_value("decoder_layer_bf16_seq512_kernels.txt", "device_busy_us_per_layer")
+    del out
+    return {"op": "decoder layer bfloat16 seq 512 (hidden 4096, 32/8 heads, FFN 14336), composed from operators", "us": round(us, 1),
+            "tflops": round(flops / us / 1e6, 2), "mfma_frac": round(flops / us / 1e6 / MFMA_PEAK_TFLOPS["bf16"], 4),
+            "bound": "host front end (one Python call per operator)", "device_busy_us": busy,
+            "device_busy_tflops": round(flops / busy / 1e6, 2) if busy else None}
 
 
 def conv_entry(b, dtype, name, xs, ws, stride, pad, iters):
@@ -214,6 +260,32 @@ def cpu_baseline(rows=64):
             "sample": f"first {rows} rows of X: [{rows},4096] . [4096,4096]^T fp16, fp32 accumulate, {dt:.1f} s of {os.cpu_count()} host CPUs' one core"}
 
 
+def secondary(b, only):
+    """Entries of the secondary workloads; `only` names one group or None for all."""
+    ta = b.ta
+    work = []
+    if only in (None, "gemm"):
+        for (m, n) in [(2048, 4096), (2048, 14336), (128, 4096), (128, 14336), (16, 4096), (16, 14336), (1, 4096), (1, 14336)]:
+            work.append(gemm_entry(b, ta.float16, m, n, 4096, 20))
+        work.append(gemm_entry(b, ta.bfloat16, 4096, 4096, 4096, 20))
+        work.append(gemm_entry(b, ta.float32, 512, 512, 512, 20))
+        work.append(gemm_entry(b, ta.float32, 4096, 4096, 4096, 5))
+    if only in (None, "conv"):
+        for dtype in (ta.float16, ta.bfloat16, ta.float32):
+            work.append(conv_entry(b, dtype, "3->64 k7 s2 p3 @224 N=32", (32, 3, 224, 224), (64, 3, 7, 7), 2, 3, 5))
+            work.append(conv_entry(b, dtype, "64->64 k3 s1 p1 @56 N=32", (32, 64, 56, 56), (64, 64, 3, 3), 1, 1, 5))
+            work.append(conv_entry(b, dtype, "256->512 k1 s2 @56 N=32", (32, 256, 56, 56), (512, 256, 1, 1), 2, 0, 5))
+    if only in (None, "elementwise"):
+        for dtype in (ta.float32, ta.float16, ta.int32):
+            work += elementwise_entries(b, dtype, 10)
+    if only in (None, "reduce"):
+        for dtype in (ta.float32, ta.float16):
+            work += reduction_entries(b, dtype, 10)
+    if only in (None, "layer"):
+        work.append(decoder_layer_entry(b, 5))
+    return work
+
+
 def main():
     args = parse()
     if args.gpus != 1:
@@ -228,6 +300,9 @@ def main():
         ms = b.event_time(b.raw_call("repack", [src], dst), args.steps)
         print(json.dumps({"op": "repack float32 [64,4096,1024]", "bytes_read": src.nbytes, "bytes_written": dst.nbytes,
                           "us": round(ms * 1e3, 1), "gbs": round(2 * src.nbytes / ms / 1e6, 1)}))
+        return
+    if args.only:
+        print(json.dumps({"workloads": secondary(b, args.only)}))
         return
     M = N = K = 4096
     x = b.filled(ta.float16, (M, K), "normal", 0, 1, 1.0)
@@ -271,19 +346,7 @@ def main():
     del x, w, wt
 
     if not args.primary_only:
-        work = []
-        for (m, n) in [(2048, 4096), (2048, 14336), (128, 4096), (128, 14336), (16, 4096), (16, 14336), (1, 4096), (1, 14336)]:
-            work.append(gemm_entry(b, ta.float16, m, n, 4096, 20))
-        work.append(gemm_entry(b, ta.bfloat16, 4096, 4096, 4096, 20))
-        for dtype in (ta.float16, ta.float32):
-            work.append(conv_entry(b, dtype, "3->64 k7 s2 p3 @224 N=32", (32, 3, 224, 224), (64, 3, 7, 7), 2, 3, 5))
-            work.append(conv_entry(b, dtype, "64->64 k3 s1 p1 @56 N=32", (32, 64, 56, 56), (64, 64, 3, 3), 1, 1, 5))
-            work.append(conv_entry(b, dtype, "256->512 k1 s2 @56 N=32", (32, 256, 56, 56), (512, 256, 1, 1), 2, 0, 5))
-        for dtype in (ta.float32, ta.float16, ta.int32):
-            work += elementwise_entries(b, dtype, 10)
-        for dtype in (ta.float32, ta.float16):
-            work += reduction_entries(b, dtype, 10)
-        result["workloads"] = work
+        result["workloads"] = secondary(b, None)
         result["cpu_baseline"] = cpu_baseline()
     print(json.dumps(result))
 
