@@ -91,6 +91,20 @@ template <class D, class X> __host__ __device__ inline D narrow(X x) {
     else return static_cast<D>(x);
 }
 
+// narrow_result<D>(x): the rounding of an fp32 accumulator in the matrix kernels.  bf16 uses the hardware's
+// round-to-nearest-even conversion there (the bit-level routine above stays for the elementwise kernels, whose
+// results are compared bit for bit, NaN payloads included).
+template <class D> __device__ inline D narrow_result(float x) {
+    if constexpr (std::is_same_v<D, bf16>) {
+        const __bf16 h = static_cast<__bf16>(x);
+        bf16 r;
+        __builtin_memcpy(&r.bits, &h, 2);
+        return r;
+    } else {
+        return static_cast<D>(x);
+    }
+}
+
 template <class T> struct type_tag { using type = T; };
 
 // Calls f(type_tag<T>{}) for the element type of a dtype code.

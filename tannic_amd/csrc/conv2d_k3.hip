@@ -276,7 +276,7 @@ __global__ __launch_bounds__(kK3Threads) void conv2d_k3_kernel(const T* x, const
             for (int g = 0; g < 4; ++g) {
                 T r[4];
 #pragma unroll
-                for (int e = 0; e < 4; ++e) r[e] = narrow<T>(acc[i][j][g * 4 + e]);
+                for (int e = 0; e < 4; ++e) r[e] = narrow_result<T>(acc[i][j][g * 4 + e]);
                 uint2 bits;
                 __builtin_memcpy(&bits, r, 8);
                 *reinterpret_cast<uint2*>(out + (i * 32 + lane % 32) * PITCH + (wave + 4 * j) * 32 + g * 8 + 4 * (lane / 32)) = bits;

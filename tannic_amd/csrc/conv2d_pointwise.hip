@@ -12,8 +12,9 @@
 
 namespace th {
 
-// out[row][ow] = x[n][c][oh * stride_h][ow * stride_w], row = (n * C + c) * HO + oh; four outputs per thread
-template <class T>
+// out[row][ow] = x[n][c][oh * stride_h][ow * stride_w], row = (n * C + c) * HO + oh; four outputs per thread.
+// PAIRS: horizontal stride 2 over contiguous, aligned rows: the eight columns the four outputs come from are one load.
+template <class T, bool PAIRS>
 __global__ __launch_bounds__(256) void conv_subsample4_kernel(const T* x, T* out, ConvProblem p, FastDiv div_quads, FastDiv div_ho, FastDiv div_c, uint32_t total) {
     const uint32_t idx = blockIdx.x * 256 + threadIdx.x;
     if (idx >= total) return;
@@ -24,8 +25,17 @@ __global__ __launch_bounds__(256) void conv_subsample4_kernel(const T* x, T* out
     const T* src = x + static_cast<int64_t>(n) * p.xs[0] + static_cast<int64_t>(c) * p.xs[1] + static_cast<int64_t>(oh * p.stride_h) * p.xs[2] +
                    static_cast<int64_t>(quad * 4 * p.stride_w) * p.xs[3];
     T v[4];
+    if constexpr (PAIRS) {
+        using Eight = std::conditional_t<sizeof(T) == 2, uint4, ulonglong4>;
+        T in[8];
+        const Eight bits8 = *reinterpret_cast<const Eight*>(src);
+        __builtin_memcpy(in, &bits8, sizeof(Eight));
 #pragma unroll
-    for (int e = 0; e < 4; ++e) v[e] = src[static_cast<int64_t>(e * p.stride_w) * p.xs[3]];
+        for (int e = 0; e < 4; ++e) v[e] = in[2 * e];
+    } else {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) v[e] = src[static_cast<int64_t>(e * p.stride_w) * p.xs[3]];
+    }
     using Quad = std::conditional_t<sizeof(T) == 2, uint2, uint4>;
     Quad bits;
     __builtin_memcpy(&bits, v, sizeof(Quad));
@@ -79,8 +89,16 @@ int run_pointwise(const ConvProblem& p, int dtype, const void* x, const void* w,
     if (quads >= (1ull << 31)) return TANNIC_UNSUPPORTED_DTYPE;
     T* dense_x = nullptr;
     if (scratch_acquire(reinterpret_cast<void**>(&dense_x), rows * p.WO * sizeof(T), stream) != TANNIC_SUCCESS) return TANNIC_ERROR;
-    hipLaunchKernelGGL((conv_subsample4_kernel<T>), dim3((quads + 255) / 256), dim3(256), 0, stream, static_cast<const T*>(x), dense_x, p, FastDiv(p.WO / 4),
-                       FastDiv(p.HO), FastDiv(p.C), static_cast<uint32_t>(quads));
+    // eight source columns per thread in one load: they must exist (the last group may reach one column past the last
+    // sampled one) and start at a multiple of the load size
+    const bool pairs = p.stride_w == 2 && p.xs[3] == 1 && static_cast<uint64_t>(p.WO) * 2 <= p.W && p.xs[2] % 8 == 0 &&
+                       p.xs[1] % 8 == 0 && p.xs[0] % 8 == 0 && reinterpret_cast<uintptr_t>(x) % (8 * sizeof(T)) == 0;
+    if (pairs)
+        hipLaunchKernelGGL((conv_subsample4_kernel<T, true>), dim3((quads + 255) / 256), dim3(256), 0, stream, static_cast<const T*>(x), dense_x, p, FastDiv(p.WO / 4),
+                           FastDiv(p.HO), FastDiv(p.C), static_cast<uint32_t>(quads));
+    else
+        hipLaunchKernelGGL((conv_subsample4_kernel<T, false>), dim3((quads + 255) / 256), dim3(256), 0, stream, static_cast<const T*>(x), dense_x, p, FastDiv(p.WO / 4),
+                           FastDiv(p.HO), FastDiv(p.C), static_cast<uint32_t>(quads));
     int status = launch_status("conv_subsample4_kernel");
     if (status == TANNIC_SUCCESS) {
         g.b_rs = static_cast<int64_t>(pixels);

@@ -243,7 +243,7 @@ __global__ __launch_bounds__(kStemThreads, 2) void conv2d_stem_kernel(const T* x
             for (int g = 0; g < 4; ++g) {
                 T r[4];
 #pragma unroll
-                for (int e = 0; e < 4; ++e) r[e] = narrow<T>(acc[i][g * 4 + e]);
+                for (int e = 0; e < 4; ++e) r[e] = narrow_result<T>(acc[i][g * 4 + e]);
                 uint2 bits;
                 __builtin_memcpy(&bits, r, 8);
                 *reinterpret_cast<uint2*>(out + (i * 32 + lane % 32) * kStemOutPitch + wave * 32 + g * 8 + 4 * (lane / 32)) = bits;

@@ -416,7 +416,7 @@ __global__ __launch_bounds__(128 * WAVES_N) void gemm16_kernel(const T* A, const
                 for (int g = 0; g < 4; ++g) {
                     T out[4];
 #pragma unroll
-                    for (int e = 0; e < 4; ++e) out[e] = narrow<T>(acc[i][j][g * 4 + e]);
+                    for (int e = 0; e < 4; ++e) out[e] = narrow_result<T>(acc[i][j][g * 4 + e]);
                     uint2 bits;
                     __builtin_memcpy(&bits, out, 8);
                     *reinterpret_cast<uint2*>(stage + (i * 32 + lane % 32) * PITCH + j * 32 + g * 8 + 4 * (lane / 32)) = bits;
@@ -439,7 +439,7 @@ __global__ __launch_bounds__(128 * WAVES_N) void gemm16_kernel(const T* A, const
 #pragma unroll
                 for (int v = 0; v < 16; ++v) {
                     const uint32_t col = n0 + wn + j * 32 + 8 * (v / 4) + 4 * (lane / 32) + v % 4;
-                    if (row < p.M && col < p.N) c[static_cast<int64_t>(row) * p.c_rs + col] = narrow<T>(acc[i][j][v]);
+                    if (row < p.M && col < p.N) c[static_cast<int64_t>(row) * p.c_rs + col] = narrow_result<T>(acc[i][j][v]);
                 }
         }
     }
@@ -487,7 +487,7 @@ __global__ __launch_bounds__(256) void gemm_split_reduce_kernel(const float* par
     int64_t oa, ob, oc;
     batch_offsets(p, batch, oa, ob, oc);
     T* dst = C + oc + static_cast<int64_t>(m) * p.c_rs + col;
-    for (uint32_t e = 0; e < live; ++e) dst[e] = narrow<T>(sum[e]);
+    for (uint32_t e = 0; e < live; ++e) dst[e] = narrow_result<T>(sum[e]);
 }
 
 // Few tiles and a long K: each tile is shared by `splits` blocks.

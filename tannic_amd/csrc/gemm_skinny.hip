@@ -95,7 +95,7 @@ __global__ __launch_bounds__(64 * kSkinnyWaves) void gemm_skinny_kernel(const T*
         if (m >= p.M) continue;
         T out[4];
 #pragma unroll
-        for (int e = 0; e < 4; ++e) out[e] = narrow<T>(sum[e]);
+        for (int e = 0; e < 4; ++e) out[e] = narrow_result<T>(sum[e]);
         T* dst = cb + static_cast<int64_t>(m) * p.c_rs + col;
         if (vector_ok) {
             if (col < p.N) {
