@@ -282,6 +282,9 @@ int tannic_hip_min(const tannic_tensor_t* src, tannic_tensor_t* dst, tannic_stre
  * ------------------------------------------------------------------ */
 int tannic_hip_gemm(const tannic_tensor_t* a, const tannic_tensor_t* b, tannic_tensor_t* dst, tannic_stream_t stream);
 
+/* cuda::conv1d(x, w, y, stream, pad, stride): x[N,C,L], w[O,C,K], y[N,O,(L+2*pad-K)/stride+1]; ERROR on rank != 3 or
+ * shape mismatch; same dtype for signal and kernel (src/cuda/conv.cuh:11; CPU: src/cpu/conv1d.cpp:17-125) */
+int tannic_hip_conv1d(const tannic_tensor_t* x, const tannic_tensor_t* w, tannic_tensor_t* y, tannic_stream_t stream, size_t pad, size_t stride);
 /* ------------------------------------------------------------------ *
  * Convolution                       replaces src/cuda/conv.cuh:12-13
  *                                   (CPU: src/cpu/conv2d.cpp:116-265)

@@ -837,6 +837,31 @@ int oracle_conv2d_biased(const tannic_tensor_t* x, const tannic_tensor_t* w, con
     return conv2d_dispatch(x, w, b, y, pad, stride);
 }
 
+/* src/cpu/conv1d.cpp:17-125: the loops of conv2d with one row (batch, channel out, position; then channel in, tap),
+ * accumulator of the operands' own type, rank 3 required */
+int oracle_conv1d(const tannic_tensor_t* x, const tannic_tensor_t* w, tannic_tensor_t* y, size_t pad, size_t stride) {
+    if (x->dtype != w->dtype) return TANNIC_UNSUPPORTED_DTYPE;
+    switch (x->dtype) {
+        case TANNIC_INT8: case TANNIC_INT16: case TANNIC_INT32: case TANNIC_INT64:
+        case TANNIC_FLOAT16: case TANNIC_BFLOAT16: case TANNIC_FLOAT32: case TANNIC_FLOAT64: break;
+        default: return TANNIC_UNSUPPORTED_DTYPE;
+    }
+    if (x->rank != 3 || w->rank != 3 || y->rank != 3) return TANNIC_ERROR;
+    auto with_row = [](const tannic_tensor_t* t) {
+        tannic_tensor_t r = *t;
+        r.rank = 4;
+        r.shape.sizes[3] = t->shape.sizes[2];
+        r.strides.sizes[3] = t->strides.sizes[2];
+        r.shape.sizes[2] = 1;
+        r.strides.sizes[2] = 0;
+        return r;
+    };
+    const tannic_tensor_t x4 = with_row(x), w4 = with_row(w);
+    tannic_tensor_t y4 = with_row(y);
+    const size_t pad2[2] = {0, pad}, stride2[2] = {1, stride};
+    return conv2d_dispatch(&x4, &w4, nullptr, &y4, pad2, stride2);
+}
+
 int oracle_view_as_cartesian(const tannic_tensor_t* a, const tannic_tensor_t* b, tannic_tensor_t* d) { return cplx_dispatch<false>(a, b, d); }
 int oracle_view_as_polar(const tannic_tensor_t* a, const tannic_tensor_t* b, tannic_tensor_t* d) { return cplx_dispatch<true>(a, b, d); }
 

@@ -51,6 +51,7 @@ int ref_conv2d(const tensor_t* x, const tensor_t* w, tensor_t* y, const size_t p
 int ref_conv2d_biased(const tensor_t* x, const tensor_t* w, const tensor_t* b, tensor_t* y, const size_t pad[2], const size_t stride[2]) {
     return cpu::conv2d(x, w, b, y, pad, stride);
 }
+int ref_conv1d(const tensor_t* x, const tensor_t* w, tensor_t* y, size_t pad, size_t stride) { return cpu::conv1d(x, w, y, pad, stride); }
 int ref_cpy(const tensor_t* s, tensor_t* d) { return cpu::cpy(s, d); }
 int ref_repeat(const tensor_t* s, tensor_t* d, int axis, int reps) { return cpu::repeat(s, d, axis, reps); }
 int ref_triu(const tensor_t* s, tensor_t* d, int k) { return cpu::triu(s, d, k); }

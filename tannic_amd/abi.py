@@ -113,6 +113,7 @@ def kernel_signatures(with_stream):
     sig["triu"] = (C.c_int, [TP, TP] + s + [C.c_int])
     sig["tril"] = (C.c_int, [TP, TP] + s + [C.c_int])
     sig["allclose"] = (C.c_int, [TP, TP] + s + [C.c_double, C.c_double])
+    sig["conv1d"] = (C.c_int, [TP, TP, TP] + s + [C.c_size_t, C.c_size_t])
     sig["conv2d"] = (C.c_int, [TP, TP, TP] + s + [SIZE2, SIZE2])
     sig["conv2d_biased"] = (C.c_int, [TP, TP, TP, TP] + s + [SIZE2, SIZE2])
     return sig

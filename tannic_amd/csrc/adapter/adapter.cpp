@@ -104,7 +104,9 @@ bool allclose(const tensor_t* a, const tensor_t* b, stream_t q, double rtol, dou
     return r == 1;
 }
 
-status conv1d(const tensor_t*, const tensor_t*, tensor_t*, stream_t, const size_t, const size_t) { return UNSUPPORTED_DTYPE; }
+status conv1d(const tensor_t* x, const tensor_t* w, tensor_t* y, stream_t q, const size_t pad, const size_t stride) {
+    return static_cast<status>(tannic_hip_conv1d(in(x), in(w), out(y), st(q), pad, stride));
+}
 status outer(const tensor_t*, const tensor_t*, tensor_t*, stream_t) { return UNSUPPORTED_DTYPE; }
 status repeat(const tensor_t* s, tensor_t* d, int axis, int reps, stream_t q) { return static_cast<status>(tannic_hip_repeat(in(s), out(d), st(q), axis, reps)); }
 status concat(const tensor_t*, const tensor_t*, tensor_t*, stream_t, int) { return UNSUPPORTED_DTYPE; }

@@ -120,9 +120,38 @@ static int conv2d_entry(const tannic_tensor_t* x, const tannic_tensor_t* w, cons
     }
 }
 
+// conv1d (src/cpu/conv1d.cpp:17-125) is conv2d on signals one row high: x[N,C,L] as [N,C,1,L], w[O,C,K] as
+// [O,C,1,K], same loops in the same order (channel, tap), same status rules with rank 3 in place of 4.
+static int conv1d_entry(const tannic_tensor_t* x, const tannic_tensor_t* w, tannic_tensor_t* y, tannic_stream_t stream, size_t pad, size_t stride) {
+    if (!x || !w || !y) return TANNIC_ERROR;
+    if (x->dtype != w->dtype) return TANNIC_UNSUPPORTED_DTYPE;
+    switch (x->dtype) {
+        case TANNIC_INT8: case TANNIC_INT16: case TANNIC_INT32: case TANNIC_INT64:
+        case TANNIC_FLOAT16: case TANNIC_BFLOAT16: case TANNIC_FLOAT32: case TANNIC_FLOAT64: break;
+        default: return TANNIC_UNSUPPORTED_DTYPE;
+    }
+    if (x->rank != 3 || w->rank != 3 || y->rank != 3) return TANNIC_ERROR;
+    auto with_row = [](const tannic_tensor_t* t) {
+        tannic_tensor_t r = *t;
+        r.rank = 4;
+        r.shape.sizes[3] = t->shape.sizes[2];
+        r.strides.sizes[3] = t->strides.sizes[2];
+        r.shape.sizes[2] = 1;
+        r.strides.sizes[2] = static_cast<int64_t>(t->shape.sizes[2]) * t->strides.sizes[2];
+        return r;
+    };
+    const tannic_tensor_t x4 = with_row(x), w4 = with_row(w);
+    tannic_tensor_t y4 = with_row(y);
+    const size_t pad2[2] = {0, pad}, stride2[2] = {1, stride};
+    return conv2d_entry(&x4, &w4, nullptr, &y4, stream, pad2, stride2);
+}
+
 }  // namespace th
 
 extern "C" {
+int tannic_hip_conv1d(const tannic_tensor_t* x, const tannic_tensor_t* w, tannic_tensor_t* y, tannic_stream_t stream, size_t pad, size_t stride) {
+    return th::conv1d_entry(x, w, y, stream, pad, stride);
+}
 int tannic_hip_conv2d(const tannic_tensor_t* x, const tannic_tensor_t* w, tannic_tensor_t* y, tannic_stream_t stream,
                       const size_t pad[2], const size_t stride[2]) {
     return th::conv2d_entry(x, w, nullptr, y, stream, pad, stride);

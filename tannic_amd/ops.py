@@ -346,6 +346,23 @@ def convolve2d(signal, kernel, bias=None, stride=1, padding=0):
     return _call("conv2d_biased" if bias is not None else "conv2d", env, operands, _new(signal.dtype, shape, env), extra=extra)
 
 
+def convolve1d(signal, kernel, stride=1, padding=0):
+    """``convolve1D(signal, kernel, stride, padding)`` (``include/tannic/convolutions.hpp:38-68, 135-145``)."""
+    if stride == 0:
+        raise TannicError("Stride must be non-zero for Conv1D.")
+    if signal.dtype is not kernel.dtype:
+        raise TannicError("Dtypes must match in convolutions.")
+    if signal.rank != 3 or kernel.rank != 3:
+        raise TannicError("Only rank 3 tensors supported for Conv1D.")
+    n, c_in, length = signal.shape
+    c_out, k_in, k_len = kernel.shape
+    if c_in != k_in:
+        raise TannicError("Input channels must match kernel channels.")
+    shape = (n, c_out, (length + 2 * padding - k_len) // stride + 1)
+    env = _resolve(signal, kernel)
+    return _call("conv1d", env, [signal, kernel], _new(signal.dtype, shape, env), extra=(C.c_size_t(padding), C.c_size_t(stride)))
+
+
 # ---- copies and checks ---------------------------------------------------
 def repeat(x, repeats, axis=0):
     """``repeat(source, repeats, axis)``: every index along ``axis`` ``repeats`` times in place

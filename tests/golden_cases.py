@@ -66,6 +66,8 @@ def run(case, env):
         out = getattr(ops, op)(ins[0], case["axis"], case.get("keepdim", False))
     elif op == "mean_sq":
         out = ops.mean(ops.mul(ins[0], ins[0]), case["axis"])
+    elif op == "conv1d":
+        out = ops.convolve1d(ins[0], ins[1], case["stride"], case["padding"])
     elif op == "repeat":
         out = ops.repeat(ins[0], case["repeats"], case["axis"])
     elif op == "polar":

@@ -134,3 +134,39 @@ def test_conv1x1_equals_gemm_on_device(device):
     _, weights = support.both(w.reshape(24, 32), ta.float16, device)
     gemm = ops.matmul(pixels, weights.transpose()).numpy().reshape(2, 6, 6, 24).transpose(0, 3, 1, 2)
     support.assert_close(conv, gemm, 2e-3, 1e-3, "1x1 conv vs gemm")
+
+
+# ---- conv1d: the one-row case of the same kernels -------------------------------------------------------------------
+CONV1D_GOLDEN = [c for c in golden_cases.TENSOR_CASES if c["op"] == "conv1d"]
+CASES_1D = {
+    "plain": ((2, 3, 17), (4, 3, 5), 1, 0),
+    "stride_pad": ((1, 2, 20), (3, 2, 4), 3, 2),
+    "few_channels_even_stride": ((2, 3, 64), (20, 3, 7), 2, 3),
+    "pointwise": ((2, 64, 40), (48, 64, 1), 1, 0),
+    "many_channels": ((1, 96, 24), (40, 96, 3), 1, 1),
+}
+
+
+@pytest.mark.parametrize("case", CONV1D_GOLDEN, ids=lambda c: c["name"])
+def test_conv1d_reference_vectors_on_device(device, case):
+    got = golden_cases.run(case, device)
+    support.assert_close(got, golden_cases.expected_of(case), 1e-5, 1e-8, case["name"])
+
+
+@pytest.mark.parametrize("name", list(CASES_1D))
+@pytest.mark.parametrize("dtype", [ta.float32, ta.float64, ta.float16, ta.bfloat16, ta.int32, ta.int8], ids=str)
+def test_conv1d(device, dtype, name):
+    xs, ws, stride, pad = CASES_1D[name]
+    fan_in = ws[1] * ws[2]
+    hx, dx = support.both(support.values_for(dtype, SEED, 11, xs, -2, 2), dtype, device)
+    lim = 100 if dtype.is_integral else 2 * (2.0 / fan_in) ** 0.5
+    hw, dw = support.both(support.values_for(dtype, SEED, 12, ws, -lim, lim), dtype, device)
+    want, got = ops.convolve1d(hx, hw, stride, pad), ops.convolve1d(dx, dw, stride, pad)
+    assert got.shape == want.shape
+    if dtype.is_integral:
+        support.assert_bit_exact(got.storage(), want.storage(), f"conv1d {dtype} {name}")
+    elif dtype in (ta.float16, ta.bfloat16):
+        support.assert_close(got.numpy(), want.numpy(), 2e-3 if dtype is ta.float16 else 2.0 ** -7, 1e-3, f"conv1d {dtype} {name}")
+    else:
+        eps = 2.0 ** -24 if dtype is ta.float32 else 2.0 ** -53
+        support.assert_close(got.numpy(), want.numpy(), 1e-5 if dtype is ta.float32 else 1e-13, fan_in * eps * 4, f"conv1d {dtype} {name}")

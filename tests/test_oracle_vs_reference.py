@@ -292,3 +292,30 @@ def test_triangular_rejects_other_ranks(oracle, reference):
         with support.use_functions(lib):
             with pytest.raises(ops.TannicError):
                 ops.triu(x, 0)
+
+
+CONV1D_CASES = {
+    "plain": ((2, 3, 17), (4, 3, 5), 1, 0),
+    "stride_pad": ((1, 2, 20), (3, 2, 4), 3, 2),
+    "wide_pad": ((2, 1, 4), (2, 1, 3), 1, 4),
+    "one_output": ((1, 4, 6), (5, 4, 6), 1, 0),
+}
+
+
+@pytest.mark.parametrize("name", list(CONV1D_CASES))
+@pytest.mark.parametrize("dtype", INTS + REALS, ids=str)
+def test_conv1d(oracle, reference, dtype, name):
+    xs, ws, stride, pad = CONV1D_CASES[name]
+    x, w = make(dtype, 41, xs, -3, 3), make(dtype, 42, ws, -3, 3)
+    check(oracle, reference, lambda: ops.convolve1d(x, w, stride, pad), f"conv1d {dtype} {name}")
+
+
+def test_conv1d_strided_signal_and_status(oracle, reference):
+    x = make(ta.float32, 43, (2, 12, 3)).transpose(1, 2)          # [2, 3, 12] with the length stride 3
+    w = make(ta.float32, 44, (4, 3, 5))
+    check(oracle, reference, lambda: ops.convolve1d(x, w, 2, 1), "conv1d strided signal")
+    bad = ta.Tensor(ta.float32, (1, 4, 2)).initialize(ta.Host())
+    for lib in (oracle, reference):
+        with support.use_functions(lib):
+            with pytest.raises(ops.TannicError):      # destination of the wrong shape: ERROR
+                ops._call("conv1d", ta.Host(), [x, w], bad, extra=(ops.C.c_size_t(1), ops.C.c_size_t(2)))
