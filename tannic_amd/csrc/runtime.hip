@@ -4,6 +4,7 @@
 #include <cstdlib>
 #include <mutex>
 #include <string>
+#include <unordered_map>
 #include <vector>
 
 #include "common.hpp"
@@ -163,18 +164,77 @@ int tannic_hip_set_device(int id) {
     return TANNIC_SUCCESS;
 }
 
+// The front end allocates a destination per operator node and drops it soon after.  A released block is kept,
+// tagged with the stream it was allocated and released on, and handed to the next request of a fitting size on that
+// SAME stream: the stream's order already separates the old user's kernels from the new user's, so neither a
+// stream-ordered free nor an allocation has to be queued between two kernels.  Requests that find no block, and
+// blocks that push the kept total over the limit, go to hipMallocAsync / hipFreeAsync.
+namespace {
+struct MemBlock {
+    size_t size;
+    hipStream_t stream;
+    int device;
+};
+struct FreeBlock {
+    void* ptr;
+    MemBlock info;
+};
+std::mutex g_mem_mutex;
+std::unordered_map<void*, MemBlock> g_mem_live;
+std::vector<FreeBlock> g_mem_free;     // oldest first
+size_t g_mem_kept = 0;
+constexpr size_t kMemKeepLimit = size_t(48) << 30;
+
+size_t block_size(size_t nbytes) {
+    if (nbytes == 0) nbytes = 1;
+    const size_t grain = nbytes < (size_t(1) << 20) ? 512 : (size_t(2) << 20);
+    return (nbytes + grain - 1) / grain * grain;
+}
+}  // namespace
+
 void* tannic_hip_allocate(const tannic_device_t* device, size_t nbytes) {
     if (!device || tannic_hip_set_device(device->id) != TANNIC_SUCCESS) return nullptr;
     retain_pool_memory(device->id);
     Streams& streams = Streams::instance();
     hipStream_t stream = streams.pop(device->id);
-    void* ptr = nullptr;
-    hipError_t err = hipMallocAsync(&ptr, nbytes ? nbytes : 1, stream);
     streams.put(device->id, stream);
+    const size_t size = block_size(nbytes);
+    {
+        std::lock_guard<std::mutex> lock(g_mem_mutex);
+        size_t best = g_mem_free.size();
+        for (size_t i = 0; i < g_mem_free.size(); ++i) {
+            const MemBlock& b = g_mem_free[i].info;
+            if (b.device != device->id || b.stream != stream || b.size < size || b.size > size + size / 4) continue;
+            if (best == g_mem_free.size() || b.size < g_mem_free[best].info.size) best = i;
+        }
+        if (best != g_mem_free.size()) {
+            const FreeBlock f = g_mem_free[best];
+            g_mem_free.erase(g_mem_free.begin() + best);
+            g_mem_kept -= f.info.size;
+            g_mem_live[f.ptr] = f.info;
+            return f.ptr;
+        }
+    }
+    void* ptr = nullptr;
+    hipError_t err = hipMallocAsync(&ptr, size, stream);
+    if (err != hipSuccess) {
+        // give the kept blocks back and try once more
+        std::vector<FreeBlock> all;
+        {
+            std::lock_guard<std::mutex> lock(g_mem_mutex);
+            all.swap(g_mem_free);
+            g_mem_kept = 0;
+        }
+        for (const FreeBlock& f : all) (void)hipFreeAsync(f.ptr, f.info.stream);
+        (void)hipGetLastError();
+        err = hipMallocAsync(&ptr, size, stream);
+    }
     if (err != hipSuccess) {
         set_error("hipMallocAsync", __FILE__, __LINE__, err);
         return nullptr;
     }
+    std::lock_guard<std::mutex> lock(g_mem_mutex);
+    g_mem_live[ptr] = MemBlock{size, stream, device->id};
     return ptr;
 }
 
@@ -183,9 +243,36 @@ void* tannic_hip_deallocate(const tannic_device_t* device, void* address) {
     if (tannic_hip_set_device(device->id) != TANNIC_SUCCESS) return nullptr;
     Streams& streams = Streams::instance();
     hipStream_t stream = streams.pop(device->id);
-    hipError_t err = hipFreeAsync(address, stream);
     streams.put(device->id, stream);
-    if (err != hipSuccess) set_error("hipFreeAsync", __FILE__, __LINE__, err);
+    std::vector<FreeBlock> evict;
+    bool kept = false;
+    {
+        std::lock_guard<std::mutex> lock(g_mem_mutex);
+        auto it = g_mem_live.find(address);
+        if (it != g_mem_live.end()) {
+            const MemBlock info = it->second;
+            g_mem_live.erase(it);
+            // only a block released on the stream it lives on can be reused without waiting
+            if (info.stream == stream && info.device == device->id && info.size <= kMemKeepLimit) {
+                g_mem_free.push_back(FreeBlock{address, info});
+                g_mem_kept += info.size;
+                kept = true;
+                while (g_mem_kept > kMemKeepLimit && !g_mem_free.empty()) {
+                    evict.push_back(g_mem_free.front());
+                    g_mem_kept -= g_mem_free.front().info.size;
+                    g_mem_free.erase(g_mem_free.begin());
+                }
+            }
+        }
+    }
+    for (const FreeBlock& f : evict) {
+        hipError_t err = hipFreeAsync(f.ptr, f.info.stream);
+        if (err != hipSuccess) set_error("hipFreeAsync", __FILE__, __LINE__, err);
+    }
+    if (!kept) {
+        hipError_t err = hipFreeAsync(address, stream);
+        if (err != hipSuccess) set_error("hipFreeAsync", __FILE__, __LINE__, err);
+    }
     return nullptr;
 }
 
