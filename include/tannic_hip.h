@@ -241,11 +241,18 @@ int tannic_hip_view_as_cartesian(const tannic_tensor_t* re, const tannic_tensor_
 int tannic_hip_view_as_polar(const tannic_tensor_t* rho, const tannic_tensor_t* theta, tannic_tensor_t* dst, tannic_stream_t stream);
 
 /* ------------------------------------------------------------------ *
- * Shape-changing copies     replaces src/cuda/reps.cuh:11, src/cuda/triang.cuh:11-12
+ * Shape-changing copies     replaces src/cuda/{reps,concat,outer,triang}.cuh
  * ------------------------------------------------------------------ */
 /* cuda::repeat(src, dst, axis, reps, stream): every index along `axis` repeated `reps` times in place
  * (dst[.., j*reps + r, ..] = src[.., j, ..]); src strided, dst contiguous (CPU: src/cpu/reps.cpp:18-99) */
 int tannic_hip_repeat(const tannic_tensor_t* src, tannic_tensor_t* dst, tannic_stream_t stream, int axis, int reps);
+/* cuda::concat(a, b, dst, stream, axis): dst = a followed by b along `axis`; same dtype and rank, other extents equal;
+ * sources strided, dst contiguous (src/cuda/concat.cuh:11; CPU: src/cpu/concat.cpp:18-129) */
+int tannic_hip_concat(const tannic_tensor_t* a, const tannic_tensor_t* b, tannic_tensor_t* dst, tannic_stream_t stream, int axis);
+/* cuda::outer(a, b, dst, stream): dst[i][j] = a[i] * b[j] for vectors a, b, in the type of the CPU path's pair table
+ * (src/cuda/outer.cuh:11; CPU: src/cpu/outer.cpp:18-110).  Pairs whose table type differs from the dtype the front end
+ * gives the destination (the larger dtype code) return UNSUPPORTED_DTYPE. */
+int tannic_hip_outer(const tannic_tensor_t* a, const tannic_tensor_t* b, tannic_tensor_t* dst, tannic_stream_t stream);
 /* cuda::triu / cuda::tril: rank 2; keeps j >= i + k (upper) or j <= i + k (lower) with the sum formed in
  * unsigned 64-bit as the CPU path forms it (src/cpu/triang.cpp:8-22, 24-105); other ranks: UNSUPPORTED_DTYPE */
 int tannic_hip_triu(const tannic_tensor_t* src, tannic_tensor_t* dst, tannic_stream_t stream, int k);

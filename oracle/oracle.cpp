@@ -711,6 +711,58 @@ template <class T, bool UPPER> int triangular_run(const tannic_tensor_t* src, ta
 }
 
 /* ------------------------------------------------------------------ *
+ * concat along one axis                    src/cpu/concat.cpp:18-98
+ * the block behind the axis is addressed with ONE stride, that of dimension axis + 1 (lines 66, 76): right whenever
+ * at most one dimension follows the axis, which is what the reference's tests cover
+ * ------------------------------------------------------------------ */
+template <class T> int concat_run(const tannic_tensor_t* a, const tannic_tensor_t* b, tannic_tensor_t* dst, int dim) {
+    const T* pa = static_cast<const T*>(a->address);
+    const T* pb = static_cast<const T*>(b->address);
+    T* pd = static_cast<T*>(dst->address);
+    const int rank = dst->rank;
+    size_t outer = 1, inner = 1;
+    for (int i = 0; i < dim; ++i) outer *= a->shape.sizes[i];
+    for (int i = dim + 1; i < rank; ++i) inner *= a->shape.sizes[i];
+    const size_t na = a->shape.sizes[dim], nb = b->shape.sizes[dim];
+    for (size_t o = 0; o < outer; ++o) {
+        size_t t = o;
+        int64_t offa = 0, offb = 0;
+        for (int i = dim - 1; i >= 0; --i) {
+            const size_t c = t % a->shape.sizes[i];
+            t /= a->shape.sizes[i];
+            offa += static_cast<int64_t>(c) * a->strides.sizes[i];
+            offb += static_cast<int64_t>(c) * b->strides.sizes[i];
+        }
+        const size_t base = o * (na + nb) * inner;
+        for (size_t j = 0; j < na; ++j)
+            for (size_t k = 0; k < inner; ++k) {
+                const int64_t in = dim == rank - 1 ? static_cast<int64_t>(k) : static_cast<int64_t>(k) * a->strides.sizes[dim + 1];
+                pd[base + j * inner + k] = pa[offa + static_cast<int64_t>(j) * a->strides.sizes[dim] + in];
+            }
+        for (size_t j = 0; j < nb; ++j)
+            for (size_t k = 0; k < inner; ++k) {
+                const int64_t in = dim == rank - 1 ? static_cast<int64_t>(k) : static_cast<int64_t>(k) * b->strides.sizes[dim + 1];
+                pd[base + (na + j) * inner + k] = pb[offb + static_cast<int64_t>(j) * b->strides.sizes[dim] + in];
+            }
+    }
+    return TANNIC_SUCCESS;
+}
+
+/* ------------------------------------------------------------------ *
+ * outer product of two vectors             src/cpu/outer.cpp:18-110
+ * dst[i][j] = a[i] * b[j] with C++'s own conversions of the pair, stored in the table's type D; contiguous vectors
+ * ------------------------------------------------------------------ */
+template <class A, class B, class D> int outer_run(const tannic_tensor_t* a, const tannic_tensor_t* b, tannic_tensor_t* dst) {
+    const A* pa = static_cast<const A*>(a->address);
+    const B* pb = static_cast<const B*>(b->address);
+    D* pd = static_cast<D*>(dst->address);
+    const size_t n1 = a->shape.sizes[0], n2 = b->shape.sizes[0];
+    for (size_t i = 0; i < n1; ++i)
+        for (size_t j = 0; j < n2; ++j) pd[i * n2 + j] = static_cast<D>(pa[i] * pb[j]);
+    return TANNIC_SUCCESS;
+}
+
+/* ------------------------------------------------------------------ *
  * allclose                                src/cpu/val.cpp:17-83
  * ------------------------------------------------------------------ */
 template <class T> int allclose_run(const tannic_tensor_t* a, const tannic_tensor_t* b, double rtol, double atol) {
@@ -880,6 +932,36 @@ int oracle_repeat(const tannic_tensor_t* s, tannic_tensor_t* d, int axis, int re
         case TANNIC_INT64: case TANNIC_FLOAT64: return repeat_run<uint64_t>(s, d, axis, reps);
         default: return TANNIC_UNSUPPORTED_DTYPE;
     }
+}
+/* src/cpu/concat.cpp:104-127: dispatch on the destination dtype */
+int oracle_concat(const tannic_tensor_t* a, const tannic_tensor_t* b, tannic_tensor_t* d, int axis) {
+    switch (d->dtype) {
+        case TANNIC_INT8: return concat_run<int8_t>(a, b, d, axis);
+        case TANNIC_INT16: case TANNIC_FLOAT16: case TANNIC_BFLOAT16: return concat_run<uint16_t>(a, b, d, axis);
+        case TANNIC_INT32: case TANNIC_FLOAT32: return concat_run<uint32_t>(a, b, d, axis);
+        case TANNIC_INT64: case TANNIC_FLOAT64: return concat_run<uint64_t>(a, b, d, axis);
+        default: return TANNIC_UNSUPPORTED_DTYPE;
+    }
+}
+/* src/cpu/outer.cpp:54-99.  Restated for the pairs whose table type is the dtype the front end sizes the destination
+ * with (the larger dtype code); the other pairs of the table overrun that destination and are not offered. */
+int oracle_outer(const tannic_tensor_t* a, const tannic_tensor_t* b, tannic_tensor_t* d) {
+    const int x = a->dtype, y = b->dtype;
+#define OUTER(X, Y, TA, TB, TD) if (x == X && y == Y) return outer_run<TA, TB, TD>(a, b, d);
+    OUTER(TANNIC_INT8, TANNIC_INT64, int8_t, int64_t, int64_t) OUTER(TANNIC_INT64, TANNIC_INT8, int64_t, int8_t, int64_t)
+    OUTER(TANNIC_INT16, TANNIC_INT64, int16_t, int64_t, int64_t) OUTER(TANNIC_INT64, TANNIC_INT16, int64_t, int16_t, int64_t)
+    OUTER(TANNIC_INT32, TANNIC_INT64, int32_t, int64_t, int64_t) OUTER(TANNIC_INT64, TANNIC_INT32, int64_t, int32_t, int64_t)
+    OUTER(TANNIC_INT64, TANNIC_INT64, int64_t, int64_t, int64_t)
+    OUTER(TANNIC_FLOAT16, TANNIC_FLOAT32, f16, float, float) OUTER(TANNIC_FLOAT32, TANNIC_FLOAT16, float, f16, float)
+    OUTER(TANNIC_FLOAT16, TANNIC_FLOAT64, f16, double, double) OUTER(TANNIC_FLOAT64, TANNIC_FLOAT16, double, f16, double)
+    OUTER(TANNIC_BFLOAT16, TANNIC_FLOAT32, b16, float, float) OUTER(TANNIC_FLOAT32, TANNIC_BFLOAT16, float, b16, float)
+    OUTER(TANNIC_BFLOAT16, TANNIC_FLOAT64, b16, double, double) OUTER(TANNIC_FLOAT64, TANNIC_BFLOAT16, double, b16, double)
+    OUTER(TANNIC_FLOAT32, TANNIC_FLOAT32, float, float, float) OUTER(TANNIC_FLOAT32, TANNIC_FLOAT64, float, double, double)
+    OUTER(TANNIC_FLOAT64, TANNIC_FLOAT32, double, float, double) OUTER(TANNIC_FLOAT64, TANNIC_FLOAT64, double, double, double)
+    OUTER(TANNIC_INT32, TANNIC_FLOAT32, int32_t, float, float) OUTER(TANNIC_FLOAT32, TANNIC_INT32, float, int32_t, float)
+    OUTER(TANNIC_INT32, TANNIC_FLOAT64, int32_t, double, double) OUTER(TANNIC_FLOAT64, TANNIC_INT32, double, int32_t, double)
+#undef OUTER
+    return TANNIC_UNSUPPORTED_DTYPE;
 }
 /* src/cpu/triang.cpp:75-103: int32, int64 and the float types */
 int oracle_triu(const tannic_tensor_t* s, tannic_tensor_t* d, int k) {

@@ -20,6 +20,8 @@
 #include "cpu/complex.hpp"
 #include "cpu/cpy.hpp"
 #include "cpu/reps.hpp"
+#include "cpu/concat.hpp"
+#include "cpu/outer.hpp"
 #include "cpu/triang.hpp"
 #include "cpu/val.hpp"
 
@@ -54,6 +56,8 @@ int ref_conv2d_biased(const tensor_t* x, const tensor_t* w, const tensor_t* b, t
 int ref_conv1d(const tensor_t* x, const tensor_t* w, tensor_t* y, size_t pad, size_t stride) { return cpu::conv1d(x, w, y, pad, stride); }
 int ref_cpy(const tensor_t* s, tensor_t* d) { return cpu::cpy(s, d); }
 int ref_repeat(const tensor_t* s, tensor_t* d, int axis, int reps) { return cpu::repeat(s, d, axis, reps); }
+int ref_concat(const tensor_t* a, const tensor_t* b, tensor_t* d, int axis) { return cpu::concat(a, b, d, axis); }
+int ref_outer(const tensor_t* a, const tensor_t* b, tensor_t* d) { return cpu::outer(a, b, d); }
 int ref_triu(const tensor_t* s, tensor_t* d, int k) { return cpu::triu(s, d, k); }
 int ref_tril(const tensor_t* s, tensor_t* d, int k) { return cpu::tril(s, d, k); }
 int ref_allclose(const tensor_t* a, const tensor_t* b, double rtol, double atol) {

@@ -110,6 +110,8 @@ def kernel_signatures(with_stream):
         sig[n] = (C.c_int, [TP, TP] + s + [C.c_uint8])
     sig["cpy"] = (C.c_int, [TP, TP] + s)
     sig["repeat"] = (C.c_int, [TP, TP] + s + [C.c_int, C.c_int])
+    sig["concat"] = (C.c_int, [TP, TP, TP] + s + [C.c_int])
+    sig["outer"] = (C.c_int, [TP, TP, TP] + s)
     sig["triu"] = (C.c_int, [TP, TP] + s + [C.c_int])
     sig["tril"] = (C.c_int, [TP, TP] + s + [C.c_int])
     sig["allclose"] = (C.c_int, [TP, TP] + s + [C.c_double, C.c_double])

@@ -107,9 +107,9 @@ bool allclose(const tensor_t* a, const tensor_t* b, stream_t q, double rtol, dou
 status conv1d(const tensor_t* x, const tensor_t* w, tensor_t* y, stream_t q, const size_t pad, const size_t stride) {
     return static_cast<status>(tannic_hip_conv1d(in(x), in(w), out(y), st(q), pad, stride));
 }
-status outer(const tensor_t*, const tensor_t*, tensor_t*, stream_t) { return UNSUPPORTED_DTYPE; }
+status outer(const tensor_t* a, const tensor_t* b, tensor_t* d, stream_t q) { return static_cast<status>(tannic_hip_outer(in(a), in(b), out(d), st(q))); }
 status repeat(const tensor_t* s, tensor_t* d, int axis, int reps, stream_t q) { return static_cast<status>(tannic_hip_repeat(in(s), out(d), st(q), axis, reps)); }
-status concat(const tensor_t*, const tensor_t*, tensor_t*, stream_t, int) { return UNSUPPORTED_DTYPE; }
+status concat(const tensor_t* a, const tensor_t* b, tensor_t* d, stream_t q, int axis) { return static_cast<status>(tannic_hip_concat(in(a), in(b), out(d), st(q), axis)); }
 status triu(const tensor_t* s, tensor_t* d, stream_t q, int k) { return static_cast<status>(tannic_hip_triu(in(s), out(d), st(q), k)); }
 status tril(const tensor_t* s, tensor_t* d, stream_t q, int k) { return static_cast<status>(tannic_hip_tril(in(s), out(d), st(q), k)); }
 

@@ -1,4 +1,4 @@
-// repeat (interleaved repetition along an axis) and triu / tril.
+// repeat (interleaved repetition along an axis), concat, outer, triu / tril.
 //
 // Both move elements as opaque bit patterns: no arithmetic, so every dtype of a
 // given width shares a kernel.  repeat gathers from an arbitrarily strided
@@ -99,6 +99,104 @@ int run_repeat(const tannic_tensor_t* src, tannic_tensor_t* dst, int axis, int r
     }
 }
 
+// concat: dst[.., j, ..] = a[.., j, ..] for j < a.extent[axis], else b[.., j - a.extent[axis], ..]; both sources strided,
+// destination contiguous.  The CPU path addresses the block behind the axis with one stride (src/cpu/concat.cpp:66,76),
+// which is the same thing whenever at most one dimension follows the axis; further in, this kernel keeps indexing
+// every dimension by its own stride.
+struct ConcatPlan {
+    int rank, axis;
+    uint32_t total, first_extent;
+    FastDiv div[8];
+    int64_t stride_a[8], stride_b[8];
+};
+
+template <class U>
+__global__ __launch_bounds__(256) void concat_kernel(const U* a, const U* b, U* dst, ConcatPlan q) {
+    const uint32_t idx = blockIdx.x * 256 + threadIdx.x;
+    if (idx >= q.total) return;
+    uint32_t rest = idx, coord[8];
+    for (int d = q.rank - 1; d >= 0; --d) {
+        uint32_t next;
+        q.div[d].divmod(rest, next, coord[d]);
+        rest = next;
+    }
+    const bool second = coord[q.axis] >= q.first_extent;
+    if (second) coord[q.axis] -= q.first_extent;
+    int64_t off = 0;
+    for (int d = 0; d < q.rank; ++d) off += static_cast<int64_t>(coord[d]) * (second ? q.stride_b[d] : q.stride_a[d]);
+    dst[idx] = second ? b[off] : a[off];
+}
+
+int run_concat(const tannic_tensor_t* a, const tannic_tensor_t* b, tannic_tensor_t* dst, int axis, hipStream_t stream) {
+    size_t esize;
+    switch (dst->dtype) {   // src/cpu/concat.cpp:104-118 dispatches on the destination
+        case TANNIC_INT8: esize = 1; break;
+        case TANNIC_INT16: case TANNIC_FLOAT16: case TANNIC_BFLOAT16: esize = 2; break;
+        case TANNIC_INT32: case TANNIC_FLOAT32: esize = 4; break;
+        case TANNIC_INT64: case TANNIC_FLOAT64: esize = 8; break;
+        default: return TANNIC_UNSUPPORTED_DTYPE;
+    }
+    const int rank = dst->rank;
+    if (rank < 1 || rank > 8 || a->rank != rank || b->rank != rank || axis < 0 || axis >= rank || a->dtype != dst->dtype || b->dtype != dst->dtype) {
+        set_error_text("concat: ranks, dtypes or axis do not match");
+        return TANNIC_ERROR;
+    }
+    uint64_t total = 1;
+    ConcatPlan q{};
+    for (int d = 0; d < rank; ++d) {
+        const size_t want = d == axis ? a->shape.sizes[d] + b->shape.sizes[d] : a->shape.sizes[d];
+        if (dst->shape.sizes[d] != want || (d != axis && b->shape.sizes[d] != a->shape.sizes[d])) {
+            set_error_text("concat: shapes do not match");
+            return TANNIC_ERROR;
+        }
+        total *= want;
+        q.div[d] = FastDiv(static_cast<uint32_t>(want));
+        q.stride_a[d] = a->strides.sizes[d];
+        q.stride_b[d] = b->strides.sizes[d];
+    }
+    if (total == 0) return TANNIC_SUCCESS;
+    if (total >= (1ull << 31)) {
+        set_error_text("concat: destination of 2^31 elements or more is not supported");
+        return TANNIC_ERROR;
+    }
+    q.rank = rank;
+    q.axis = axis;
+    q.total = static_cast<uint32_t>(total);
+    q.first_extent = static_cast<uint32_t>(a->shape.sizes[axis]);
+    const dim3 grid((q.total + 255) / 256);
+    switch (esize) {
+        case 1: hipLaunchKernelGGL((concat_kernel<uint8_t>), grid, dim3(256), 0, stream, static_cast<const uint8_t*>(a->address), static_cast<const uint8_t*>(b->address), static_cast<uint8_t*>(dst->address), q); break;
+        case 2: hipLaunchKernelGGL((concat_kernel<uint16_t>), grid, dim3(256), 0, stream, static_cast<const uint16_t*>(a->address), static_cast<const uint16_t*>(b->address), static_cast<uint16_t*>(dst->address), q); break;
+        case 4: hipLaunchKernelGGL((concat_kernel<uint32_t>), grid, dim3(256), 0, stream, static_cast<const uint32_t*>(a->address), static_cast<const uint32_t*>(b->address), static_cast<uint32_t*>(dst->address), q); break;
+        default: hipLaunchKernelGGL((concat_kernel<uint64_t>), grid, dim3(256), 0, stream, static_cast<const uint64_t*>(a->address), static_cast<const uint64_t*>(b->address), static_cast<uint64_t*>(dst->address), q); break;
+    }
+    return launch_status("concat_kernel");
+}
+
+// outer: dst[i][j] = a[i] * b[j] in the type the CPU path's table gives the pair (src/cpu/outer.cpp:54-99).  It is the
+// product of a column [n1,1] and a row [1,n2], so it runs as the broadcasting multiply — for the pairs whose table type
+// is also what the front end sizes the destination with (the larger dtype code, include/tannic/transformations.hpp:208-212).
+// For the others (int8 x int8 -> int32, fp16 x fp16 -> fp32, ...) the CPU kernel writes wider elements than the
+// destination holds; those are not offered.
+static int outer_table(int first, int second) {
+    auto is_int = [](int t) { return t >= TANNIC_INT8 && t <= TANNIC_INT64; };
+    if (is_int(first) && is_int(second)) {
+        if (first == TANNIC_INT64 || second == TANNIC_INT64) return TANNIC_INT64;
+        if (first == TANNIC_INT32 && second == TANNIC_INT32) return TANNIC_INT64;
+        return TANNIC_INT32;
+    }
+    auto half = [](int t) { return t == TANNIC_FLOAT16 || t == TANNIC_BFLOAT16; };
+    const int lo = first < second ? first : second, hi = first < second ? second : first;
+    if (half(first) && half(second)) return first == second ? TANNIC_FLOAT32 : -1;
+    if (lo == TANNIC_INT32 && (half(hi) || hi == TANNIC_FLOAT32)) return TANNIC_FLOAT32;
+    if (lo == TANNIC_INT32 && hi == TANNIC_FLOAT64) return TANNIC_FLOAT64;
+    if (half(lo) && hi == TANNIC_FLOAT32) return TANNIC_FLOAT32;
+    if (half(lo) && hi == TANNIC_FLOAT64) return TANNIC_FLOAT64;
+    if (lo == TANNIC_FLOAT32 && hi == TANNIC_FLOAT32) return TANNIC_FLOAT32;
+    if ((lo == TANNIC_FLOAT32 || lo == TANNIC_FLOAT64) && hi == TANNIC_FLOAT64) return TANNIC_FLOAT64;
+    return -1;
+}
+
 template <class U, bool UPPER>
 __global__ __launch_bounds__(256) void triangular_kernel(const U* src, U* dst, uint32_t rows, uint32_t cols, int64_t ss0, int64_t ss1, int64_t ds0, int64_t ds1, int k, FastDiv div_cols) {
     const uint32_t idx = blockIdx.x * 256 + threadIdx.x;
@@ -147,6 +245,30 @@ extern "C" {
 int tannic_hip_repeat(const tannic_tensor_t* src, tannic_tensor_t* dst, tannic_stream_t stream, int axis, int reps) {
     if (!src || !dst) return TANNIC_ERROR;
     return th::run_repeat(src, dst, axis, reps, th::as_stream(stream));
+}
+int tannic_hip_concat(const tannic_tensor_t* a, const tannic_tensor_t* b, tannic_tensor_t* dst, tannic_stream_t stream, int axis) {
+    if (!a || !b || !dst) return TANNIC_ERROR;
+    return th::run_concat(a, b, dst, axis, th::as_stream(stream));
+}
+int tannic_hip_outer(const tannic_tensor_t* a, const tannic_tensor_t* b, tannic_tensor_t* dst, tannic_stream_t stream) {
+    if (!a || !b || !dst) return TANNIC_ERROR;
+    const int result = th::outer_table(a->dtype, b->dtype);
+    const int sized_as = a->dtype > b->dtype ? a->dtype : b->dtype;
+    if (result < 0 || result != sized_as || dst->dtype != result) return TANNIC_UNSUPPORTED_DTYPE;
+    if (a->rank != 1 || b->rank != 1 || dst->rank != 2 || dst->shape.sizes[0] != a->shape.sizes[0] || dst->shape.sizes[1] != b->shape.sizes[0]) {
+        th::set_error_text("outer: operands must be vectors and the destination their [n1, n2] product");
+        return TANNIC_ERROR;
+    }
+    tannic_tensor_t column = *a, row = *b;
+    column.rank = row.rank = 2;
+    column.shape.sizes[1] = 1;
+    column.strides.sizes[1] = 0;
+    row.shape.sizes[1] = b->shape.sizes[0];
+    row.strides.sizes[1] = b->strides.sizes[0];
+    row.shape.sizes[0] = 1;
+    row.strides.sizes[0] = 0;
+    column.layout = row.layout = TANNIC_STRIDED;
+    return tannic_hip_mul(&column, &row, dst, stream);
 }
 int tannic_hip_triu(const tannic_tensor_t* src, tannic_tensor_t* dst, tannic_stream_t stream, int k) {
     if (!src || !dst) return TANNIC_ERROR;

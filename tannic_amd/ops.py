@@ -378,6 +378,37 @@ def repeat(x, repeats, axis=0):
     return dst
 
 
+def concatenate(first, second, axis=0):
+    """``concatenate(first, second, axis)`` (``include/tannic/transformations.hpp:241-262, 344-352``)."""
+    if axis < 0:
+        raise TannicError("Negative index not supported in concat")
+    if first.dtype is not second.dtype:
+        raise TannicError("Cannot concatenate tensors of different dtypes")
+    if first.rank != second.rank or axis >= first.rank:
+        raise TannicError("Ranks must match for concatenation")
+    shape = list(first.shape)
+    for d in range(first.rank):
+        if d == axis:
+            shape[d] = first.shape[d] + second.shape[d]
+        elif first.shape[d] != second.shape[d]:
+            raise TannicError("All dimensions except concat axis must match")
+    env = _resolve(first, second)
+    dst = Tensor(first.dtype, tuple(shape)).initialize(env)
+    _call("concat", env, [first, second], dst, (C.c_int(axis),))
+    return dst
+
+
+def outer(first, second):
+    """``outer(first, second)``: vectors only; the destination takes the dtype with the larger code
+    (``include/tannic/transformations.hpp:208-221, 306-312``)."""
+    if first.rank != 1 or second.rank != 1:
+        raise TannicError("Outer product of tensors with rank more than 1 not supported")
+    dtype = first.dtype if first.dtype.code > second.dtype.code else second.dtype
+    env = _resolve(first, second)
+    dst = Tensor(dtype, (first.shape[0], second.shape[0])).initialize(env)
+    return _call("outer", env, [first, second], dst)
+
+
 def _triangular(name, x, k):
     env = _resolve(x)
     dst = Tensor(x.dtype, x.shape).initialize(env)

@@ -41,9 +41,10 @@ class Device:
         if id < 0 or id >= count:
             raise IndexError("Invalid device ID")
         self.id = id
+        self._structure = abi.device_t(id)
 
     def structure(self):
-        return abi.device_t(self.id)
+        return self._structure
 
     def __eq__(self, other):
         return isinstance(other, Device) and other.id == self.id
@@ -213,6 +214,10 @@ class Tensor:
 
     # ---- the descriptor handed to the backend ---------------------------
     def descriptor(self):
+        """The ``tensor_t`` of this view; built once (a view's shape, strides, offset and buffer never change)."""
+        cached = self.__dict__.get("_descriptor")
+        if cached is not None:
+            return cached
         t = abi.tensor_t()
         t.address = self.address
         t.rank = self.rank
@@ -228,6 +233,7 @@ class Tensor:
             t.environment.resource.host.traits = abi.PAGEABLE
         t.size = self.nelements
         t.layout = abi.SINGLETON if self.is_singleton() else abi.CONTIGUOUS if self.is_contiguous() else abi.STRIDED
+        self._descriptor = t
         return t
 
     # ---- views (include/tannic/views.hpp) --------------------------------

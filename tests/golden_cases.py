@@ -24,6 +24,8 @@ def build(spec, env):
     t = ta.tensor(np.array(spec["data"], dtype=np.float64).reshape(spec["shape"]), dtype, env)
     if "transpose" in spec:
         t = t.transpose(*spec["transpose"])
+    if "expand" in spec:
+        t = t.expand(*spec["expand"])
     if "permute" in spec:
         t = t.permute(*spec["permute"])
     return t
@@ -68,6 +70,10 @@ def run(case, env):
         out = ops.mean(ops.mul(ins[0], ins[0]), case["axis"])
     elif op == "conv1d":
         out = ops.convolve1d(ins[0], ins[1], case["stride"], case["padding"])
+    elif op == "concat":
+        out = ops.concatenate(ins[0], ins[1], case["axis"])
+    elif op == "outer":
+        out = ops.outer(ins[0], ins[1])
     elif op == "repeat":
         out = ops.repeat(ins[0], case["repeats"], case["axis"])
     elif op == "polar":

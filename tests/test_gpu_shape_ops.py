@@ -73,3 +73,64 @@ def test_status_codes(device):
     b = ta.Tensor(ta.boolean, (8,)).initialize(device)
     with pytest.raises(ops.TannicError):
         ops.repeat(b, 2, 0)                 # no boolean repeat
+
+
+# ---- concat and outer ---------------------------------------------------------------------------------------------------
+MORE_GOLDEN = [c for c in golden_cases.TENSOR_CASES if c["op"] in ("concat", "outer")]
+
+
+@pytest.mark.parametrize("case", MORE_GOLDEN, ids=lambda c: c["name"])
+def test_concat_outer_reference_vectors_on_device(device, case):
+    got = golden_cases.run(case, device)
+    np.testing.assert_array_equal(got, golden_cases.expected_of(case))
+
+
+CONCAT = {
+    "rows": ((2, 3), (4, 3), 0, [], []),
+    "columns": ((3, 2), (3, 5), 1, [], []),
+    "last_axis_rank3": ((2, 3, 4), (2, 3, 2), 2, [], []),
+    "middle_axis_rank3": ((2, 3, 4), (2, 5, 4), 1, [], []),
+    "expanded_operand": ((1, 1, 3), (2, 4, 3), 1, [("expand", (2, 1, 3))], []),
+    "transposed_operands": ((2, 3, 4), (2, 3, 5), 1, [("transpose", (1, 2))], [("transpose", (1, 2))]),
+    "sequence_with_token": ((4, 1, 64), (4, 50, 64), 1, [], []),
+}
+
+
+@pytest.mark.parametrize("name", list(CONCAT))
+@pytest.mark.parametrize("dtype", DTYPES, ids=str)
+def test_concat_bit_exact(device, dtype, name):
+    sa, sb, axis, va, vb = CONCAT[name]
+    ha, da = support.both(support.values_for(dtype, SEED, 3, sa, -4, 4), dtype, device)
+    hb, db = support.both(support.values_for(dtype, SEED, 4, sb, -4, 4), dtype, device)
+    ha, da, hb, db = support.apply_view(ha, va), support.apply_view(da, va), support.apply_view(hb, vb), support.apply_view(db, vb)
+    want, got = ops.concatenate(ha, hb, axis), ops.concatenate(da, db, axis)
+    assert got.shape == want.shape
+    support.assert_bit_exact(got.storage(), want.storage(), f"concat {dtype} {name}")
+
+
+@pytest.mark.parametrize("axis", [0, 1])
+def test_concat_leading_axes_follow_numpy(device, axis):
+    """More than one dimension behind the axis: every dimension is indexed by its own stride (the CPU path is not)."""
+    a = support.values_for(ta.float32, SEED, 5, (2, 3, 4, 5), -4, 4)
+    b = support.values_for(ta.float32, SEED, 6, (3, 3, 4, 5) if axis == 0 else (2, 2, 4, 5), -4, 4)
+    got = ops.concatenate(ta.tensor(a, ta.float32, device), ta.tensor(b, ta.float32, device), axis).numpy()
+    np.testing.assert_array_equal(got, np.concatenate([a, b], axis=axis))
+
+
+OUTER = [(ta.int8, ta.int64), (ta.int64, ta.int32), (ta.int64, ta.int64), (ta.float32, ta.float32), (ta.float32, ta.float64),
+         (ta.float64, ta.float64), (ta.int32, ta.float32), (ta.float64, ta.int32), (ta.float16, ta.float32), (ta.float32, ta.bfloat16)]
+
+
+@pytest.mark.parametrize("pair", OUTER, ids=lambda p: f"{p[0]}-{p[1]}")
+def test_outer_bit_exact(device, pair):
+    ha, da = support.both(support.values_for(pair[0], SEED, 7, (300,), -3, 3), pair[0], device)
+    hb, db = support.both(support.values_for(pair[1], SEED, 8, (77,), -3, 3), pair[1], device)
+    want, got = ops.outer(ha, hb), ops.outer(da, db)
+    assert got.shape == want.shape == (300, 77) and got.dtype is want.dtype
+    support.assert_bit_exact(got.storage(), want.storage(), f"outer {pair}")
+
+
+def test_outer_pairs_that_overrun_their_destination_are_refused(device):
+    a = ta.tensor(np.ones(4), ta.float16, device)
+    with pytest.raises(ops.TannicError):
+        ops.outer(a, a)     # the table says fp32, the destination is fp16

@@ -224,3 +224,25 @@ def test_triangular_negative_offset_wraps_for_the_first_rows(oracle):
     np.testing.assert_array_equal(up[2:], np.triu(x, -2)[2:])
     np.testing.assert_array_equal(lo[:2], x[:2])
     np.testing.assert_array_equal(lo[2:], np.tril(x, -2)[2:])
+
+
+# ---- concat and outer against numpy --------------------------------------------------------------------------------
+@pytest.mark.parametrize("axis", [1, 2])
+def test_concat_is_numpy_concatenate_for_the_last_two_axes(oracle, axis):
+    a = support.values_for(ta.float32, 5, 44, (2, 3, 4), -2, 2)
+    shape_b = (2, 5, 4) if axis == 1 else (2, 3, 6)
+    b = support.values_for(ta.float32, 5, 45, shape_b, -2, 2)
+    with support.use_functions(oracle):
+        got = ops.concatenate(support.host_tensor(a, ta.float32), support.host_tensor(b, ta.float32), axis).numpy()
+    np.testing.assert_array_equal(got, np.concatenate([a, b], axis=axis))
+
+
+def test_outer_is_numpy_outer_and_unsupported_pairs_say_so(oracle):
+    a = support.values_for(ta.float64, 5, 46, (6,), -2, 2)
+    b = support.values_for(ta.float32, 5, 47, (4,), -2, 2)
+    with support.use_functions(oracle):
+        got = ops.outer(support.host_tensor(a, ta.float64), support.host_tensor(b, ta.float32)).numpy()
+        np.testing.assert_array_equal(got, np.outer(a, b.astype(np.float64)))
+        # int8 x int8: the reference's kernel writes int32 into the int8 destination the front end made
+        with pytest.raises(ops.TannicError):
+            ops.outer(support.host_tensor(np.ones(3), ta.int8), support.host_tensor(np.ones(3), ta.int8))

@@ -319,3 +319,43 @@ def test_conv1d_strided_signal_and_status(oracle, reference):
         with support.use_functions(lib):
             with pytest.raises(ops.TannicError):      # destination of the wrong shape: ERROR
                 ops._call("conv1d", ta.Host(), [x, w], bad, extra=(ops.C.c_size_t(1), ops.C.c_size_t(2)))
+
+
+# concat: the reference addresses the block behind the axis with one stride, so the A/B covers what it gets right —
+# at most one dimension behind the axis — with every kind of view in front of it
+CONCAT_CASES = {
+    "rows": ((2, 3), (4, 3), 0, [], []),
+    "columns": ((3, 2), (3, 5), 1, [], []),
+    "last_axis_rank3": ((2, 3, 4), (2, 3, 2), 2, [], []),
+    "middle_axis_rank3": ((2, 3, 4), (2, 5, 4), 1, [], []),
+    "transposed_operand": ((2, 4, 3), (2, 5, 3), 1, [("transpose", (1, 2))], []),   # first becomes [2, 3, 4]... see below
+    "expanded_operand": ((1, 1, 3), (2, 4, 3), 1, [("expand", (2, 1, 3))], []),
+    "sliced_operands": ((4, 6), (4, 8), 1, [("index", (slice(0, 4, 2), slice(0, 6, 2)))], [("index", (slice(1, 4, 2), slice(0, 8, 2)))]),
+    "vectors": ((5,), (3,), 0, [], []),
+}
+
+
+@pytest.mark.parametrize("name", [n for n in CONCAT_CASES if n != "transposed_operand"])
+@pytest.mark.parametrize("dtype", INTS + REALS, ids=str)
+def test_concat(oracle, reference, dtype, name):
+    sa, sb, axis, va, vb = CONCAT_CASES[name]
+    a = support.apply_view(make(dtype, 51, sa), va)
+    b = support.apply_view(make(dtype, 52, sb), vb)
+    check(oracle, reference, lambda: ops.concatenate(a, b, axis), f"concat {dtype} {name}")
+
+
+def test_concat_transposed_operands(oracle, reference):
+    a = make(ta.float32, 53, (2, 3, 4)).transpose(1, 2)     # [2, 4, 3], strides (12, 1, 4)
+    b = make(ta.float32, 54, (2, 3, 5)).transpose(1, 2)     # [2, 5, 3]
+    check(oracle, reference, lambda: ops.concatenate(a, b, 1), "concat transposed")
+
+
+OUTER_PAIRS = [(ta.int8, ta.int64), (ta.int64, ta.int16), (ta.int32, ta.int64), (ta.int64, ta.int64),
+               (ta.float32, ta.float32), (ta.float32, ta.float64), (ta.float64, ta.float32), (ta.float64, ta.float64),
+               (ta.int32, ta.float32), (ta.float32, ta.int32), (ta.int32, ta.float64), (ta.float64, ta.int32)]
+
+
+@pytest.mark.parametrize("pair", OUTER_PAIRS, ids=lambda p: f"{p[0]}-{p[1]}")
+def test_outer(oracle, reference, pair):
+    a, b = make(pair[0], 55, (7,), -3, 3), make(pair[1], 56, (5,), -3, 3)
+    check(oracle, reference, lambda: ops.outer(a, b), f"outer {pair}")
