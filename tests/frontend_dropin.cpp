@@ -20,6 +20,7 @@
 #include "comparisons.hpp"
 #include "complex.hpp"
 #include "convolutions.hpp"
+#include "filter.hpp"
 #include "functions.hpp"
 #include "reductions.hpp"
 #include "transformations.hpp"
@@ -81,6 +82,11 @@ int main() {
     const Tensor Bias = seeded(float32, {5}, 14, -1, 1);
     const Tensor Rho = seeded(float32, {6, 10}, 15, 0.5, 2);
     const Tensor Theta = seeded(float32, {6, 10}, 16, -3, 3);
+    const Tensor V1 = seeded(float32, {40}, 17, -2, 2);
+    const Tensor V2 = seeded(float64, {25}, 18, -2, 2);
+    const Tensor Sig = seeded(float32, {2, 6, 50}, 19, -1, 1);
+    const Tensor W1 = seeded(float32, {5, 6, 4}, 20, -0.4, 0.4);
+    const Tensor Sq = seeded(float32, {12, 12}, 21, -1, 1);
 
     std::vector<Case> cases = {
         {"log(P)", 1e-5, 1e-8, [&](Environment e) { return Tensor(log(place(P, e))); }},
@@ -108,6 +114,11 @@ int main() {
         {"sum over last axis", 1e-5, 1e-5, [&](Environment e) { return Tensor(sum(place(X, e), -1, true)); }},
         {"mean of squares over axis 1", 1e-5, 1e-5, [&](Environment e) { Tensor x = place(X, e); return Tensor(mean(x * x, 1)); }},
         {"polar -> realify", 1e-5, 1e-6, [&](Environment e) { return Tensor(realify(polar(place(Rho, e), place(Theta, e)))); }},
+        {"repeat heads (axis 1, 4 times)", 0, 0, [&](Environment e) { return Tensor(repeat(place(Q, e), 4, 1)); }},
+        {"concatenate along axis 1", 0, 0, [&](Environment e) { Tensor a = place(A, e); return Tensor(concatenate(a, a * 2.0f, 1)); }},
+        {"outer float32 x float64", 0, 0, [&](Environment e) { return Tensor(outer(place(V1, e), place(V2, e))); }},
+        {"triangular lower, offset 1", 0, 0, [&](Environment e) { return Tensor(triangular(place(Sq, e), Position::Lower, 1)); }},
+        {"conv1d k4 s2 p1", 1e-5, 1e-5, [&](Environment e) { return Tensor(convolve1D(place(Sig, e), place(W1, e), 2, 1)); }},
     };
 
     int failures = 0;
