@@ -39,18 +39,22 @@ constexpr int kSkinnyUnroll = 8;   // K steps of 32 whose loads are issued toget
 // what a chunk past the end of K reads instead: both operands, so that the product is an exact zero
 __device__ const uint4y skinny_zeros = {0, 0, 0, 0};
 
-// MB: blocks of 16 rows of x
-template <class T, int MB>
+// MB: blocks of 16 rows of x; NB: blocks of 16 columns per wavefront (a fragment of x then serves NB fragments of W)
+template <class T, int MB, int NB>
 __global__ __launch_bounds__(64 * kSkinnyWaves) void gemm_skinny_kernel(const T* x, const T* w, T* c, GemmProblem p, uint32_t k_per_wave) {
-    __shared__ float4y partial[kSkinnyWaves][MB][64];
+    __shared__ float4y partial[kSkinnyWaves][MB * NB][64];
     int64_t ox, ow, oc;
     batch_offsets(p, blockIdx.y, ox, ow, oc);
     const int wave = threadIdx.x / 64, lane = threadIdx.x % 64;
     const uint32_t r = lane % 16, kc = lane / 16;
-    const uint32_t n0 = blockIdx.x * 16;
+    const uint32_t n0 = blockIdx.x * 16 * NB;
     // rows past the end are read from the last row: they only feed results that are never stored
-    const uint32_t n = n0 + r < p.N ? n0 + r : p.N - 1;
-    const T* wrow = w + ow + static_cast<int64_t>(n) * p.b_cs + kc * 8;
+    const T* wrow[NB];
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb) {
+        const uint32_t n = n0 + nb * 16 + r < p.N ? n0 + nb * 16 + r : p.N - 1;
+        wrow[nb] = w + ow + static_cast<int64_t>(n) * p.b_cs + kc * 8;
+    }
     const T* xrow[MB];
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb) {
@@ -61,37 +65,45 @@ __global__ __launch_bounds__(64 * kSkinnyWaves) void gemm_skinny_kernel(const T*
     const uint32_t k_end = k_begin + k_per_wave < p.K ? k_begin + k_per_wave : p.K;
     const T* zeros = reinterpret_cast<const T*>(&skinny_zeros) - kc * 8;
 
-    float4y acc[MB];
+    float4y acc[MB][NB];
 #pragma unroll
-    for (int mb = 0; mb < MB; ++mb) acc[mb] = float4y{0.0f, 0.0f, 0.0f, 0.0f};
+    for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb) acc[mb][nb] = float4y{0.0f, 0.0f, 0.0f, 0.0f};
     for (uint32_t k0 = k_begin; k0 < k_end; k0 += 32 * kSkinnyUnroll) {
-        uint4y fw[kSkinnyUnroll], fx[kSkinnyUnroll][MB];
+        uint4y fw[kSkinnyUnroll][NB], fx[kSkinnyUnroll][MB];
 #pragma unroll
         for (int u = 0; u < kSkinnyUnroll; ++u) {
             const uint32_t k = k0 + 32 * u;
             const bool live = k + kc * 8 < k_end;   // K and the ranges are multiples of 8: a chunk is inside or outside
-            fw[u] = *reinterpret_cast<const uint4y*>(live ? wrow + k : zeros + kc * 8);
+#pragma unroll
+            for (int nb = 0; nb < NB; ++nb) fw[u][nb] = *reinterpret_cast<const uint4y*>(live ? wrow[nb] + k : zeros + kc * 8);
 #pragma unroll
             for (int mb = 0; mb < MB; ++mb) fx[u][mb] = *reinterpret_cast<const uint4y*>(live ? xrow[mb] + k : zeros + kc * 8);
         }
 #pragma unroll
         for (int u = 0; u < kSkinnyUnroll; ++u)
 #pragma unroll
-            for (int mb = 0; mb < MB; ++mb) acc[mb] = skinny_mfma<T>(fw[u], fx[u][mb], acc[mb]);
+            for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+                for (int nb = 0; nb < NB; ++nb) acc[mb][nb] = skinny_mfma<T>(fw[u][nb], fx[u][mb], acc[mb][nb]);
     }
 #pragma unroll
-    for (int mb = 0; mb < MB; ++mb) partial[wave][mb][lane] = acc[mb];
+    for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb) partial[wave][mb * NB + nb][lane] = acc[mb][nb];
     __syncthreads();
     if (wave != 0) return;
     // accumulator: lane -> row of x (m) lane % 16; value v -> column n0 + 4 * (lane / 16) + v
     T* cb = c + oc;
     const bool vector_ok = p.c_rs % 4 == 0 && p.N % 4 == 0 && reinterpret_cast<uintptr_t>(cb) % 8 == 0;
 #pragma unroll
-    for (int mb = 0; mb < MB; ++mb) {
-        float4y sum = partial[0][mb][lane];
+    for (int t = 0; t < MB * NB; ++t) {
+        const int mb = t / NB, nb = t % NB;
+        float4y sum = partial[0][t][lane];
 #pragma unroll
-        for (int v = 1; v < kSkinnyWaves; ++v) sum += partial[v][mb][lane];
-        const uint32_t m = mb * 16 + r, col = n0 + 4 * kc;
+        for (int v = 1; v < kSkinnyWaves; ++v) sum += partial[v][t][lane];
+        const uint32_t m = mb * 16 + r, col = n0 + nb * 16 + 4 * kc;
         if (m >= p.M) continue;
         T out[4];
 #pragma unroll
@@ -124,12 +136,21 @@ int run_skinny(const GemmProblem& p, const void* a, const void* b, void* c, hipS
     // K is split evenly over the wavefronts, in whole steps of 32
     const uint32_t steps = (p.K + 31) / 32, per_wave = (steps + kSkinnyWaves - 1) / kSkinnyWaves;
     const uint32_t k_per_wave = per_wave * 32;
-    const uint32_t blocks = (p.N + 15) / 16;
+    // A single row costs almost nothing to load next to W; with more rows, two column blocks per wavefront halve
+    // what x costs, as long as there are still blocks for every compute unit.
+    const bool pairs = p.M > 4 && static_cast<uint64_t>((p.N + 31) / 32) * p.batches >= 224;
+    const uint32_t blocks = pairs ? (p.N + 31) / 32 : (p.N + 15) / 16;
     const dim3 grid(blocks, p.batches), block(64 * kSkinnyWaves);
-    if (p.M <= 16)
-        hipLaunchKernelGGL((gemm_skinny_kernel<T, 1>), grid, block, 0, stream, static_cast<const T*>(a), static_cast<const T*>(b), static_cast<T*>(c), p, k_per_wave);
-    else
-        hipLaunchKernelGGL((gemm_skinny_kernel<T, 2>), grid, block, 0, stream, static_cast<const T*>(a), static_cast<const T*>(b), static_cast<T*>(c), p, k_per_wave);
+    const T* pa = static_cast<const T*>(a);
+    const T* pb = static_cast<const T*>(b);
+    T* pc = static_cast<T*>(c);
+    if (p.M <= 16) {
+        if (pairs) hipLaunchKernelGGL((gemm_skinny_kernel<T, 1, 2>), grid, block, 0, stream, pa, pb, pc, p, k_per_wave);
+        else hipLaunchKernelGGL((gemm_skinny_kernel<T, 1, 1>), grid, block, 0, stream, pa, pb, pc, p, k_per_wave);
+    } else {
+        if (pairs) hipLaunchKernelGGL((gemm_skinny_kernel<T, 2, 2>), grid, block, 0, stream, pa, pb, pc, p, k_per_wave);
+        else hipLaunchKernelGGL((gemm_skinny_kernel<T, 2, 1>), grid, block, 0, stream, pa, pb, pc, p, k_per_wave);
+    }
     return launch_status("gemm_skinny_kernel");
 }
 
