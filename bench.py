@@ -257,8 +257,22 @@ def cpu_baseline(rows=64):
     t0 = time.perf_counter()
     ops.matmul(x, w.transpose())
     dt = time.perf_counter() - t0
-    return {"value": round(2.0 * rows * N * K / dt / 1e12, 6), "unit": "TFLOP/s", "cores": 1, "kind": "port",
-            "sample": f"first {rows} rows of X: [{rows},4096] . [4096,4096]^T fp16, fp32 accumulate, {dt:.1f} s of {os.cpu_count()} host CPUs' one core"}
+    result = {"value": round(2.0 * rows * N * K / dt / 1e12, 6), "unit": "TFLOP/s", "cores": 1, "kind": "port",
+              "sample": f"first {rows} rows of X: [{rows},4096] . [4096,4096]^T fp16, fp32 accumulate, {dt:.1f} s of {os.cpu_count()} host CPUs' one core"}
+    # The reference's own CPU kernels, where a build of them came along (fp32 only: its 16-bit kernels need <stdfloat>):
+    # the fp32 512^3 product of the parity configuration, one core.
+    reference = support.reference_library()
+    if reference is not None:
+        ops.set_host_functions(reference.functions)
+        a = support.host_tensor(support.uniform(0, 0, (512, 512)).astype(np.float32), ta.float32)
+        bm = support.host_tensor(support.uniform(0, 1, (512, 512)).astype(np.float32), ta.float32)
+        t0 = time.perf_counter()
+        ops.matmul(a, bm)
+        dr = time.perf_counter() - t0
+        result["reference_fp32_512"] = {"value": round(2.0 * 512 ** 3 / dr / 1e12, 6), "unit": "TFLOP/s", "cores": 1, "kind": "reference",
+                                        "sample": f"fp32 [512,512] . [512,512], the reference's cpu::gemm, {dr:.2f} s"}
+    ops.set_host_functions(None)
+    return result
 
 
 def secondary(b, only):
