@@ -297,7 +297,7 @@ def secondary(b, only):
         for dtype in (ta.float32, ta.float16):
             work += reduction_entries(b, dtype, 10)
     if only in (None, "layer"):
-        work.append(decoder_layer_entry(b, 5))
+        work.append(decoder_layer_entry(b, 20))
     return work
 
 

@@ -482,12 +482,29 @@ __global__ __launch_bounds__(256) void gemm_split_reduce_kernel(const float* par
     const float* src = partials + static_cast<size_t>(r) * p.N + col;
     float sum[4] = {0.0f, 0.0f, 0.0f, 0.0f};
     const uint32_t live = p.N - col < 4 ? p.N - col : 4;
-    for (uint32_t sp = 0; sp < splits; ++sp)
-        for (uint32_t e = 0; e < live; ++e) sum[e] += src[sp * share + e];
+    if (p.N % 4 == 0) {   // rows of the partial sums start at multiples of 16 bytes
+        for (uint32_t sp = 0; sp < splits; ++sp) {
+            const float4 v = *reinterpret_cast<const float4*>(src + sp * share);
+            sum[0] += v.x; sum[1] += v.y; sum[2] += v.z; sum[3] += v.w;
+        }
+    } else {
+        for (uint32_t sp = 0; sp < splits; ++sp)
+            for (uint32_t e = 0; e < live; ++e) sum[e] += src[sp * share + e];
+    }
     int64_t oa, ob, oc;
     batch_offsets(p, batch, oa, ob, oc);
     T* dst = C + oc + static_cast<int64_t>(m) * p.c_rs + col;
-    for (uint32_t e = 0; e < live; ++e) dst[e] = narrow_result<T>(sum[e]);
+    if (live == 4 && reinterpret_cast<uintptr_t>(dst) % (4 * sizeof(T)) == 0) {
+        T out[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) out[e] = narrow_result<T>(sum[e]);
+        using Quad = std::conditional_t<sizeof(T) == 2, uint2, uint4>;
+        Quad bits;
+        __builtin_memcpy(&bits, out, sizeof(Quad));
+        *reinterpret_cast<Quad*>(dst) = bits;
+    } else {
+        for (uint32_t e = 0; e < live; ++e) dst[e] = narrow_result<T>(sum[e]);
+    }
 }
 
 // Few tiles and a long K: each tile is shared by `splits` blocks.
@@ -536,17 +553,33 @@ int run16(const GemmProblem& p, const void* a, const void* b, void* c, hipStream
     // Tile height by M (a tile taller than M multiplies padding), large tiles only when they still give every CU work.
     const uint64_t big = static_cast<uint64_t>((p.M + 255) / 256) * ((p.N + 255) / 256) * p.batches;
     if (p.M > 192 && big >= 200) return pick_layout16<T, 256, 256, 2>(p, ak, bk, a, b, c, stream);
+    // Fewer large tiles than compute units: choose between the two smaller tiles and between whole K per block and a
+    // share of it, by a model of the time (microseconds): blocks on the busiest compute unit x steps per block x the
+    // measured time of one 64-wide step of that tile, a fixed start-up and write-out, and for shared K the second pass
+    // over the fp32 partial sums.
     const bool tall = p.M > 64;
-    const uint64_t tiles = tall ? static_cast<uint64_t>((p.M + 127) / 128) * ((p.N + 127) / 128) * p.batches
-                                : static_cast<uint64_t>((p.M + 63) / 64) * ((p.N + 127) / 128) * p.batches;
-    // too few tiles for the chip: a share of K per block while a block keeps four steps
-    uint64_t splits = tiles < 256 ? 256 / tiles : 1;
-    if (splits > p.K / 256) splits = p.K / 256;
-    if (splits > 1 && !p.row_bias) {
-        if (tall) return run16_split<T, 128>(p, ak, bk, static_cast<uint32_t>(splits), a, b, c, stream);
-        return run16_split<T, 64>(p, ak, bk, static_cast<uint32_t>(splits), a, b, c, stream);
+    const double steps_all = (p.K + 63) / 64;
+    double best_cost = 1e30;
+    int best_bm = tall ? 128 : 64;
+    uint32_t best_splits = 1;
+    for (int bm : {128, 64}) {
+        if (bm == 128 && !tall) continue;
+        const double step_us = bm == 128 ? 0.55 : 0.40;
+        const uint64_t tiles = static_cast<uint64_t>((p.M + bm - 1) / bm) * ((p.N + 127) / 128) * p.batches;
+        for (uint32_t splits : {1u, 2u, 4u, 8u, 16u}) {
+            if (splits > 1 && (p.row_bias || splits > p.K / 256)) break;
+            const double blocks = static_cast<double>(tiles) * splits;
+            const double rounds = static_cast<double>((static_cast<uint64_t>(blocks) + 255) / 256);
+            double cost = rounds * (steps_all / splits) * step_us + 5.0;
+            if (splits > 1) cost += 4.0 + (splits + 0.5) * static_cast<double>(p.M) * p.N * p.batches * 4.0 / 5.0e6;
+            if (cost < best_cost) { best_cost = cost; best_bm = bm; best_splits = splits; }
+        }
     }
-    if (tall) return pick_layout16<T, 128, 128, 2>(p, ak, bk, a, b, c, stream);
+    if (best_splits > 1) {
+        if (best_bm == 128) return run16_split<T, 128>(p, ak, bk, best_splits, a, b, c, stream);
+        return run16_split<T, 64>(p, ak, bk, best_splits, a, b, c, stream);
+    }
+    if (best_bm == 128) return pick_layout16<T, 128, 128, 2>(p, ak, bk, a, b, c, stream);
     return pick_layout16<T, 64, 128, 2>(p, ak, bk, a, b, c, stream);
 }
 

@@ -8,6 +8,7 @@ address = buffer + offset, strides in elements, size = element count,
 layout SINGLETON / CONTIGUOUS / STRIDED.
 """
 import ctypes as C
+import math
 
 import numpy as np
 
@@ -101,7 +102,7 @@ class Tensor:
         self.strides = contiguous_strides(shape) if strides is None else tuple(int(s) for s in strides)
         self.offset = int(offset)  # bytes
         self.buffer = None
-        self.nelements = int(np.prod(shape, dtype=np.int64)) if shape else 1
+        self.nelements = math.prod(shape)
 
     # ---- metadata -------------------------------------------------------
     @property
@@ -278,9 +279,9 @@ class Tensor:
             raise ValueError("view needs a contiguous tensor")
         shape = list(shape)
         if -1 in shape:
-            known = int(np.prod([s for s in shape if s != -1], dtype=np.int64))
+            known = math.prod(s for s in shape if s != -1)
             shape[shape.index(-1)] = self.nelements // known
-        if int(np.prod(shape, dtype=np.int64)) != self.nelements:
+        if math.prod(shape) != self.nelements:
             raise ValueError("view: element count differs")
         return self._view(shape, contiguous_strides(shape))
 
