@@ -147,8 +147,8 @@ def measured_value(name, key):
 
 def decoder_layer_entry(b, iters):
     """One Llama-3-8B decoder layer, seq 512, bf16, written with the operators (about 65 backend calls).
-    The time is wall-clock through this Python front end, which is what bounds it; the device-busy time of the
-    same calls comes from the committed kernel trace."""
+    The time is wall-clock through this Python front end; the device-busy time of the same calls comes from the
+    committed kernel trace."""
     from tannic_amd import decoder_layer as dl
     import support
     ta = b.ta
@@ -172,7 +172,7 @@ def decoder_layer_entry(b, iters):
     del out
     return {"op": "decoder layer bfloat16 seq 512 (hidden 4096, 32/8 heads, FFN 14336), composed from operators", "us": round(us, 1),
             "tflops": round(flops / us / 1e6, 2), "mfma_frac": round(flops / us / 1e6 / MFMA_PEAK_TFLOPS["bf16"], 4),
-            "bound": "host front end (one Python call per operator)", "device_busy_us": busy,
+            "bound": "mixed: matrix products plus about 45 launch-bound elementwise, reduction and copy kernels", "device_busy_us": busy,
             "device_busy_tflops": round(flops / busy / 1e6, 2) if busy else None}
 
 
