@@ -219,6 +219,25 @@ def elementwise_entries(b, dtype, iters):
         add("X - X2 (full)", b.raw_call("sub", [x, x2], y), 3 * nb)
         raw = C.create_string_buffer(ops.scalar_bytes(3, dtype), 16)
         add("3 * X (scale)", b.raw_call("scale", [x], y, scalar=abi.scalar_t(C.cast(raw, C.c_void_p), dtype.code)), 2 * nb)
+        del x2, y
+
+        # the whole chain as the front end evaluates it: eight operator nodes, each with its own destination
+        def chain():
+            t = ops.log(ops.add(ops.abs(x), one))
+            t = ops.add(t, ops.mul(z, z))
+            t = ops.sub(t, ops.exp(x))
+            return ops.add(t, ops.scale(x, 3))
+        for _ in range(2):
+            chain()
+        b.sync()
+        t0 = time.perf_counter()
+        for _ in range(3):
+            chain()
+        b.sync()
+        ms = (time.perf_counter() - t0) / 3 * 1e3
+        traffic = 18 * nb   # abs 2, +1 2, log 2, +Z*Z 2 (Z*Z is 4096 elements), exp 2, sub 3, scale 2, add 3
+        out.append({"op": f"chain log(|X|+1) + Z*Z - exp(X) + 3*X, 8 nodes {dtype}", "us": round(ms * 1e3, 1), "gbs": round(traffic / ms / 1e6, 1),
+                    "bound": "hbm", "frac": round(traffic / ms / 1e6 / HBM_PEAK_GBS, 4)})
     else:
         add("X + Z[1,4096,1] (broadcast)", b.raw_call("add", [x, z], y), 2 * nb)
         mask = ta.Tensor(ta.boolean, shape).initialize(b.device)
