@@ -57,7 +57,7 @@ def parse():
     ap.add_argument("--primary-only", action="store_true", help="skip the secondary workloads and the CPU baseline")
     ap.add_argument("--copy-only", action="store_true",
                     help="run only a plain 1 GiB -> 1 GiB contiguous copy (repack): the known-size kernel that calibrates the HBM byte counters")
-    ap.add_argument("--only", choices=["gemm", "conv", "elementwise", "reduce", "layer"],
+    ap.add_argument("--only", choices=["gemm", "conv", "elementwise", "reduce", "layer", "layer-one-pass"],
                     help="run one group of the secondary workloads alone and print its entries (for profiling that group)")
     return ap.parse_args()
 
@@ -138,14 +138,14 @@ def measured_value(name, key):
     """A number recorded in a committed profile summary under profiles/ (None if absent)."""
     try:
         for line in open(os.path.join(ROOT, "profiles", name)):
-            if line.strip().startswith(key):
+            if "=" in line and line.split("=")[0].strip() == key:
                 return float(line.split("=")[1])
     except OSError:
         pass
     return None
 
 
-def decoder_layer_entry(b, iters):
+def decoder_layer_entry(b, iters, composed=True, one_pass=True):
     """One Llama-3-8B decoder layer, seq 512, bf16, written with the operators (about 65 backend calls).
     The time is wall-clock through this Python front end; the device-busy time of the same calls comes from the
     committed kernel trace."""
@@ -159,21 +159,35 @@ def decoder_layer_entry(b, iters):
     x = b.filled(dtype, (1, seq, s.hidden), "normal", 0, 39, 1.0)
     cos, sin = dl.rotary_tables(s, seq, dtype, b.device)
     mask, one = dl.causal_mask(seq, dtype, b.device), ta.tensor(np.ones(1), dtype, b.device)
-    for _ in range(2):
-        dl.forward(s, w, x, cos, sin, mask, one)
-    b.sync()
-    t0 = time.perf_counter()
-    for _ in range(iters):
-        out = dl.forward(s, w, x, cos, sin, mask, one)
-    b.sync()
-    us = (time.perf_counter() - t0) / iters * 1e6
+
+    def timed(step):
+        for _ in range(2):
+            step()
+        b.sync()
+        t0 = time.perf_counter()
+        for _ in range(iters):
+            out = step()
+        b.sync()
+        del out
+        return (time.perf_counter() - t0) / iters * 1e6
+
     flops = dl.flop_count(s, seq)
-    busy = measured_value("decoder_layer_bf16_seq512_kernels.txt", "device_busy_us_per_layer")
-    del out
-    return {"op": "decoder layer bfloat16 seq 512 (hidden 4096, 32/8 heads, FFN 14336), composed from operators", "us": round(us, 1),
-            "tflops": round(flops / us / 1e6, 2), "mfma_frac": round(flops / us / 1e6 / MFMA_PEAK_TFLOPS["bf16"], 4),
-            "bound": "mixed: matrix products plus about 45 launch-bound elementwise, reduction and copy kernels", "device_busy_us": busy,
-            "device_busy_tflops": round(flops / busy / 1e6, 2) if busy else None}
+    entries = []
+    if composed:
+        us = timed(lambda: dl.forward(s, w, x, cos, sin, mask, one))
+        busy = measured_value("decoder_layer_bf16_seq512_kernels.txt", "device_busy_us_per_layer")
+        entries.append({"op": "decoder layer bfloat16 seq 512 (hidden 4096, 32/8 heads, FFN 14336), composed from operators", "us": round(us, 1),
+                        "tflops": round(flops / us / 1e6, 2), "mfma_frac": round(flops / us / 1e6 / MFMA_PEAK_TFLOPS["bf16"], 4),
+                        "bound": "mixed: matrix products plus about 45 launch-bound elementwise, reduction and copy kernels", "device_busy_us": busy,
+                        "device_busy_tflops": round(flops / busy / 1e6, 2) if busy else None})
+    if one_pass:
+        us = timed(lambda: dl.forward_fused(s, w, x, cos, sin, mask))
+        busy = measured_value("decoder_layer_one_pass_bf16_seq512_kernels.txt", "device_busy_us_per_layer")
+        entries.append({"op": "the same layer with the one-pass rms_norm / rope / softmax / swiglu operators (no counterpart in the reference)",
+                        "us": round(us, 1), "tflops": round(flops / us / 1e6, 2), "mfma_frac": round(flops / us / 1e6 / MFMA_PEAK_TFLOPS["bf16"], 4),
+                        "bound": "matrix products plus 12 row-wise, elementwise and copy kernels", "device_busy_us": busy,
+                        "device_busy_tflops": round(flops / busy / 1e6, 2) if busy else None})
+    return entries
 
 
 def conv_entry(b, dtype, name, xs, ws, stride, pad, iters):
@@ -315,8 +329,8 @@ def secondary(b, only):
     if only in (None, "reduce"):
         for dtype in (ta.float32, ta.float16):
             work += reduction_entries(b, dtype, 10)
-    if only in (None, "layer"):
-        work.append(decoder_layer_entry(b, 20))
+    if only in (None, "layer", "layer-one-pass"):
+        work.extend(decoder_layer_entry(b, 20, composed=only != "layer-one-pass", one_pass=only != "layer"))
     return work
 
 

@@ -302,6 +302,28 @@ int tannic_hip_conv2d(const tannic_tensor_t* signal, const tannic_tensor_t* kern
 int tannic_hip_conv2d_biased(const tannic_tensor_t* signal, const tannic_tensor_t* kernel, const tannic_tensor_t* bias,
                              tannic_tensor_t* dst, tannic_stream_t stream, const size_t pad[2], const size_t stride[2]);
 
+/* ------------------------------------------------------------------ *
+ * Operators with no counterpart in the reference.  A Tannic program
+ * spells them today as chains of the operators above (there is no
+ * division, no cast, no softmax in include/tannic/*.hpp); each is one
+ * pass here.  16- and 32-bit types are evaluated in float, float64 in
+ * double, and rounded once.
+ * ------------------------------------------------------------------ */
+/* dst = a / b, broadcasting like mul; the floating pairs of mul's table (src/cpu/ops-binary.cpp:286-360). */
+int tannic_hip_div(const tannic_tensor_t* a, const tannic_tensor_t* b, tannic_tensor_t* dst, tannic_stream_t stream);
+/* dst[i] = src[i] in dst's dtype, any two real types; dst contiguous with src's shape.  Float to integer truncates
+ * toward zero, out-of-range values give the nearest end of the range, NaN gives 0. */
+int tannic_hip_cast(const tannic_tensor_t* src, tannic_tensor_t* dst, tannic_stream_t stream);
+/* dst = gate / (1 + exp(-gate)) * up, broadcasting like mul; one floating dtype for all three. */
+int tannic_hip_swiglu(const tannic_tensor_t* gate, const tannic_tensor_t* up, tannic_tensor_t* dst, tannic_stream_t stream);
+/* dst[.., i] = x[.., i] / sqrt(mean_i(x[.., i]^2) + eps) * gain[i] over the last axis; x, dst contiguous. */
+int tannic_hip_rms_norm(const tannic_tensor_t* x, const tannic_tensor_t* gain, tannic_tensor_t* dst, tannic_stream_t stream, float eps);
+/* softmax over the last axis of s = x * scale + mask; mask is NULL or a contiguous [Q, L] table for x [.., Q, L]. */
+int tannic_hip_softmax(const tannic_tensor_t* x, const tannic_tensor_t* mask, tannic_tensor_t* dst, tannic_stream_t stream, float scale);
+/* Rotary embedding of x [.., n, d] (any strides) by cos, sin [n, d/2]: the pair (x[2i], x[2i+1]) turns by the
+ * angle of position n; dst contiguous. */
+int tannic_hip_rope(const tannic_tensor_t* x, const tannic_tensor_t* cos, const tannic_tensor_t* sin, tannic_tensor_t* dst, tannic_stream_t stream);
+
 #ifdef __cplusplus
 } /* extern "C" */
 #endif

@@ -118,6 +118,13 @@ def kernel_signatures(with_stream):
     sig["conv1d"] = (C.c_int, [TP, TP, TP] + s + [C.c_size_t, C.c_size_t])
     sig["conv2d"] = (C.c_int, [TP, TP, TP] + s + [SIZE2, SIZE2])
     sig["conv2d_biased"] = (C.c_int, [TP, TP, TP, TP] + s + [SIZE2, SIZE2])
+    # operators without a twin in the reference
+    sig["div"] = (C.c_int, [TP, TP, TP] + s)
+    sig["swiglu"] = (C.c_int, [TP, TP, TP] + s)
+    sig["cast"] = (C.c_int, [TP, TP] + s)
+    sig["rms_norm"] = (C.c_int, [TP, TP, TP] + s + [C.c_float])
+    sig["softmax"] = (C.c_int, [TP, TP, TP] + s + [C.c_float])   # the second operand (mask) may be NULL
+    sig["rope"] = (C.c_int, [TP, TP, TP, TP] + s)
     return sig
 
 

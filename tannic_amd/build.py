@@ -34,6 +34,9 @@ UNITS = [
     ("binary.hip", "binary_mul.o", EXACT + ["-DTH_BINARY_ONLY=2"]),
     ("binary.hip", "binary_pow.o", EXACT + ["-DTH_BINARY_ONLY=3"]),
     ("misc.hip", "misc.o", EXACT),
+    ("extended.hip", "extended_pairs.o", EXACT + ["-DTH_EXTENDED_ONLY=0"]),
+    ("extended.hip", "extended_cast.o", EXACT + ["-DTH_EXTENDED_ONLY=1"]),
+    ("rows.hip", "rows.o", []),
     ("reduce.hip", "reduce.o", []),
     ("shape_ops.hip", "shape_ops.o", []),
     ("gemm.hip", "gemm.o", []),

@@ -5,6 +5,7 @@
 
 #include <hip/hip_runtime.h>
 
+#include <atomic>
 #include <cstdint>
 #include <cstdio>
 #include <cstring>
@@ -31,6 +32,17 @@ void set_error_text(const char* text);
     } while (0)
 
 inline hipStream_t as_stream(tannic_stream_t s) { return reinterpret_cast<hipStream_t>(s.address); }
+
+// Raises a kernel's dynamic LDS limit, once per device: the attribute belongs to the device's copy of the code.
+inline int raise_lds_limit(const void* kernel, size_t bytes, std::atomic<uint64_t>& done) {
+    int device = 0;
+    TH_TRY(hipGetDevice(&device));
+    const uint64_t bit = uint64_t(1) << (device & 63);
+    if (done.load(std::memory_order_acquire) & bit) return TANNIC_SUCCESS;
+    TH_TRY(hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(bytes)));
+    done.fetch_or(bit, std::memory_order_release);
+    return TANNIC_SUCCESS;
+}
 
 // Result of the launch that was just enqueued.
 inline int launch_status(const char* what) {

@@ -305,11 +305,8 @@ __global__ __launch_bounds__(kK3Threads) void conv2d_k3_kernel(const T* x, const
 template <class T, int TN>
 int launch_k3(const ConvProblem& p, const K3Plan& q, size_t lds, uint32_t blocks, const void* x, const void* w, const void* bias, void* y, hipStream_t stream) {
     auto kernel = conv2d_k3_kernel<T, TN>;
-    static bool configured = false;
-    if (!configured) {
-        TH_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
-        configured = true;
-    }
+    static std::atomic<uint64_t> configured{0};
+    if (int rc = raise_lds_limit(reinterpret_cast<const void*>(kernel), 160 * 1024, configured)) return rc;
     hipLaunchKernelGGL(kernel, dim3(blocks), dim3(kK3Threads), lds, stream, static_cast<const T*>(x), static_cast<const T*>(w), static_cast<const T*>(bias),
                        static_cast<T*>(y), p, q);
     return launch_status("conv2d_k3_kernel");

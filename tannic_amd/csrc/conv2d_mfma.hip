@@ -249,12 +249,9 @@ int launch_conv16(const ConvProblem& p, uint32_t K, uint32_t pixels, const void*
     const size_t lds = sizeof(T) * 2 * (BCO + kConvBP) * kConvBK + sizeof(Tap) * ksteps * kConvBK;
     const uint32_t co_tiles = (p.O + BCO - 1) / BCO, p_tiles = (pixels + kConvBP - 1) / kConvBP;
     auto kernel = conv2d_mfma16_kernel<T, BCO, WV>;
-    static bool configured = false;
-    if (!configured) {
-        const size_t most = sizeof(T) * 2 * (BCO + kConvBP) * kConvBK + sizeof(Tap) * kMaxTableK;
-        TH_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(most)));
-        configured = true;
-    }
+    static std::atomic<uint64_t> configured{0};
+    const size_t most = sizeof(T) * 2 * (BCO + kConvBP) * kConvBK + sizeof(Tap) * kMaxTableK;
+    if (int rc = raise_lds_limit(reinterpret_cast<const void*>(kernel), most, configured)) return rc;
     hipLaunchKernelGGL(kernel, dim3(co_tiles * p_tiles), dim3(kConvThreads), lds, stream, static_cast<const T*>(x), static_cast<const T*>(w),
                        static_cast<const T*>(bias), static_cast<T*>(y), p, K, pixels, co_tiles);
     return launch_status("conv2d_mfma16_kernel");

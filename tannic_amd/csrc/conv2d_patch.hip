@@ -194,11 +194,8 @@ __global__ __launch_bounds__(kPatchThreads, 2) void conv2d_patch_kernel(const T*
 template <class T, int BCO>
 int launch_patch(const ConvProblem& p, const PatchPlan& q, size_t lds, const void* x, const T* wt, const void* bias, void* y, hipStream_t stream) {
     auto kernel = conv2d_patch_kernel<T, BCO>;
-    static bool configured = false;
-    if (!configured) {
-        TH_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
-        configured = true;
-    }
+    static std::atomic<uint64_t> configured{0};
+    if (int rc = raise_lds_limit(reinterpret_cast<const void*>(kernel), 160 * 1024, configured)) return rc;
     const uint32_t grid = p.N * q.row_blocks * q.co_tiles;
     hipLaunchKernelGGL(kernel, dim3(grid), dim3(kPatchThreads), lds, stream, static_cast<const T*>(x), wt, static_cast<const T*>(bias),
                        static_cast<T*>(y), p, q);

@@ -292,11 +292,8 @@ __global__ __launch_bounds__(kResThreads) void conv2d_resident_kernel(const T* x
 template <class T, int BCO, int WSPLIT, int PASSES>
 int launch_resident(const ConvProblem& p, const ResidentPlan& q, size_t lds, const void* x, const T* wt, const void* bias, void* y, hipStream_t stream) {
     auto kernel = conv2d_resident_kernel<T, BCO, WSPLIT, PASSES>;
-    static bool configured = false;
-    if (!configured) {
-        TH_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
-        configured = true;
-    }
+    static std::atomic<uint64_t> configured{0};
+    if (int rc = raise_lds_limit(reinterpret_cast<const void*>(kernel), 160 * 1024, configured)) return rc;
     hipLaunchKernelGGL(kernel, dim3(q.workers * q.co_tiles), dim3(kResThreads), lds, stream, static_cast<const T*>(x), wt, static_cast<const T*>(bias),
                        static_cast<T*>(y), p, q);
     return launch_status("conv2d_resident_kernel");

@@ -273,11 +273,8 @@ __global__ __launch_bounds__(kStemThreads, 2) void conv2d_stem_kernel(const T* x
 template <class T, int NS>
 int launch_stem(const ConvProblem& p, const StemPlan& q, uint32_t blocks, size_t lds, const void* x, const void* w, const void* bias, void* y, hipStream_t stream) {
     auto kernel = conv2d_stem_kernel<T, NS>;
-    static bool configured = false;
-    if (!configured) {
-        TH_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, 64 * 1024));
-        configured = true;
-    }
+    static std::atomic<uint64_t> configured{0};
+    if (int rc = raise_lds_limit(reinterpret_cast<const void*>(kernel), 64 * 1024, configured)) return rc;
     hipLaunchKernelGGL(kernel, dim3(blocks), dim3(kStemThreads), lds, stream, static_cast<const T*>(x), static_cast<const T*>(w), static_cast<const T*>(bias),
                        static_cast<T*>(y), p, q);
     return launch_status("conv2d_stem_kernel");

@@ -453,11 +453,8 @@ int launch16(const GemmProblem& p, const void* a, const void* b, void* c, hipStr
     constexpr size_t stage_bytes = sizeof(T) * 2 * WAVES_N * (BM / 2) * (BN / WAVES_N + 8);
     constexpr size_t lds_bytes = (sizeof(T) == 2 && stage_bytes > tile_bytes) ? stage_bytes : tile_bytes;   // fp32 results are not staged
     auto kernel = gemm16_kernel<T, BM, BN, WAVES_N, AK, BK_, SPLIT>;
-    static bool configured = false;
-    if (!configured) {
-        TH_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes)));
-        configured = true;
-    }
+    static std::atomic<uint64_t> configured{0};
+    if (int rc = raise_lds_limit(reinterpret_cast<const void*>(kernel), lds_bytes, configured)) return rc;
     hipLaunchKernelGGL(kernel, dim3(tiles_m * tiles_n * sk.splits, p.batches), dim3(128 * WAVES_N), lds_bytes, stream, static_cast<const T*>(a),
                        static_cast<const T*>(b), static_cast<T*>(c), p, tiles_m, tiles_n, sk);
     return launch_status("gemm16_kernel");
@@ -552,6 +549,12 @@ int run16(const GemmProblem& p, const void* a, const void* b, void* c, hipStream
     if (p.batches > 65535) return TANNIC_UNSUPPORTED_DTYPE;
     // Tile height by M (a tile taller than M multiplies padding), large tiles only when they still give every CU work.
     const uint64_t big = static_cast<uint64_t>((p.M + 255) / 256) * ((p.N + 255) / 256) * p.batches;
+#ifdef TH_EXP
+    if (const char* e = getenv("TH_TILE")) {
+        if (e[0] == '1') return pick_layout16<T, 128, 128, 2>(p, ak, bk, a, b, c, stream);
+        if (e[0] == '6') return pick_layout16<T, 64, 128, 2>(p, ak, bk, a, b, c, stream);
+    }
+#endif
     if (p.M > 192 && big >= 200) return pick_layout16<T, 256, 256, 2>(p, ak, bk, a, b, c, stream);
     // Fewer large tiles than compute units: choose between the two smaller tiles and between whole K per block and a
     // share of it, by a model of the time (microseconds): blocks on the busiest compute unit x steps per block x the

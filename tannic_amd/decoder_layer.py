@@ -76,6 +76,25 @@ def silu(g, one):
     return ops.mul(ops.mul(g, sg), sg)
 
 
+def forward_fused(s, w, x, cos, sin, mask):
+    """The same layer with the device library's one-pass operators (``ops.rms_norm``, ``ops.rope``, ``ops.softmax``,
+    ``ops.swiglu``) in place of the chains; these have no counterpart in the reference's front end."""
+    _, seq, _ = x.shape
+    xn = ops.rms_norm(x, w["g1"], s.eps)
+    q = ops.matmul(xn, w["wq"].transpose()).view(1, seq, s.heads, s.head_dim).transpose(1, 2)
+    k = ops.matmul(xn, w["wk"].transpose()).view(1, seq, s.kv_heads, s.head_dim).transpose(1, 2)
+    v = ops.matmul(xn, w["wv"].transpose()).view(1, seq, s.kv_heads, s.head_dim).transpose(1, 2)
+    q, k = ops.rope(q, cos, sin), ops.rope(k, cos, sin)
+    group = s.heads // s.kv_heads
+    k, v = ops.repeat(k, group, 1), ops.repeat(v, group, 1)
+    p = ops.softmax(ops.matmul(q, k.transpose(-1, -2)), mask, 1.0 / math.sqrt(s.head_dim))
+    o = ops.repack(ops.matmul(p, v).transpose(1, 2)).view(1, seq, s.heads * s.head_dim)
+    h = ops.add(x, ops.matmul(o, w["wo"].transpose()))
+    hn = ops.rms_norm(h, w["g2"], s.eps)
+    act = ops.swiglu(ops.matmul(hn, w["w1"].transpose()), ops.matmul(hn, w["w3"].transpose()))
+    return ops.add(h, ops.matmul(act, w["w2"].transpose()))
+
+
 def forward(s, w, x, cos, sin, mask, one):
     """x: [1, seq, hidden].  Returns the layer's output, same shape and dtype."""
     _, seq, _ = x.shape

@@ -448,3 +448,54 @@ def allclose(a, b, rtol=1e-5, atol=1e-8):
     if r < 0:
         raise TannicError("Unsupported dtype")
     return bool(r)
+
+
+# ---- operators without a twin in the reference ---------------------------------------
+# A Tannic program has no division, cast, softmax or normalisation (``include/tannic/functions.hpp``,
+# ``include/tannic/operations.hpp``) and spells them as chains; these are the one-pass forms the device library adds.
+def div(a, b):
+    """``a / b`` with the broadcasting and promotion of the other binary operations; floating types only."""
+    env = _resolve(a, b)
+    return _call("div", env, [a, b], _new(promote(a.dtype, b.dtype), broadcast(a.shape, b.shape), env))
+
+
+def cast(x, dtype):
+    """``x`` in ``dtype`` (real types), contiguous."""
+    return _call("cast", x.environment, [x], _new(dtype, x.shape, x.environment))
+
+
+def swiglu(gate, up):
+    """``gate / (1 + exp(-gate)) * up``."""
+    env = _resolve(gate, up)
+    return _call("swiglu", env, [gate, up], _new(gate.dtype, broadcast(gate.shape, up.shape), env))
+
+
+def rms_norm(x, gain, eps=1e-5):
+    """``x / sqrt(mean(x**2, -1) + eps) * gain`` over the last axis of a contiguous ``x``."""
+    env = _resolve(x, gain)
+    return _call("rms_norm", env, [x, gain], _new(x.dtype, x.shape, env), extra=(C.c_float(eps),))
+
+
+def softmax(x, mask=None, scale=1.0):
+    """Softmax over the last axis of ``x * scale + mask``; ``mask`` is ``None`` or ``[x.shape[-2], x.shape[-1]]``."""
+    env = _resolve(x) if mask is None else _resolve(x, mask)
+    if not isinstance(env, Device):
+        raise BackendError("softmax: operands are on the host and tannic_amd holds device kernels only")
+    dst = _new(x.dtype, x.shape, env)
+    dx, dd = x.descriptor(), dst.descriptor()
+    dm = None if mask is None else mask.descriptor()
+    lib = library()
+    dvc = env.structure()
+    stream = lib.pop_stream(C.byref(dvc))
+    status = lib.kernels["softmax"](C.byref(dx), None if dm is None else C.byref(dm), C.byref(dd), stream, C.c_float(scale))
+    lib.put_stream(C.byref(dvc), stream)
+    if status != abi.SUCCESS:
+        detail = lib.error_message() if status == abi.ERROR else ""
+        raise TannicError(f"Unsupported dtype (softmax: {abi.STATUS_NAMES[status]}{' ' + detail if detail else ''})")
+    return dst
+
+
+def rope(x, cos, sin):
+    """Rotary embedding of ``x [.., n, d]`` by ``cos, sin [n, d/2]`` on the pairs ``(2i, 2i+1)``; contiguous result."""
+    env = _resolve(x, cos, sin)
+    return _call("rope", env, [x, cos, sin], _new(x.dtype, x.shape, env))

@@ -53,3 +53,17 @@ def test_layer_is_causal(device):
     b = dl.forward(s, w, ta.tensor(xv, ta.float32, device), cos, sin, mask, one).numpy()
     np.testing.assert_array_equal(a[0, :10], b[0, :10])
     assert np.abs(a[0, 10:] - b[0, 10:]).max() > 1e-3
+
+
+@pytest.mark.parametrize("dtype,bar", [(ta.float32, 2e-4), (ta.bfloat16, 0.06)], ids=["float32", "bfloat16"])
+def test_one_pass_operators_give_the_same_layer(device, oracle, dtype, bar):
+    """The layer written with rms_norm / rope / softmax / swiglu against the checker's evaluation of the chains."""
+    s = dl.LayerShape(hidden=256, heads=4, kv_heads=2, head_dim=64, ffn=512)
+    seq = 40
+    host = build(s, seq, dtype, ta.Host(), 5)
+    w, x, cos, sin, mask, one = build(s, seq, dtype, device, 5)
+    with support.use_functions(oracle):
+        want = dl.forward(s, *host).numpy().astype(np.float64)
+    got = dl.forward_fused(s, w, x, cos, sin, mask).numpy().astype(np.float64)
+    assert got.shape == want.shape and np.isfinite(got).all()
+    assert np.abs(got - want).max() <= bar * want.std(), (np.abs(got - want).max(), want.std())
