@@ -47,6 +47,7 @@ UNITS = [
     ("conv2d_patch.hip", "conv2d_patch.o", []),
     ("conv2d_resident.hip", "conv2d_resident.o", []),
     ("conv2d_k3.hip", "conv2d_k3.o", []),
+    ("conv2d_k1.hip", "conv2d_k1.o", []),
     ("conv2d_pointwise.hip", "conv2d_pointwise.o", []),
     ("conv2d_stem.hip", "conv2d_stem.o", []),
     ("conv2d_unfold.hip", "conv2d_unfold.o", []),

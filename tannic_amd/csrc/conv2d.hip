@@ -89,11 +89,12 @@ static int conv2d_entry(const tannic_tensor_t* x, const tannic_tensor_t* w, cons
     // the bias is read as b[co]: element stride 1 (src/cpu/conv2d.cpp:90)
     const void* pb = bias ? bias->address : nullptr;
     hipStream_t s = as_stream(stream);
-    // Kernels in order of preference.  A 1x1 kernel has no tap to amortise a staged patch over:
-    // the gathering implicit GEMM serves it better than the LDS-patch kernels.
+    // Kernels in order of preference.  A 1x1 kernel has no tap to amortise a staged patch over: its weights stay in
+    // registers when they fit (conv2d_k1.hip), otherwise it is a matrix product per image (conv2d_pointwise.hip).
     int status = TANNIC_UNSUPPORTED_DTYPE;
     const bool pointwise = p.KH == 1 && p.KW == 1;
-    if (pointwise) status = conv2d_pointwise(p, x->dtype, x->address, w->address, pb, y->address, s);
+    if (pointwise) status = conv2d_k1(p, x->dtype, x->address, w->address, pb, y->address, s);
+    if (pointwise && status == TANNIC_UNSUPPORTED_DTYPE) status = conv2d_pointwise(p, x->dtype, x->address, w->address, pb, y->address, s);
     if (status != TANNIC_UNSUPPORTED_DTYPE) return status;
     if (!pointwise) status = conv2d_stem(p, x->dtype, x->address, w->address, pb, y->address, s);
     if (status != TANNIC_UNSUPPORTED_DTYPE) return status;

@@ -1,0 +1,323 @@
+// conv2d with a 1x1 kernel on MFMA, 16-bit signals, up to 256 input channels, horizontal/vertical stride 1 or 2.
+//
+// The layer is a product  y[n] (O x pixels) = w (O x C) * x[n] (C x sampled pixels)  with a short inner dimension:
+// a tiled matrix multiply spends as long filling and draining its tile as multiplying, and a strided layer would
+// first need the sampled pixels gathered into a dense copy.  Here the weights never move: a wavefront keeps the
+// 64 x C weights of its output channels in registers as MFMA fragments for the whole launch (C <= 256: at most 128
+// registers), and the block (four wavefronts, 256 output channels) walks over tiles of 64 pixels:
+//   * the C x 64 signal tile is read as 8 channels x 8 pixels micro-blocks, one per thread; with stride 2 the eight
+//     pixels are the even elements of two 16-byte loads (four pixels each; the two groups may sit on different rows),
+//   * transposed in registers and written to LDS pixel-major, [64-channel panel][pixel][64 channels], 16-byte slots
+//     XOR-swizzled by the pixel number so that fragment reads are bank-conflict free,
+//   * multiplied: the pixel fragment is the MFMA's first operand, so a lane's accumulators are runs of four
+//     consecutive pixels of one output channel,
+//   * rounded into LDS as [channel][pixel] and written out as whole rows of the NCHW result, 16 bytes per lane.
+// The loads of two tiles are in flight at any time (a tile's loads are issued three tiles ahead of its product) and a
+// tile's transposition into the other LDS buffer is spread between the MFMAs of the tile before it.  HBM-bound: every sampled input row
+// is read once per group of 256 output channels, the result written once.
+#include "conv_common.hpp"
+
+namespace th {
+
+typedef _Float16 half8p __attribute__((ext_vector_type(8)));
+typedef __bf16 bfloat8p __attribute__((ext_vector_type(8)));
+typedef float float16p __attribute__((ext_vector_type(16)));
+typedef unsigned int uint4p __attribute__((ext_vector_type(4)));
+typedef unsigned int uint2p __attribute__((ext_vector_type(2)));
+
+template <class T> __device__ inline float16p k1_mfma(uint4p a, uint4p b, float16p c) {
+    if constexpr (std::is_same_v<T, f16>) {
+        half8p x, y;
+        __builtin_memcpy(&x, &a, 16);
+        __builtin_memcpy(&y, &b, 16);
+        return __builtin_amdgcn_mfma_f32_32x32x16_f16(x, y, c, 0, 0, 0);
+    } else {
+        bfloat8p x, y;
+        __builtin_memcpy(&x, &a, 16);
+        __builtin_memcpy(&y, &b, 16);
+        return __builtin_amdgcn_mfma_f32_32x32x16_bf16(x, y, c, 0, 0, 0);
+    }
+}
+
+template <int N, class F, int I = 0>
+__device__ inline void k1_static_for(F&& f) {
+    if constexpr (I < N) {
+        f(std::integral_constant<int, I>{});
+        k1_static_for<N, F, I + 1>(static_cast<F&&>(f));
+    }
+}
+
+constexpr int kK1Threads = 256;
+constexpr int kK1Pixels = 64;          // pixels per tile
+constexpr int kK1CoWave = 64;          // output channels per wavefront
+constexpr int kK1CoBlock = 256;        // per block
+constexpr int kK1Panel = 64 * 64;      // elements of one 64-channel panel of a tile
+constexpr int kK1Pitch = kK1Pixels + 8;   // staged result rows, elements
+
+struct K1Plan {
+    uint32_t pixels;            // HO * WO
+    uint32_t tiles, workers;    // (image, 64-pixel range) pairs; blocks per group of 256 output channels
+    FastDiv div_wo, div_tiles_per_image;
+};
+
+// element offset of 16-byte slot `kc` of pixel `px` in a panel: rows of 128 bytes, slots swizzled so that both the
+// fragment reads (16 consecutive pixels, one slot) and the transposing writes (8 pixel blocks x 2 channel blocks,
+// odd pixel blocks one pixel ahead) of 16 lanes cover all 64 banks
+__device__ inline uint32_t k1_offset(uint32_t px, uint32_t kc) { return px * 64u + ((kc ^ (((px >> 1) ^ (px >> 3)) & 7u)) * 8u); }
+
+template <class T, int KSTEPS, int S>
+__global__ __launch_bounds__(kK1Threads) void conv2d_k1_kernel(const T* x, const T* w, const T* bias, T* y, ConvProblem p, K1Plan q) {
+    constexpr int C = KSTEPS * 16;
+    constexpr int PANELS = C / 64;
+    constexpr int LOADS = S;                                  // 16-byte loads per channel of a micro-block
+    constexpr uint32_t BUFFER = PANELS * kK1Panel;             // elements of one signal tile in LDS
+    extern __shared__ __align__(16) unsigned char k1_lds[];
+    T* lds = reinterpret_cast<T*>(k1_lds);
+    const int wave = threadIdx.x / 64, lane = threadIdx.x % 64;
+    T* stage = lds + 2 * BUFFER + wave * (kK1CoWave * kK1Pitch);
+
+    const uint32_t group = blockIdx.x / q.workers, worker = blockIdx.x % q.workers;
+    const uint32_t co0 = group * kK1CoBlock + wave * kK1CoWave;
+
+    // ---- this thread's micro-block: 8 channels x 8 pixels ----------------------------------------
+    // C / 8 channel blocks x 8 pixel blocks; with fewer than 256 channels the other threads repeat a micro-block's
+    // loads and skip its writes, so that every wavefront issues the same memory operations in every tile
+    const bool mine = threadIdx.x < C;
+    const uint32_t pxb = threadIdx.x % 8, kb = (threadIdx.x % C) / 8;
+    const int64_t cstep = p.xs[1];
+    const T* src[LOADS];
+    uint4p raw[2][8][LOADS];   // two tiles on their way from HBM
+
+    auto locate = [&](uint32_t tile) {
+        uint32_t n, pt;
+        q.div_tiles_per_image.divmod(tile, n, pt);
+        const T* image = x + static_cast<int64_t>(n) * p.xs[0] + static_cast<int64_t>(kb * 8) * cstep;
+#pragma unroll
+        for (int g = 0; g < LOADS; ++g) {
+            uint32_t pix = pt * kK1Pixels + pxb * 8 + (S == 2 ? 4 * g : 0);
+            if (pix >= q.pixels) pix = 0;                    // past the image: loads something valid, never stored
+            uint32_t oh, ow;
+            q.div_wo.divmod(pix, oh, ow);
+            src[g] = image + static_cast<int64_t>(oh * p.stride_h) * p.xs[2] + ow * S;
+        }
+    };
+    auto fetch = [&](auto set_, uint32_t tile) {
+        constexpr int set = decltype(set_)::value;
+        // never skipped: the count of memory operations between a tile's loads and their use is the same on every
+        // path, which lets the wait before the use leave the younger loads and stores in flight
+        locate(tile < q.tiles ? tile : q.tiles - 1);
+#pragma unroll
+        for (int kk = 0; kk < 8; ++kk)
+#pragma unroll
+            for (int g = 0; g < LOADS; ++g) raw[set][kk][g] = *reinterpret_cast<const uint4p*>(src[g] + kk * cstep);
+    };
+    // records 2m and 2m+1 of the transposed micro-block (pixels 2m, 2m+1; this thread's 8 channels): two 16-byte LDS
+    // writes; threads of odd pixel blocks write the odd pixel first, which spreads a write over all banks
+    auto commit_pair = [&](auto set_, auto m_, T* buffer) {
+        constexpr int set = decltype(set_)::value, m = decltype(m_)::value;
+        if (!mine) return;
+        uint32_t words[2][4];
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            const int e = 2 * m + h;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                uint32_t a[4], b[4];
+                __builtin_memcpy(a, &raw[set][2 * j][S == 2 ? e / 4 : 0], 16);
+                __builtin_memcpy(b, &raw[set][2 * j + 1][S == 2 ? e / 4 : 0], 16);
+                if (S == 2) words[h][j] = (a[e % 4] & 0xFFFFu) | (b[e % 4] << 16);        // even elements only
+                else if (e % 2 == 0) words[h][j] = (a[e / 2] & 0xFFFFu) | (b[e / 2] << 16);
+                else words[h][j] = (a[e / 2] >> 16) | (b[e / 2] & 0xFFFF0000u);
+            }
+        }
+        const bool odd = pxb & 1;
+        T* panel = buffer + (kb / 8) * kK1Panel;
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            uint32_t out[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) out[j] = odd ? words[1 - h][j] : words[h][j];
+            uint4p v;
+            __builtin_memcpy(&v, out, 16);
+            *reinterpret_cast<uint4p*>(panel + k1_offset(pxb * 8 + 2 * m + (odd ? 1 - h : h), kb % 8)) = v;
+        }
+    };
+    using Zero = std::integral_constant<int, 0>;
+    using One = std::integral_constant<int, 1>;
+
+    uint32_t tile = worker;
+    if (tile >= q.tiles) return;    // whole block: no barrier has been reached
+    // the first two signal tiles start their way from HBM before the weights are asked for
+    fetch(Zero{}, tile);
+    fetch(One{}, tile + q.workers);
+
+    // ---- the wavefront's weights, for the whole launch: 64 rows x C as MFMA fragments ---------------
+    uint4p afrag[2][KSTEPS];
+    float start[2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+        const uint32_t co = co0 + 32 * i + lane % 32;
+        const T* row = w + static_cast<int64_t>(co) * p.ws[0] + 8 * (lane / 32);
+#pragma unroll
+        for (int ks = 0; ks < KSTEPS; ++ks) afrag[i][ks] = *reinterpret_cast<const uint4p*>(row + ks * 16);
+        start[i] = bias ? static_cast<float>(widen(bias[co])) : 0.0f;
+    }
+
+    k1_static_for<4>([&](auto m_) { commit_pair(Zero{}, m_, lds); });
+    // The weights have arrived before the loop starts; said here, outside any branch, so that no wait for them is
+    // placed inside the loop, where it would also wait for the signal loads that are meant to stay in flight.
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int ks = 0; ks < KSTEPS; ++ks) asm volatile("" : "+v"(afrag[i][ks]));
+    fetch(Zero{}, tile + 2 * q.workers);
+    __syncthreads();
+
+    // One tile: multiply from LDS buffer PAR; between the MFMAs of the second half the next tile (registers, set
+    // 1 - PAR) is transposed into the other buffer; then those registers start loading the tile three ahead, and
+    // the result is rounded, staged as [channel][pixel] and written as whole rows.
+    auto one_tile = [&](auto par_) -> bool {
+        constexpr int PAR = decltype(par_)::value;
+        using Next = std::integral_constant<int, 1 - PAR>;
+        const uint32_t next = tile + q.workers;
+        const bool more = next < q.tiles;
+        float16p acc[2][2];
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+#pragma unroll
+            for (int j = 0; j < 2; ++j)
+#pragma unroll
+                for (int v = 0; v < 16; ++v) acc[i][j][v] = start[i];
+        const T* buffer = lds + PAR * BUFFER;
+        T* other = lds + (1 - PAR) * BUFFER;
+        uint4p bfrag[2][2];   // [step parity][pixel tile]: the fragments of a step are read during the step before
+        auto read_fragments = [&](auto ks_) {
+            constexpr int ks = decltype(ks_)::value;
+            const T* panel = buffer + (ks / 4) * kK1Panel;
+            const uint32_t kc = (ks % 4) * 2 + lane / 32;
+#pragma unroll
+            for (int j = 0; j < 2; ++j) bfrag[ks % 2][j] = *reinterpret_cast<const uint4p*>(panel + k1_offset(32 * j + lane % 32, kc));
+        };
+        read_fragments(Zero{});
+        k1_static_for<KSTEPS>([&](auto ks_) {
+            constexpr int ks = decltype(ks_)::value;
+            if constexpr (ks + 1 < KSTEPS) read_fragments(std::integral_constant<int, ks + 1>{});
+#pragma unroll
+            for (int i = 0; i < 2; ++i)
+#pragma unroll
+                for (int j = 0; j < 2; ++j) acc[i][j] = k1_mfma<T>(bfrag[ks % 2][j], afrag[i][ks], acc[i][j]);
+            constexpr int HALF = KSTEPS / 2;
+            if constexpr (ks >= HALF) {
+                // pair m goes after step HALF + m * HALF / 4
+                if (more) k1_static_for<4>([&](auto m_) {
+                    if constexpr (HALF + decltype(m_)::value * HALF / 4 == ks) commit_pair(Next{}, m_, other);
+                });
+            }
+        });
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+#pragma unroll
+            for (int j = 0; j < 2; ++j)
+#pragma unroll
+                for (int v4 = 0; v4 < 4; ++v4) {
+                    T four[4];
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) four[e] = narrow_result<T>(acc[i][j][4 * v4 + e]);
+                    uint2p bits;
+                    __builtin_memcpy(&bits, four, 8);
+                    *reinterpret_cast<uint2p*>(stage + (32 * i + lane % 32) * kK1Pitch + 32 * j + 8 * v4 + 4 * (lane / 32)) = bits;
+                }
+        __syncthreads();   // staged rows complete; the next tile's buffer is complete; this tile's buffer is free
+        {
+            // a row of the tile is eight 16-byte pieces; in the last tile of an image the lanes of the missing pieces
+            // repeat the last present one (same bytes to the same address) instead of being switched off
+            uint32_t n, pt;
+            q.div_tiles_per_image.divmod(tile, n, pt);
+            const uint32_t present = (q.pixels - pt * kK1Pixels) / 8;     // >= 1
+            const uint32_t piece = lane % 8 < present ? lane % 8 : present - 1;
+            T* out = y + static_cast<int64_t>(n) * p.ys[0] + pt * kK1Pixels + piece * 8;
+#pragma unroll
+            for (int r = 0; r < 8; ++r) {
+                const uint32_t row = r * 8 + lane / 8;
+                const uint4p v = *reinterpret_cast<const uint4p*>(stage + row * kK1Pitch + piece * 8);
+                *reinterpret_cast<uint4p*>(out + static_cast<int64_t>(co0 + row) * p.ys[1]) = v;
+            }
+        }
+        // the registers of the tile just transposed start loading the tile three ahead
+        fetch(Next{}, tile + 3 * q.workers);
+        // the staged rows are read before the next tile's are written: same wavefront, LDS operations stay in order
+        tile = next;
+        return more;
+    };
+    while (one_tile(Zero{}) && one_tile(One{})) {
+    }
+}
+
+template <class T, int KSTEPS, int S>
+int launch_k1(const ConvProblem& p, const K1Plan& q, uint32_t groups, const void* x, const void* w, const void* bias, void* y, hipStream_t stream) {
+    constexpr int C = KSTEPS * 16;
+    constexpr size_t lds = sizeof(T) * (2 * (C / 64) * kK1Panel + 4 * kK1CoWave * kK1Pitch);
+    auto kernel = conv2d_k1_kernel<T, KSTEPS, S>;
+    static std::atomic<uint64_t> configured{0};
+    if (int rc = raise_lds_limit(reinterpret_cast<const void*>(kernel), lds, configured)) return rc;
+    hipLaunchKernelGGL(kernel, dim3(groups * q.workers), dim3(kK1Threads), lds, stream, static_cast<const T*>(x), static_cast<const T*>(w),
+                       static_cast<const T*>(bias), static_cast<T*>(y), p, q);
+    return launch_status("conv2d_k1_kernel");
+}
+
+template <class T, int S>
+int pick_k1(const ConvProblem& p, const K1Plan& q, uint32_t groups, const void* x, const void* w, const void* bias, void* y, hipStream_t stream) {
+    switch (p.C) {
+        case 64: return launch_k1<T, 4, S>(p, q, groups, x, w, bias, y, stream);
+        case 128: return launch_k1<T, 8, S>(p, q, groups, x, w, bias, y, stream);
+        case 192: return launch_k1<T, 12, S>(p, q, groups, x, w, bias, y, stream);
+        case 256: return launch_k1<T, 16, S>(p, q, groups, x, w, bias, y, stream);
+        default: return TANNIC_UNSUPPORTED_DTYPE;
+    }
+}
+
+template <class T>
+int run_k1(const ConvProblem& p, const void* x, const void* w, const void* bias, void* y, hipStream_t stream) {
+    if (p.KH != 1 || p.KW != 1 || p.pad_h != 0 || p.pad_w != 0) return TANNIC_UNSUPPORTED_DTYPE;
+    if (p.stride_h != p.stride_w || (p.stride_w != 1 && p.stride_w != 2)) return TANNIC_UNSUPPORTED_DTYPE;
+    if (p.C == 0 || p.C % 64 != 0 || p.C > 256 || p.O == 0 || p.O % kK1CoBlock != 0) return TANNIC_UNSUPPORTED_DTYPE;
+    if (p.N == 0 || p.HO == 0 || p.WO == 0) return TANNIC_SUCCESS;
+    const uint64_t pixels = static_cast<uint64_t>(p.HO) * p.WO;
+    if (pixels % 8 != 0 || pixels >= (1ull << 31)) return TANNIC_UNSUPPORTED_DTYPE;
+    // weights: rows of C contiguous channels, 16-byte fragments
+    if (p.ws[1] != 1 || p.ws[0] % 8 != 0 || reinterpret_cast<uintptr_t>(w) % 16 != 0) return TANNIC_UNSUPPORTED_DTYPE;
+    // result: the pixels of a channel contiguous, rows written 16 bytes at a time
+    if (p.ys[3] != 1 || p.ys[2] != static_cast<int64_t>(p.WO) || p.ys[1] % 8 != 0 || p.ys[0] % 8 != 0 || reinterpret_cast<uintptr_t>(y) % 16 != 0)
+        return TANNIC_UNSUPPORTED_DTYPE;
+    // signal: 16-byte loads along W
+    if (p.xs[3] != 1 || p.xs[2] % 8 != 0 || p.xs[1] % 8 != 0 || p.xs[0] % 8 != 0 || reinterpret_cast<uintptr_t>(x) % 16 != 0) return TANNIC_UNSUPPORTED_DTYPE;
+    if (p.stride_w == 1) {
+        // eight consecutive pixels are one load: a run must not cross a row
+        if (p.WO % 8 != 0) return TANNIC_UNSUPPORTED_DTYPE;
+    } else {
+        // four pixels are the even elements of one load of eight: the eighth must exist
+        if (p.WO % 4 != 0 || static_cast<uint64_t>(p.WO) * 2 > p.W) return TANNIC_UNSUPPORTED_DTYPE;
+    }
+    K1Plan q{};
+    q.pixels = static_cast<uint32_t>(pixels);
+    const uint32_t tiles_per_image = (q.pixels + kK1Pixels - 1) / kK1Pixels;
+    const uint64_t tiles = static_cast<uint64_t>(p.N) * tiles_per_image;
+    if (tiles >= (1ull << 31)) return TANNIC_UNSUPPORTED_DTYPE;
+    q.tiles = static_cast<uint32_t>(tiles);
+    const uint32_t groups = p.O / kK1CoBlock;
+    // one block per compute unit (100 KB of LDS, every register): as many workers per group as that allows
+    const uint32_t per_group = groups >= 256 ? 1 : 256 / groups;
+    q.workers = q.tiles < per_group ? q.tiles : per_group;
+    q.div_wo = FastDiv(p.WO);
+    q.div_tiles_per_image = FastDiv(tiles_per_image);
+    if (p.stride_w == 1) return pick_k1<T, 1>(p, q, groups, x, w, bias, y, stream);
+    return pick_k1<T, 2>(p, q, groups, x, w, bias, y, stream);
+}
+
+int conv2d_k1(const ConvProblem& p, int dtype, const void* x, const void* w, const void* bias, void* y, hipStream_t stream) {
+    if (dtype == TANNIC_FLOAT16) return run_k1<f16>(p, x, w, bias, y, stream);
+    if (dtype == TANNIC_BFLOAT16) return run_k1<bf16>(p, x, w, bias, y, stream);
+    return TANNIC_UNSUPPORTED_DTYPE;
+}
+
+}  // namespace th

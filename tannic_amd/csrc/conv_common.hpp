@@ -18,6 +18,7 @@ struct ConvProblem {
 
 // Each returns TANNIC_UNSUPPORTED_DTYPE when the problem does not meet its
 // conditions, so that the caller can try the next, more general kernel.
+int conv2d_k1(const ConvProblem& p, int dtype, const void* x, const void* w, const void* bias, void* y, hipStream_t stream);
 int conv2d_pointwise(const ConvProblem& p, int dtype, const void* x, const void* w, const void* bias, void* y, hipStream_t stream);
 int conv2d_stem(const ConvProblem& p, int dtype, const void* x, const void* w, const void* bias, void* y, hipStream_t stream);
 int conv2d_k3(const ConvProblem& p, int dtype, const void* x, const void* w, const void* bias, void* y, hipStream_t stream);

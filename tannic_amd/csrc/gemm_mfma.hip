@@ -578,6 +578,10 @@ int run16(const GemmProblem& p, const void* a, const void* b, void* c, hipStream
             if (cost < best_cost) { best_cost = cost; best_bm = bm; best_splits = splits; }
         }
     }
+#ifdef TH_EXP
+    if (const char* e = getenv("TH_BM")) best_bm = atoi(e);
+    if (const char* e = getenv("TH_SPLITS")) best_splits = atoi(e);
+#endif
     if (best_splits > 1) {
         if (best_bm == 128) return run16_split<T, 128>(p, ak, bk, best_splits, a, b, c, stream);
         return run16_split<T, 64>(p, ak, bk, best_splits, a, b, c, stream);

@@ -45,6 +45,14 @@ CASES = {
     "stem_c4_k5x8_s3x2": ((1, 4, 17, 32), (8, 4, 5, 8), (3, 2), (0, 4)),
     "stem_c2_k7_s2_tall": ((1, 2, 64, 16), (5, 2, 7, 7), (2, 2), (3, 3)),
     "k3_rect_stride_pad": ((1, 96, 13, 24), (64, 96, 3, 3), (2, 1), (0, 2)),
+    # 1x1 kernels with the weights resident in registers: 64..256 channels in, multiples of 256 out, stride 1 and 2,
+    # pixel counts that end inside a 64-pixel tile, several images per worker
+    "k1_s2_256ch": ((2, 256, 24, 24), (256, 256, 1, 1), (2, 2), (0, 0)),
+    "k1_s2_64ch_two_groups": ((1, 64, 16, 16), (512, 64, 1, 1), (2, 2), (0, 0)),
+    "k1_s1_128ch_short_tile": ((3, 128, 5, 8), (256, 128, 1, 1), (1, 1), (0, 0)),
+    "k1_s1_192ch": ((1, 192, 10, 16), (256, 192, 1, 1), (1, 1), (0, 0)),
+    "k1_s2_odd_rows": ((1, 64, 15, 24), (256, 64, 1, 1), (2, 2), (0, 0)),
+    "k1_s2_many_images": ((40, 64, 8, 8), (256, 64, 1, 1), (2, 2), (0, 0)),
 }
 
 
