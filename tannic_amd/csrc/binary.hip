@@ -97,8 +97,8 @@ int run_binary(const tannic_tensor_t* a, const tannic_tensor_t* b, tannic_tensor
         // one element: *dst = op(*a, *b) (src/cpu/ops-binary.cpp:67-73)
         if (!build_plan(plan, 1, &one, strides, 3)) return TANNIC_ERROR;
     } else {
-        if (a->rank > rank || b->rank > rank) {
-            set_error_text("binary op: operand rank exceeds destination rank");
+        if (!broadcasts_to(a, dst) || !broadcasts_to(b, dst)) {
+            set_error_text("binary op: an operand's shape does not broadcast to the destination's");
             return TANNIC_ERROR;
         }
         aligned_strides(a, rank, strides[0]);

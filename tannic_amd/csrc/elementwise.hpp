@@ -273,6 +273,29 @@ inline void aligned_strides(const tannic_tensor_t* t, int rank, int64_t* out) {
     }
 }
 
+// Whether `t`, right-aligned on `dst`, matches it in every dim or has extent 1 there: the kernels index `t` by
+// dst's coordinates, so anything else would read outside `t`.
+inline bool broadcasts_to(const tannic_tensor_t* t, const tannic_tensor_t* dst) {
+    if (t->rank > dst->rank) return false;
+    const int off = dst->rank - t->rank;
+    for (int d = 0; d < t->rank; ++d)
+        if (t->shape.sizes[d] != 1 && t->shape.sizes[d] != dst->shape.sizes[d + off]) return false;
+    return true;
+}
+
+// Same rank and extents: what the kernels that walk one tensor by another's coordinates rely on.
+inline bool same_extents(const tannic_tensor_t* a, const tannic_tensor_t* b) {
+    if (a->rank != b->rank) return false;
+    for (int d = 0; d < a->rank; ++d)
+        if (a->shape.sizes[d] != b->shape.sizes[d]) return false;
+    return true;
+}
+
+inline int shape_mismatch(const char* what) {
+    set_error_text(what);
+    return TANNIC_ERROR;
+}
+
 inline void contiguous_strides(int rank, const size_t* extent, int64_t* out) {
     int64_t run = 1;
     for (int d = rank - 1; d >= 0; --d) {

@@ -121,8 +121,8 @@ int run_pair(const tannic_tensor_t* a, const tannic_tensor_t* b, tannic_tensor_t
     if (rank == 0) {
         if (!build_plan(plan, 1, &one, strides, 3)) return TANNIC_ERROR;
     } else {
-        if (a->rank > rank || b->rank > rank) {
-            set_error_text("binary op: operand rank exceeds destination rank");
+        if (!broadcasts_to(a, dst) || !broadcasts_to(b, dst)) {
+            set_error_text("binary op: an operand's shape does not broadcast to the destination's");
             return TANNIC_ERROR;
         }
         aligned_strides(a, rank, strides[0]);
@@ -139,6 +139,7 @@ int run_pair(const tannic_tensor_t* a, const tannic_tensor_t* b, tannic_tensor_t
 
 template <class A, class B>
 int run_cast(const tannic_tensor_t* src, tannic_tensor_t* dst, hipStream_t stream) {
+    if (!same_extents(src, dst)) return shape_mismatch("cast: source and destination shapes differ");
     int64_t strides[kMaxOperands][TANNIC_DIMENSIONS] = {};
     const int rank = dst->rank;
     contiguous_strides(rank, dst->shape.sizes, strides[2]);

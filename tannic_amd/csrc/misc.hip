@@ -25,6 +25,7 @@ struct ScaleF {
 
 template <class T>
 int run_scale(const tannic_tensor_t* src, const tannic_scalar_t* sc, tannic_tensor_t* dst, hipStream_t stream) {
+    if (!same_extents(src, dst)) return shape_mismatch("scale: source and destination shapes differ");
     int64_t strides[kMaxOperands][TANNIC_DIMENSIONS] = {};
     const int rank = dst->rank;
     contiguous_strides(rank, dst->shape.sizes, strides[2]);
@@ -230,6 +231,7 @@ __global__ __launch_bounds__(kBlock) void compare_flat_kernel(const T* a, const 
 
 template <class T, int K>
 int run_compare(const tannic_tensor_t* a, const tannic_tensor_t* b, tannic_tensor_t* dst, hipStream_t stream) {
+    if (!same_extents(a, dst) || !same_extents(b, dst)) return shape_mismatch("compare: operand and destination shapes differ");
     int64_t strides[kMaxOperands][TANNIC_DIMENSIONS] = {};
     const int rank = dst->rank;
     // each source is walked with its own strides over the destination's shape
@@ -302,6 +304,10 @@ __global__ __launch_bounds__(kBlock) void allclose_kernel(const T* a, const T* b
 
 template <class T>
 int run_allclose(const tannic_tensor_t* a, const tannic_tensor_t* b, hipStream_t stream, double rtol, double atol) {
+    if (!same_extents(a, b)) {
+        set_error_text("allclose: operand shapes differ");
+        return -1;
+    }
     int64_t strides[kMaxOperands][TANNIC_DIMENSIONS] = {};
     const int rank = a->rank;
     for (int d = 0; d < rank; ++d) {

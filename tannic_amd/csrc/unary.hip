@@ -76,6 +76,7 @@ struct UnaryF {
 
 template <class T, int K>
 int run_unary(const tannic_tensor_t* src, tannic_tensor_t* dst, hipStream_t stream, double eps) {
+    if (!same_extents(src, dst)) return shape_mismatch("unary op: source and destination shapes differ");
     int64_t strides[kMaxOperands][TANNIC_DIMENSIONS] = {};
     const int rank = dst->rank;
     contiguous_strides(rank, dst->shape.sizes, strides[2]);
