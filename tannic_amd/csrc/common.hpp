@@ -147,6 +147,13 @@ inline size_t dtype_size(int dtype) {
     }
 }
 
+// Elements a descriptor's shape spans (1 for rank 0).
+inline size_t element_count(const tannic_tensor_t* t) {
+    size_t n = 1;
+    for (int d = 0; d < t->rank; ++d) n *= t->shape.sizes[d];
+    return n;
+}
+
 // ---- 32-bit division by a launch-time constant ------------------------------
 // q = n / d for n < 2^31 with one multiply-high, one add and one shift.
 struct FastDiv {

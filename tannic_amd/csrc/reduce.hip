@@ -331,6 +331,7 @@ int run_reduce(const tannic_tensor_t* src, tannic_tensor_t* dst, hipStream_t str
         }
         if (slots == 0) return TANNIC_SUCCESS;
         if (slots >= (1ull << 31)) { set_error_text("reduce: too many outputs"); return TANNIC_ERROR; }
+        if (element_count(dst) != slots) { set_error_text("reduce: the destination does not hold one element per reduced slice"); return TANNIC_ERROR; }
         hipLaunchKernelGGL((reduce_strided_kernel<Op>), dim3((slots + kThreads - 1) / kThreads), dim3(kThreads), 0, stream, ps, pd, w,
                            static_cast<uint32_t>(slots));
         return launch_status("reduce_strided_kernel");
@@ -343,6 +344,7 @@ int run_reduce(const tannic_tensor_t* src, tannic_tensor_t* dst, hipStream_t str
     const size_t slots = outer * inner;
     if (slots == 0) return TANNIC_SUCCESS;
     if (slots >= (1ull << 31) || outer >= (1ull << 31)) { set_error_text("reduce: too many outputs"); return TANNIC_ERROR; }
+    if (element_count(dst) != slots) { set_error_text("reduce: the destination does not hold one element per reduced slice"); return TANNIC_ERROR; }
     constexpr int VEC = sizeof(T) >= 16 ? 1 : static_cast<int>(16 / sizeof(T));
     const bool aligned = reinterpret_cast<uintptr_t>(ps) % 16 == 0;
 

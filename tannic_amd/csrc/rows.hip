@@ -256,12 +256,6 @@ inline bool is_contiguous(const tannic_tensor_t* t) {
     return true;
 }
 
-inline size_t element_count(const tannic_tensor_t* t) {
-    size_t n = 1;
-    for (int d = 0; d < t->rank; ++d) n *= t->shape.sizes[d];
-    return n;
-}
-
 inline bool same_shape(const tannic_tensor_t* a, const tannic_tensor_t* b) {
     if (a->rank != b->rank) return false;
     for (int d = 0; d < a->rank; ++d)

@@ -63,3 +63,15 @@ def test_well_formed_calls_still_succeed(device):
     status, _ = call("add", device, [a, b], zeros((4, 6), ta.float32, device))
     assert status == abi.SUCCESS
     assert ops.add(a, b).shape == (4, 6)
+
+
+@pytest.mark.parametrize("name", ["argsum", "argmax", "max"])
+def test_reduction_destination_must_hold_one_element_per_slice(device, name):
+    src = zeros((4, 6, 8), ta.float32, device)
+    dtype = ta.int64 if name == "argmax" else ta.float32
+    status, message = call(name, device, [src], zeros((4, 6), dtype, device), (C.c_uint8(1),))
+    assert status == abi.ERROR and "destination" in message
+    status, _ = call(name, device, [src], zeros((4, 8), dtype, device), (C.c_uint8(1),))
+    assert status == abi.SUCCESS
+    status, _ = call(name, device, [src], zeros((4, 1, 8), dtype, device), (C.c_uint8(1),))   # kept dimension
+    assert status == abi.SUCCESS
