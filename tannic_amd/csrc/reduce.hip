@@ -206,6 +206,86 @@ __global__ __launch_bounds__(kThreads) void reduce_rows_kernel(const typename Op
     }
 }
 
+// ---- rows, argmax / argmin of 16-bit floats ------------------------------------------------------
+// The generic row kernel carries (value, index) pairs through every step, which makes these the one
+// reduction bound by the vector ALU rather than by HBM.  Here a wavefront holds its row in registers (up
+// to four 16-byte pieces per lane), finds the extreme VALUE first (one max/min per element, NaN ignored,
+// the -inf / +inf start kept when nothing beats it), then the lowest index holding it.  Same answers as
+// the strict comparison from the start value: ties go to the lowest index, NaN never wins, and a row in
+// which nothing beats the start gives 0 (src/cpu/argred.cpp:95-101, :317-347).
+struct MinIndexOp {
+    __device__ static inline uint32_t combine(uint32_t x, uint32_t y) { return x < y ? x : y; }
+};
+template <bool MAX> struct ExtremeOp {
+    __device__ static inline float combine(float x, float y) { return MAX ? fmaxf(x, y) : fminf(x, y); }
+};
+
+// A wavefront takes kArgRows rows at once: all their loads are issued before any arithmetic, which keeps enough
+// bytes in flight per compute unit for the longer life of these wavefronts.
+constexpr int kArgRows = 2;
+
+template <class T, bool MAX, int NCH>
+__global__ __launch_bounds__(kThreads) void arg_rows16_kernel(const T* src, int64_t* dst, uint32_t rows, uint32_t R) {
+    const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+    const uint32_t row0 = (blockIdx.x * (kThreads / kWave) + wave) * kArgRows;
+    if (row0 >= rows) return;   // whole wavefronts; nothing below synchronises across them
+    const uint32_t chunks = R / 8;
+    const float start = MAX ? -__builtin_inff() : __builtin_inff();
+    Vec<T, 8> raw[kArgRows][NCH];
+#pragma unroll
+    for (int r = 0; r < kArgRows; ++r) {
+        const uint32_t row = row0 + r < rows ? row0 + r : rows - 1;   // the odd last row is done twice
+        const T* p = src + static_cast<size_t>(row) * R;
+#pragma unroll
+        for (int i = 0; i < NCH; ++i) {
+            const uint32_t c = lane + i * kWave;
+            raw[r][i] = load_vec<T, 8>(p + static_cast<size_t>(c < chunks ? c : 0) * 8);
+        }
+    }
+#pragma unroll
+    for (int r = 0; r < kArgRows; ++r) {
+        float f[NCH][8];
+        float best = start;
+#pragma unroll
+        for (int i = 0; i < NCH; ++i) {
+            const bool present = lane + i * kWave < chunks;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                f[i][e] = present ? widen(raw[r][i].v[e]) : __builtin_nanf("");   // an absent piece equals nothing
+                best = ExtremeOp<MAX>::combine(best, f[i][e]);
+            }
+        }
+        best = wave_reduce<ExtremeOp<MAX>>(best);
+        // the lane's first position holding the extreme, walking backwards so that the lowest one stays
+        uint32_t pos = 0xFFu;
+#pragma unroll
+        for (int i = NCH - 1; i >= 0; --i)
+#pragma unroll
+            for (int e = 7; e >= 0; --e) pos = f[i][e] == best ? static_cast<uint32_t>(i * 8 + e) : pos;
+        uint32_t index = pos == 0xFFu ? 0xFFFFFFFFu : ((pos / 8) * kWave + lane) * 8 + pos % 8;
+        index = wave_reduce<MinIndexOp>(index);
+        // nothing beat the start (all NaN, or only the start value itself): the strict comparison never moved off 0
+        if (lane == 0 && row0 + r < rows) dst[row0 + r] = (best == start || index == 0xFFFFFFFFu) ? 0 : static_cast<int64_t>(index);
+    }
+}
+
+template <class T, bool MAX>
+int launch_arg_rows16(const T* src, int64_t* dst, uint32_t rows, uint32_t R, hipStream_t stream) {
+    const uint32_t per_lane = (R / 8 + kWave - 1) / kWave;
+    const uint32_t per_block = (kThreads / kWave) * kArgRows;
+    const dim3 grid((rows + per_block - 1) / per_block);
+    if (per_lane <= 1) hipLaunchKernelGGL((arg_rows16_kernel<T, MAX, 1>), grid, dim3(kThreads), 0, stream, src, dst, rows, R);
+    else if (per_lane <= 2) hipLaunchKernelGGL((arg_rows16_kernel<T, MAX, 2>), grid, dim3(kThreads), 0, stream, src, dst, rows, R);
+    else hipLaunchKernelGGL((arg_rows16_kernel<T, MAX, 4>), grid, dim3(kThreads), 0, stream, src, dst, rows, R);
+    return launch_status("arg_rows16_kernel");
+}
+
+template <class Op> struct ArgRows16 { static constexpr bool value = false; };
+template <class T, bool MAX> struct ArgRows16<ArgOp<T, MAX, false>> {
+    static constexpr bool value = is_16bit<T>::value;
+    static int run(const T* src, int64_t* dst, uint32_t rows, uint32_t R, hipStream_t stream) { return launch_arg_rows16<T, MAX>(src, dst, rows, R, stream); }
+};
+
 // ---- columns: inner > 1 ----------------------------------------------------------
 // Thread (tx, ty): VEC columns starting at (blockIdx.x*TX + tx)*VEC, rows
 // ty + k*TY*gridDim.z offset by blockIdx.z*TY.  LOG_TX picks the block shape.
@@ -351,6 +431,10 @@ int run_reduce(const tannic_tensor_t* src, tannic_tensor_t* dst, hipStream_t str
     if (inner == 1) {
         const uint32_t rows = static_cast<uint32_t>(outer);
         const bool vec = VEC > 1 && aligned && R % VEC == 0;
+        if constexpr (ArgRows16<Op>::value) {
+            // rows that fit the registers of one wavefront (four 16-byte pieces per lane)
+            if (vec && R <= 8 * kWave * 4 && rows >= 1024) return ArgRows16<Op>::run(ps, pd, rows, static_cast<uint32_t>(R), stream);
+        }
         // few long rows: a whole block per row
         const bool wide = rows < 2048 && R >= 8192;
         const uint32_t grid = wide ? rows : (rows + 3) / 4;
@@ -377,14 +461,20 @@ int run_reduce(const tannic_tensor_t* src, tannic_tensor_t* dst, hipStream_t str
 
     const bool vec = VEC > 1 && aligned && inner % VEC == 0;
     const uint32_t column_groups = static_cast<uint32_t>(vec ? inner / VEC : inner);
-    // block shape: TX lanes across columns, the rest of the 256 threads across R
-    const int TX = column_groups >= 64 ? 64 : column_groups >= 16 ? 16 : 4;
+    // block shape: TX lanes across columns, the rest of the 256 threads across R.  About two blocks per compute unit
+    // (512) stream best on this chip: fewer leave units idle, more only add partial results and a longer second pass.
+    int TX = column_groups >= 64 ? 64 : column_groups >= 16 ? 16 : 4;
+    if (TX == 64) {
+        // narrow blocks reach that count without sharing R between blocks: no partial results, no second kernel
+        const size_t narrow = static_cast<size_t>((column_groups + 15) / 16) * outer;
+        const size_t wide_blocks = static_cast<size_t>((column_groups + 63) / 64) * outer;
+        if (wide_blocks < 512 && narrow >= 512 && narrow < 1024 && R >= 512) TX = 16;
+    }
     const int TY = kThreads / TX;
     const uint32_t gx = (column_groups + TX - 1) / TX;
-    // split R over blocks until the chip has ~8 blocks per CU or slices get short
     uint32_t splits = 1;
     const size_t base_blocks = static_cast<size_t>(gx) * outer;
-    while (base_blocks * splits < 2048 && R / (static_cast<size_t>(TY) * splits * 2) >= 16 && splits < 64) splits *= 2;
+    while (base_blocks * splits < 512 && R / (static_cast<size_t>(TY) * splits * 2) >= 16 && splits < 64) splits *= 2;
     A* partial = nullptr;
     if (splits > 1) {
         if (scratch_acquire(reinterpret_cast<void**>(&partial), sizeof(A) * splits * slots, stream) != TANNIC_SUCCESS) return TANNIC_ERROR;
