@@ -135,7 +135,6 @@ __device__ inline Pack<T, N> load_or_splat(const T* p, bool splat) {
 }
 
 constexpr int kBlock = 256;
-constexpr int kUnroll = 1;
 
 // Element offsets of vector `v` in the three operands.
 struct Offsets {
@@ -165,8 +164,11 @@ __device__ inline Offsets decode(const Plan& p, uint32_t v) {
 
 // F: { using S0, S1, D; static constexpr int sources; const S0* a; const S1* b; D* out;
 //      __device__ D operator()(S0, S1) const; }   (S1/b unused when sources == 1)
-template <class F, int VEC>
+// UNROLL vectors per thread, kBlock apart.  One is best for plain contiguous operands; with a broadcast operand a
+// thread lives longer (row decoding, the dependent load of the repeated value) and two keep enough bytes in flight.
+template <class F, int VEC, int UNROLL>
 __global__ __launch_bounds__(kBlock) void elementwise_kernel(F f, Plan p) {
+    constexpr int kUnroll = UNROLL;
     using S0 = typename F::S0;
     using S1 = typename F::S1;
     using D = typename F::D;
@@ -251,14 +253,18 @@ int launch_elementwise(F f, Plan p, hipStream_t stream) {
     p.row_div = FastDiv(p.row_vectors);
     p.total_vectors = rows * p.row_vectors;
     if (p.total_vectors == 0) return TANNIC_SUCCESS;
-    const uint32_t grid = (p.total_vectors + kBlock * kUnroll - 1) / (kBlock * kUnroll);
+    const bool repeats = p.rank > 1 || p.stride[0][last] == 0 || (F::sources == 2 && p.stride[1][last] == 0);
+    const uint32_t per_block = kBlock * (repeats ? 2 : 1);
+    const uint32_t grid = (p.total_vectors + per_block - 1) / per_block;
     if constexpr (VEC > 1) {
         if (vec) {
-            hipLaunchKernelGGL((elementwise_kernel<F, VEC>), dim3(grid), dim3(kBlock), 0, stream, f, p);
+            if (repeats) hipLaunchKernelGGL((elementwise_kernel<F, VEC, 2>), dim3(grid), dim3(kBlock), 0, stream, f, p);
+            else hipLaunchKernelGGL((elementwise_kernel<F, VEC, 1>), dim3(grid), dim3(kBlock), 0, stream, f, p);
             return launch_status("elementwise_kernel");
         }
     }
-    hipLaunchKernelGGL((elementwise_kernel<F, 1>), dim3(grid), dim3(kBlock), 0, stream, f, p);
+    if (repeats) hipLaunchKernelGGL((elementwise_kernel<F, 1, 2>), dim3(grid), dim3(kBlock), 0, stream, f, p);
+    else hipLaunchKernelGGL((elementwise_kernel<F, 1, 1>), dim3(grid), dim3(kBlock), 0, stream, f, p);
     return launch_status("elementwise_kernel");
 }
 
