@@ -47,6 +47,7 @@ constexpr int kStemBCO = 64;       // output channels per block
 constexpr int kStemOutPitch = kStemPixels + 8;
 constexpr int kStemLeft = 8;       // zero columns in front of a row in LDS (keeps the 16-byte row chunks aligned)
 constexpr int kStemUnits = 4;      // 16-byte chunks of input rows a thread can hold at a time
+constexpr int kStemWeightPieces = 6;   // 16-byte pieces of a block's weights per thread: 64 channels x (22 slots x 8 columns) at most
 
 struct StemPlan {
     uint32_t slots;             // C * KH
@@ -76,21 +77,72 @@ __global__ __launch_bounds__(kStemThreads, 2) void conv2d_stem_kernel(const T* x
     const uint32_t oh_end = oh_first + q.strip < p.HO ? oh_first + q.strip : p.HO;
     const T* ximg = x + static_cast<int64_t>(n) * p.xs[0];
 
+    // ---- input rows: global -> registers -> ring --------------------------------------------------------------
+    // a unit is one 16-byte chunk of one row of one channel; rows outside the image are stored as zeros
+    const uint32_t chunks = p.W / 8;
+    uint4s rows_reg[kStemUnits];
+    auto load_rows = [&](int32_t ih_from, uint32_t count) {   // rows ih_from .. ih_from + count - 1 of every channel
+        const uint32_t units = p.C * count * chunks;
+#pragma unroll
+        for (int u = 0; u < kStemUnits; ++u) {
+            if (kStemThreads * u >= units) continue;   // the same for the whole block
+            const uint32_t idx = threadIdx.x + kStemThreads * u;
+            uint32_t t1, chunk, r, c;
+            q.div_chunks.divmod(idx, t1, chunk);
+            q.div_c.divmod(t1, r, c);
+            const int32_t ih = ih_from + static_cast<int32_t>(r);
+            const bool live = idx < units && ih >= 0 && ih < static_cast<int32_t>(p.H);
+            rows_reg[u] = uint4s{0, 0, 0, 0};
+            if (live) rows_reg[u] = *reinterpret_cast<const uint4s*>(ximg + static_cast<int64_t>(c) * p.xs[1] + static_cast<int64_t>(ih) * p.xs[2] + chunk * 8);
+        }
+    };
+    auto store_rows = [&](int32_t ih_from, uint32_t count) {
+        const uint32_t units = p.C * count * chunks;
+#pragma unroll
+        for (int u = 0; u < kStemUnits; ++u) {
+            const uint32_t idx = threadIdx.x + kStemThreads * u;
+            if (idx >= units) continue;
+            uint32_t t1, chunk, r, c;
+            q.div_chunks.divmod(idx, t1, chunk);
+            q.div_c.divmod(t1, r, c);
+            const uint32_t slot = static_cast<uint32_t>(ih_from + static_cast<int32_t>(r) + (1 << 20) * static_cast<int32_t>(q.ring)) & (q.ring - 1);
+            *reinterpret_cast<uint4s*>(ring + (c * q.ring + slot) * q.pitch + kStemLeft + chunk * 8) = rows_reg[u];
+        }
+    };
+    // Every global load of the start is issued before the first wait: the block's weights (at most six 16-byte pieces
+    // per thread), the input rows of the first output row (as many as the registers hold) and the bias.
+    const int32_t top = static_cast<int32_t>(oh_first * p.stride_h) - static_cast<int32_t>(p.pad_h);
+    const uint32_t per_step = (kStemUnits * kStemThreads) / (p.C * chunks);   // >= 1 by the plan
+    const uint32_t first_count = p.KH < per_step ? p.KH : per_step;
+
     // ---- weights: this lane's fragments for every slice, kept in registers --------------------------------
     // The block's rows of the OIHW tensor (one contiguous run) are copied to LDS 16 bytes at a time first.
     // fragment (s, i): channel co0 + i * 32 + lane % 32, slot 2 s + lane / 32; element e of a slot is kernel column e - delta
     const uint32_t taps = q.slots * p.KW;   // elements per output channel
     const uint32_t wrows = p.O - co0 < kStemBCO ? p.O - co0 : kStemBCO;
+    float bias_v[2];
     {
         T* raw = ring;
         const uint32_t count = wrows * taps;   // the run starts at a multiple of 8 elements (64 * taps is one)
         const T* src = w + static_cast<int64_t>(co0) * taps;
-        for (uint32_t i = threadIdx.x * 8; i < count; i += kStemThreads * 8) {
-            if (i + 8 <= count) {
-                *reinterpret_cast<uint4s*>(raw + i) = *reinterpret_cast<const uint4s*>(src + i);
-            } else {
+        uint4s wreg[kStemWeightPieces];
+#pragma unroll
+        for (int j = 0; j < kStemWeightPieces; ++j) {
+            const uint32_t i = (threadIdx.x + kStemThreads * j) * 8;
+            if (i + 8 <= count) wreg[j] = *reinterpret_cast<const uint4s*>(src + i);
+        }
+        load_rows(top, first_count);
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            const uint32_t co = co0 + i * 32 + lane % 32;
+            bias_v[i] = (p.has_bias && co < p.O) ? static_cast<float>(widen(bias[co])) : 0.0f;
+        }
+#pragma unroll
+        for (int j = 0; j < kStemWeightPieces; ++j) {
+            const uint32_t i = (threadIdx.x + kStemThreads * j) * 8;
+            if (i + 8 <= count) *reinterpret_cast<uint4s*>(raw + i) = wreg[j];
+            else if (i < count)
                 for (uint32_t e = i; e < count; ++e) raw[e] = src[e];
-            }
         }
         __syncthreads();
     }
@@ -135,58 +187,17 @@ __global__ __launch_bounds__(kStemThreads, 2) void conv2d_stem_kernel(const T* x
     for (int s = 0; s < NS; ++s)
 #pragma unroll
         for (int i = 0; i < 2; ++i) afrag[s][i] = *reinterpret_cast<const uint4s*>(records + ((2 * s + lane / 32) * kStemBCO + i * 32 + lane % 32) * 8);
-    float bias_v[2];
-#pragma unroll
-    for (int i = 0; i < 2; ++i) {
-        const uint32_t co = co0 + i * 32 + lane % 32;
-        bias_v[i] = (p.has_bias && co < p.O) ? static_cast<float>(widen(bias[co])) : 0.0f;
-    }
     __syncthreads();   // the copy is consumed: its memory becomes the ring
     // zero everything once: the columns beside the rows are never written again
     for (uint32_t i = threadIdx.x; i < q.ring_elems / 8; i += kStemThreads) reinterpret_cast<uint4s*>(ring)[i] = uint4s{0, 0, 0, 0};
     __syncthreads();
 
-    // ---- input rows: global -> registers -> ring --------------------------------------------------------------
-    // a unit is one 16-byte chunk of one row of one channel; rows outside the image are stored as zeros
-    const uint32_t chunks = p.W / 8;
-    uint4s rows_reg[kStemUnits];
-    auto load_rows = [&](int32_t ih_from, uint32_t count) {   // rows ih_from .. ih_from + count - 1 of every channel
-        const uint32_t units = p.C * count * chunks;
-#pragma unroll
-        for (int u = 0; u < kStemUnits; ++u) {
-            if (kStemThreads * u >= units) continue;   // the same for the whole block
-            const uint32_t idx = threadIdx.x + kStemThreads * u;
-            uint32_t t1, chunk, r, c;
-            q.div_chunks.divmod(idx, t1, chunk);
-            q.div_c.divmod(t1, r, c);
-            const int32_t ih = ih_from + static_cast<int32_t>(r);
-            const bool live = idx < units && ih >= 0 && ih < static_cast<int32_t>(p.H);
-            rows_reg[u] = uint4s{0, 0, 0, 0};
-            if (live) rows_reg[u] = *reinterpret_cast<const uint4s*>(ximg + static_cast<int64_t>(c) * p.xs[1] + static_cast<int64_t>(ih) * p.xs[2] + chunk * 8);
-        }
-    };
-    auto store_rows = [&](int32_t ih_from, uint32_t count) {
-        const uint32_t units = p.C * count * chunks;
-#pragma unroll
-        for (int u = 0; u < kStemUnits; ++u) {
-            const uint32_t idx = threadIdx.x + kStemThreads * u;
-            if (idx >= units) continue;
-            uint32_t t1, chunk, r, c;
-            q.div_chunks.divmod(idx, t1, chunk);
-            q.div_c.divmod(t1, r, c);
-            const uint32_t slot = static_cast<uint32_t>(ih_from + static_cast<int32_t>(r) + (1 << 20) * static_cast<int32_t>(q.ring)) & (q.ring - 1);
-            *reinterpret_cast<uint4s*>(ring + (c * q.ring + slot) * q.pitch + kStemLeft + chunk * 8) = rows_reg[u];
-        }
-    };
     // the rows of the first tile, in as many steps as the registers need
-    {
-        const int32_t top = static_cast<int32_t>(oh_first * p.stride_h) - static_cast<int32_t>(p.pad_h);
-        const uint32_t per_step = (kStemUnits * kStemThreads) / (p.C * chunks);   // >= 1 by the plan
-        for (uint32_t done = 0; done < p.KH; done += per_step) {
-            const uint32_t count = p.KH - done < per_step ? p.KH - done : per_step;
-            load_rows(top + static_cast<int32_t>(done), count);
-            store_rows(top + static_cast<int32_t>(done), count);
-        }
+    store_rows(top, first_count);   // loaded at the very start
+    for (uint32_t done = first_count; done < p.KH; done += per_step) {
+        const uint32_t count = p.KH - done < per_step ? p.KH - done : per_step;
+        load_rows(top + static_cast<int32_t>(done), count);
+        store_rows(top + static_cast<int32_t>(done), count);
     }
 
     // ---- per-lane constants of the operand reads ------------------------------------------------------------------
