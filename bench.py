@@ -181,11 +181,12 @@ def decoder_layer_entry(b, iters, composed=True, one_pass=True):
                         "bound": "mixed: matrix products plus about 45 launch-bound elementwise, reduction and copy kernels", "device_busy_us": busy,
                         "device_busy_tflops": round(flops / busy / 1e6, 2) if busy else None})
     if one_pass:
-        us = timed(lambda: dl.forward_fused(s, w, x, cos, sin, mask))
+        packed = dl.pack_weights(w)
+        us = timed(lambda: dl.forward_fused(s, packed, x, cos, sin, mask))
         busy = measured_value("decoder_layer_one_pass_bf16_seq512_kernels.txt", "device_busy_us_per_layer")
         entries.append({"op": "the same layer with the one-pass rms_norm / rope / softmax / swiglu operators (no counterpart in the reference)",
                         "us": round(us, 1), "tflops": round(flops / us / 1e6, 2), "mfma_frac": round(flops / us / 1e6 / MFMA_PEAK_TFLOPS["bf16"], 4),
-                        "bound": "matrix products plus 12 row-wise, elementwise and copy kernels", "device_busy_us": busy,
+                        "bound": "seven matrix products (q/k/v and gate/up as one each) plus 12 row-wise, elementwise and copy kernels", "device_busy_us": busy,
                         "device_busy_tflops": round(flops / busy / 1e6, 2) if busy else None})
     return entries
 

@@ -76,14 +76,36 @@ def silu(g, one):
     return ops.mul(ops.mul(g, sg), sg)
 
 
+def pack_weights(w):
+    """Adds the row-wise concatenations ``wqkv = [wq; wk; wv]`` and ``w13 = [w1; w3]`` to the parameter dictionary, so
+    that the projections sharing an input are one product each (done once, when the parameters are loaded)."""
+    packed = dict(w)
+    packed["wqkv"] = ops.concatenate(ops.concatenate(w["wq"], w["wk"], 0), w["wv"], 0)
+    packed["w13"] = ops.concatenate(w["w1"], w["w3"], 0)
+    return packed
+
+
+def split_heads(t, heads):
+    """``[1, seq, heads * d]`` with unit stride along the last axis (a column slice included) seen as ``[1, heads, seq, d]``."""
+    b, seq, width = t.shape
+    d = width // heads
+    return t._view((b, seq, heads, d), (t.strides[0], t.strides[1], d, 1)).transpose(1, 2)
+
+
 def forward_fused(s, w, x, cos, sin, mask):
     """The same layer with the device library's one-pass operators (``ops.rms_norm``, ``ops.rope``, ``ops.softmax``,
-    ``ops.swiglu``) in place of the chains; these have no counterpart in the reference's front end."""
+    ``ops.swiglu``) in place of the chains; these have no counterpart in the reference's front end.  With the
+    concatenated parameters of ``pack_weights`` the q/k/v and the gate/up projections are one product each and their
+    parts are column slices of its result."""
     _, seq, _ = x.shape
+    nq, nkv = s.heads * s.head_dim, s.kv_heads * s.head_dim
     xn = ops.rms_norm(x, w["g1"], s.eps)
-    q = ops.matmul(xn, w["wq"].transpose()).view(1, seq, s.heads, s.head_dim).transpose(1, 2)
-    k = ops.matmul(xn, w["wk"].transpose()).view(1, seq, s.kv_heads, s.head_dim).transpose(1, 2)
-    v = ops.matmul(xn, w["wv"].transpose()).view(1, seq, s.kv_heads, s.head_dim).transpose(1, 2)
+    if "wqkv" in w:
+        qkv = ops.matmul(xn, w["wqkv"].transpose())
+        q, k, v = qkv[..., 0:nq], qkv[..., nq:nq + nkv], qkv[..., nq + nkv:nq + 2 * nkv]
+    else:
+        q, k, v = (ops.matmul(xn, w[name].transpose()) for name in ("wq", "wk", "wv"))
+    q, k, v = split_heads(q, s.heads), split_heads(k, s.kv_heads), split_heads(v, s.kv_heads)
     q, k = ops.rope(q, cos, sin), ops.rope(k, cos, sin)
     group = s.heads // s.kv_heads
     k, v = ops.repeat(k, group, 1), ops.repeat(v, group, 1)
@@ -91,7 +113,11 @@ def forward_fused(s, w, x, cos, sin, mask):
     o = ops.repack(ops.matmul(p, v).transpose(1, 2)).view(1, seq, s.heads * s.head_dim)
     h = ops.add(x, ops.matmul(o, w["wo"].transpose()))
     hn = ops.rms_norm(h, w["g2"], s.eps)
-    act = ops.swiglu(ops.matmul(hn, w["w1"].transpose()), ops.matmul(hn, w["w3"].transpose()))
+    if "w13" in w:
+        both = ops.matmul(hn, w["w13"].transpose())
+        act = ops.swiglu(both[..., 0:s.ffn], both[..., s.ffn:2 * s.ffn])
+    else:
+        act = ops.swiglu(ops.matmul(hn, w["w1"].transpose()), ops.matmul(hn, w["w3"].transpose()))
     return ops.add(h, ops.matmul(act, w["w2"].transpose()))
 
 

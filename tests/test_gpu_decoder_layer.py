@@ -67,3 +67,8 @@ def test_one_pass_operators_give_the_same_layer(device, oracle, dtype, bar):
     got = dl.forward_fused(s, w, x, cos, sin, mask).numpy().astype(np.float64)
     assert got.shape == want.shape and np.isfinite(got).all()
     assert np.abs(got - want).max() <= bar * want.std(), (np.abs(got - want).max(), want.std())
+    # with q/k/v and gate/up as one product each: the same arithmetic per output element, so the same bits
+    packed = dl.forward_fused(s, dl.pack_weights(w), x, cos, sin, mask).numpy().astype(np.float64)
+    assert np.abs(packed - want).max() <= bar * want.std()
+    if dtype is ta.float32:
+        np.testing.assert_allclose(packed, got, rtol=1e-5, atol=1e-6)
