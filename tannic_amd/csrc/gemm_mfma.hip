@@ -549,28 +549,22 @@ int run16(const GemmProblem& p, const void* a, const void* b, void* c, hipStream
     if (p.batches > 65535) return TANNIC_UNSUPPORTED_DTYPE;
     // Tile height by M (a tile taller than M multiplies padding), large tiles only when they still give every CU work.
     const uint64_t big = static_cast<uint64_t>((p.M + 255) / 256) * ((p.N + 255) / 256) * p.batches;
-#ifdef TH_EXP
-    if (const char* e = getenv("TH_TILE")) {
-        if (e[0] == '1') return pick_layout16<T, 128, 128, 2>(p, ak, bk, a, b, c, stream);
-        if (e[0] == '6') return pick_layout16<T, 64, 128, 2>(p, ak, bk, a, b, c, stream);
-    }
-#endif
     if (p.M > 192 && big >= 200) return pick_layout16<T, 256, 256, 2>(p, ak, bk, a, b, c, stream);
-    // Fewer large tiles than compute units: choose between the two smaller tiles and between whole K per block and a
-    // share of it, by a model of the time (microseconds): blocks on the busiest compute unit x steps per block x the
-    // measured time of one 64-wide step of that tile, a fixed start-up and write-out, and for shared K the second pass
-    // over the fp32 partial sums.
+    // Fewer large tiles than compute units: choose between the smaller tiles (256 x 128, 128 x 128, 64 x 128) and between
+    // whole K per block and a share of it, by a model of the time (microseconds): blocks on the busiest compute unit x
+    // steps per block x the measured time of one 64-wide step of that tile, a fixed start-up and write-out, and for
+    // shared K the second pass over the fp32 partial sums.
     const bool tall = p.M > 64;
     const double steps_all = (p.K + 63) / 64;
     double best_cost = 1e30;
     int best_bm = tall ? 128 : 64;
     uint32_t best_splits = 1;
-    for (int bm : {128, 64}) {
-        if (bm == 128 && !tall) continue;
-        const double step_us = bm == 128 ? 0.55 : 0.40;
+    for (int bm : {256, 128, 64}) {
+        if ((bm == 128 && !tall) || (bm == 256 && p.M <= 192)) continue;
+        const double step_us = bm == 256 ? 1.0 : bm == 128 ? 0.55 : 0.40;
         const uint64_t tiles = static_cast<uint64_t>((p.M + bm - 1) / bm) * ((p.N + 127) / 128) * p.batches;
         for (uint32_t splits : {1u, 2u, 4u, 8u, 16u}) {
-            if (splits > 1 && (p.row_bias || splits > p.K / 256)) break;
+            if (splits > 1 && (bm == 256 || p.row_bias || splits > p.K / 256)) break;
             const double blocks = static_cast<double>(tiles) * splits;
             const double rounds = static_cast<double>((static_cast<uint64_t>(blocks) + 255) / 256);
             double cost = rounds * (steps_all / splits) * step_us + 5.0;
@@ -578,14 +572,11 @@ int run16(const GemmProblem& p, const void* a, const void* b, void* c, hipStream
             if (cost < best_cost) { best_cost = cost; best_bm = bm; best_splits = splits; }
         }
     }
-#ifdef TH_EXP
-    if (const char* e = getenv("TH_BM")) best_bm = atoi(e);
-    if (const char* e = getenv("TH_SPLITS")) best_splits = atoi(e);
-#endif
     if (best_splits > 1) {
         if (best_bm == 128) return run16_split<T, 128>(p, ak, bk, best_splits, a, b, c, stream);
         return run16_split<T, 64>(p, ak, bk, best_splits, a, b, c, stream);
     }
+    if (best_bm == 256) return pick_layout16<T, 256, 128, 2>(p, ak, bk, a, b, c, stream);
     if (best_bm == 128) return pick_layout16<T, 128, 128, 2>(p, ak, bk, a, b, c, stream);
     return pick_layout16<T, 64, 128, 2>(p, ak, bk, a, b, c, stream);
 }
