@@ -152,6 +152,10 @@ class Tensor:
         raw = types.to_storage(values, self.dtype)
         if self.dtype is not types.boolean:
             raw = np.ascontiguousarray(raw.reshape(self.shape))
+        self.write_raw(raw)
+
+    def write_raw(self, raw):
+        """Stores ``raw`` (the tensor's bytes in storage form, row-major) into a contiguous tensor: one bulk copy."""
         raw = np.ascontiguousarray(raw)
         assert raw.nbytes == self.nbytes, (raw.nbytes, self.nbytes)
         if isinstance(self.environment, Device):
