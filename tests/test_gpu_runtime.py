@@ -102,3 +102,40 @@ def test_unsupported_dtypes_report_status(device):
         lib.put_stream(C.byref(dvc), stream)
     with pytest.raises(ta.TannicError):
         ops.exp(ta.Tensor(ta.int32, (4,)).initialize(device))
+
+
+def test_released_blocks_are_reused_on_their_stream_only(device):
+    """A released block goes to the next fitting request on the same stream (stream order already separates the
+    two users); a request on another stream, or of a very different size, does not get it."""
+    lib = ta.library()
+    dvc = device.structure()
+    size = 3 << 20
+    first = lib.allocate(C.byref(dvc), size)
+    lib.deallocate(C.byref(dvc), first)
+    again = lib.allocate(C.byref(dvc), size)
+    assert again == first
+    lib.deallocate(C.byref(dvc), again)
+    small = lib.allocate(C.byref(dvc), size // 4)       # the kept block would waste three quarters
+    assert small != first
+    lib.deallocate(C.byref(dvc), small)
+    # take the pool's stream away: allocations now ride on another stream and must not see the kept block
+    held = lib.pop_stream(C.byref(dvc))
+    elsewhere = lib.allocate(C.byref(dvc), size)
+    assert elsewhere and elsewhere != first
+    lib.deallocate(C.byref(dvc), elsewhere)
+    lib.put_stream(C.byref(dvc), held)
+    back = lib.allocate(C.byref(dvc), size)
+    assert back == first
+    lib.deallocate(C.byref(dvc), back)
+
+
+def test_temporaries_reusing_blocks_keep_results_right(device, oracle):
+    """A chain of operators whose temporaries are released and handed out again at once: every result is still right."""
+    x = support.values_for(ta.float32, 5, 1, (64, 257))
+    dx, hx = ta.tensor(x, ta.float32, device), ta.tensor(x, ta.float32, ta.Host())
+    got, want = dx, hx
+    for step in range(40):
+        got = ops.add(ops.mul(got, dx), ops.neg(got)) if step % 2 else ops.sub(ops.abs(got), dx)
+        want = ops.add(ops.mul(want, hx), ops.neg(want)) if step % 2 else ops.sub(ops.abs(want), hx)
+        got, want = ops.tanh(got), ops.tanh(want)
+    support.assert_close(got.numpy(), want.numpy(), 1e-5, 1e-6, "forty operators over reused blocks")
