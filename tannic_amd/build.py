@@ -50,6 +50,7 @@ UNITS = [
     ("conv2d_k1.hip", "conv2d_k1.o", []),
     ("conv2d_pointwise.hip", "conv2d_pointwise.o", []),
     ("conv2d_stem.hip", "conv2d_stem.o", []),
+    ("conv2d_gather32.hip", "conv2d_gather32.o", []),
     ("conv2d_unfold.hip", "conv2d_unfold.o", []),
 ]
 

@@ -104,6 +104,8 @@ static int conv2d_entry(const tannic_tensor_t* x, const tannic_tensor_t* w, cons
     if (status != TANNIC_UNSUPPORTED_DTYPE) return status;
     if (!pointwise) status = conv2d_patch(p, x->dtype, x->address, w->address, pb, y->address, s);
     if (status != TANNIC_UNSUPPORTED_DTYPE) return status;
+    status = conv2d_gather32(p, x->dtype, x->address, w->address, pb, y->address, s);
+    if (status != TANNIC_UNSUPPORTED_DTYPE) return status;
     status = conv2d_unfold(p, x->dtype, x->address, w->address, pb, y->address, s);
     if (status != TANNIC_UNSUPPORTED_DTYPE) return status;
     status = conv2d_mfma(p, x->dtype, x->address, w->address, pb, y->address, s);

@@ -16,7 +16,7 @@
 //   tile, so that a lane ends up with one pixel column: the 32 lanes of a half
 //   wavefront store 32 consecutive pixels of one output channel.
 //
-// fp32 runs the same scheme on v_mfma_f32_32x32x2f32 with padded LDS rows.
+// fp32 signals take conv2d_gather32.hip, the same scheme on v_mfma_f32_32x32x2f32.
 #include "conv_common.hpp"
 
 namespace th {
