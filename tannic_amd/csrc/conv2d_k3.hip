@@ -8,7 +8,9 @@
 //     channels-last, [row][column + padding][32 channels], with real zeros in the padding,
 // in two stages: while the MFMAs of chunk c read one stage, the registers that
 // hold chunk c+1 are written to the other stage and refilled with chunk c+2
-// from global memory, one memory operation between MFMAs.
+// from global memory, one memory operation between MFMAs.  With ONE_STAGE the
+// block has a single stage (chunk c+1 is written after the MFMAs of chunk c) and
+// half the registers, so that two blocks fit a compute unit and cover each other.
 // Weights are read straight from the OIHW tensor: a thread loads the 8 channels x
 // 9 taps of one output channel (72 consecutive elements) and regroups them in
 // registers into nine 8-channel vectors.  The signal is read as 8 channels x 8
@@ -55,7 +57,7 @@ constexpr int kK3Threads = 256;
 constexpr int kK3Taps = 9;
 constexpr int kK3BCO = 64;     // output channels per block
 constexpr int kK3CH = 32;      // input channels per chunk = elements per LDS record
-constexpr int kK3Passes = 2;   // micro-blocks per thread and chunk
+constexpr int kK3Passes = 2;   // micro-blocks per thread and chunk (one where two blocks share a compute unit)
 constexpr uint32_t kK3WeightElems = kK3Taps * kK3BCO * kK3CH;
 
 struct K3Plan {
@@ -72,9 +74,10 @@ __device__ const uint4k k3_zeros = {0, 0, 0, 0};
 
 __device__ inline uint32_t k3_offset(uint32_t rec, uint32_t slot) { return rec * kK3CH + ((slot ^ ((rec >> 2) & 3u)) * 8u); }
 
-template <class T, int TN>
-__global__ __launch_bounds__(kK3Threads) void conv2d_k3_kernel(const T* x, const T* w, const T* bias, T* y, ConvProblem p, K3Plan q) {
+template <class T, int TN, bool ONE_STAGE>
+__global__ __launch_bounds__(kK3Threads, ONE_STAGE ? 2 : 1) void conv2d_k3_kernel(const T* x, const T* w, const T* bias, T* y, ConvProblem p, K3Plan q) {
     constexpr int TM = kK3BCO / 32;
+    constexpr int PASSES = ONE_STAGE ? 1 : kK3Passes;   // micro-blocks per thread and chunk
     extern __shared__ __align__(16) unsigned char k3_lds[];
     T* lds = reinterpret_cast<T*>(k3_lds);
 
@@ -92,12 +95,12 @@ __global__ __launch_bounds__(kK3Threads) void conv2d_k3_kernel(const T* x, const
     const T* w_src = w + static_cast<int64_t>(co0 + w_co < p.O ? co0 + w_co : p.O - 1) * p.ws[0] + w_c8 * 8 * kK3Taps;
     const uint32_t w_dst = k3_offset(w_co, w_c8);   // + tap * 64 records; 64 is a multiple of 16, the swizzle stays
     // signal micro-blocks: index -> (row of the patch, block of 8 columns, block of 8 channels)
-    const T* p_src[kK3Passes];
-    int64_t p_cstep[kK3Passes];
-    uint32_t p_dst[kK3Passes], p_slot[kK3Passes];
-    bool p_mine[kK3Passes];
+    const T* p_src[PASSES];
+    int64_t p_cstep[PASSES];
+    uint32_t p_dst[PASSES], p_slot[PASSES];
+    bool p_mine[PASSES];
 #pragma unroll
-    for (int ps = 0; ps < kK3Passes; ++ps) {
+    for (int ps = 0; ps < PASSES; ++ps) {
         const uint32_t mb = threadIdx.x + kK3Threads * ps;
         const uint32_t cb = mb % 4, t1 = mb / 4;
         uint32_t prow, colb;
@@ -114,7 +117,7 @@ __global__ __launch_bounds__(kK3Threads) void conv2d_k3_kernel(const T* x, const
     }
 
     uint4k wreg[kK3Taps];
-    uint4k preg[kK3Passes][8];
+    uint4k preg[PASSES][8];
     auto fetch_w = [&](int k, uint32_t chunk) {
         wreg[k] = *reinterpret_cast<const uint4k*>(w_src + static_cast<int64_t>(chunk) * (kK3CH * kK3Taps) + k * 8);
     };
@@ -150,14 +153,14 @@ __global__ __launch_bounds__(kK3Threads) void conv2d_k3_kernel(const T* x, const
 #pragma unroll
     for (int k = 0; k < kK3Taps; ++k) fetch_w(k, 0);
 #pragma unroll
-    for (int ps = 0; ps < kK3Passes; ++ps)
+    for (int ps = 0; ps < PASSES; ++ps)
 #pragma unroll
         for (int cc = 0; cc < 8; ++cc) fetch_p(ps, cc, 0);
     // the padding columns of both stages are zero and no staging write ever touches them
     {
         const uint32_t per_row = 2 * p.pad_w * 4;   // 16-byte slots of padding per patch row
         const uint32_t total = per_row * q.IH;
-        for (uint32_t i = threadIdx.x; i < 2 * total; i += kK3Threads) {
+        for (uint32_t i = threadIdx.x; i < (ONE_STAGE ? 1 : 2) * total; i += kK3Threads) {
             const uint32_t st = i >= total ? 1 : 0, r = i - st * total;
             uint32_t row, e;
             q.div_pad.divmod(r, row, e);
@@ -185,14 +188,14 @@ __global__ __launch_bounds__(kK3Threads) void conv2d_k3_kernel(const T* x, const
 #pragma unroll
     for (int k = 0; k < kK3Taps; ++k) commit_w(k, lds);
 #pragma unroll
-    for (int ps = 0; ps < kK3Passes; ++ps)
+    for (int ps = 0; ps < PASSES; ++ps)
 #pragma unroll
         for (int px = 0; px < 8; ++px) commit_p(ps, px, lds);
     if (chunks > 1) {
 #pragma unroll
         for (int k = 0; k < kK3Taps; ++k) fetch_w(k, 1);
 #pragma unroll
-        for (int ps = 0; ps < kK3Passes; ++ps)
+        for (int ps = 0; ps < PASSES; ++ps)
 #pragma unroll
             for (int cc = 0; cc < 8; ++cc) fetch_p(ps, cc, 1);
     }
@@ -229,9 +232,9 @@ __global__ __launch_bounds__(kK3Threads) void conv2d_k3_kernel(const T* x, const
         constexpr bool COMMIT = decltype(commit_tag)::value, FETCH = decltype(fetch_tag)::value;
         constexpr int PER_HALF = TM * TN, PER_TAP = 2 * PER_HALF, MFMAS = kK3Taps * PER_TAP;
         // memory operations of the chunk in order: weights out, weights in, then each pass of the signal out and in
-        constexpr int OPS = 2 * kK3Taps + kK3Passes * 16;
-        const T* stage = lds + (chunk & 1) * q.stage_elems;
-        T* next = lds + ((chunk & 1) ^ 1) * q.stage_elems;
+        constexpr int OPS = 2 * kK3Taps + PASSES * 16;
+        const T* stage = lds + (ONE_STAGE ? 0 : (chunk & 1) * q.stage_elems);
+        T* next = lds + (ONE_STAGE ? 0 : ((chunk & 1) ^ 1) * q.stage_elems);
         read_fragments(stage, 0, 0);
         __builtin_amdgcn_sched_barrier(0);
         k3_static_for<MFMAS>([&](auto m_tag) {
@@ -242,7 +245,7 @@ __global__ __launch_bounds__(kK3Threads) void conv2d_k3_kernel(const T* x, const
                 __builtin_amdgcn_sched_barrier(0);
             }
             acc[i][j] = k3_mfma<T>(fx[tap & 1][half][j], fw[tap & 1][half][i], acc[i][j]);
-            constexpr int first = m * OPS / MFMAS, last = (m + 1) * OPS / MFMAS;
+            constexpr int first = ONE_STAGE ? 0 : m * OPS / MFMAS, last = ONE_STAGE ? 0 : (m + 1) * OPS / MFMAS;
             k3_static_for<last - first>([&](auto o_tag) {
                 constexpr int o = first + decltype(o_tag)::value;
                 if constexpr (o < kK3Taps) { if constexpr (COMMIT) commit_w(o, next); }
@@ -256,6 +259,24 @@ __global__ __launch_bounds__(kK3Threads) void conv2d_k3_kernel(const T* x, const
             __builtin_amdgcn_sched_barrier(0);
         });
         __syncthreads();
+        if constexpr (ONE_STAGE && COMMIT) {
+            // the only stage is free now: the next chunk goes in, the one after it into the registers
+#pragma unroll
+            for (int k = 0; k < kK3Taps; ++k) commit_w(k, next);
+#pragma unroll
+            for (int ps = 0; ps < PASSES; ++ps)
+#pragma unroll
+                for (int px = 0; px < 8; ++px) commit_p(ps, px, next);
+            if constexpr (FETCH) {
+#pragma unroll
+                for (int k = 0; k < kK3Taps; ++k) fetch_w(k, chunk + 2);
+#pragma unroll
+                for (int ps = 0; ps < PASSES; ++ps)
+#pragma unroll
+                    for (int cc = 0; cc < 8; ++cc) fetch_p(ps, cc, chunk + 2);
+            }
+            __syncthreads();
+        }
     };
     using Yes = std::true_type;
     using No = std::false_type;
@@ -302,9 +323,9 @@ __global__ __launch_bounds__(kK3Threads) void conv2d_k3_kernel(const T* x, const
     }
 }
 
-template <class T, int TN>
+template <class T, int TN, bool ONE_STAGE>
 int launch_k3(const ConvProblem& p, const K3Plan& q, size_t lds, uint32_t blocks, const void* x, const void* w, const void* bias, void* y, hipStream_t stream) {
-    auto kernel = conv2d_k3_kernel<T, TN>;
+    auto kernel = conv2d_k3_kernel<T, TN, ONE_STAGE>;
     static std::atomic<uint64_t> configured{0};
     if (int rc = raise_lds_limit(reinterpret_cast<const void*>(kernel), 160 * 1024, configured)) return rc;
     hipLaunchKernelGGL(kernel, dim3(blocks), dim3(kK3Threads), lds, stream, static_cast<const T*>(x), static_cast<const T*>(w), static_cast<const T*>(bias),
@@ -326,18 +347,27 @@ int run_k3(const ConvProblem& p, const void* x, const void* w, const void* bias,
     // the largest number of output rows whose tile fits: pixels, LDS, staging registers
     int tn = 0;
     double best = 0.0;
-    for (uint32_t R = 1; R <= p.HO && R * p.WO <= 512; ++R) {
+    bool one_stage = false;
+    auto consider = [&](uint32_t R, bool single, double weight) {
         const uint32_t IH = (R - 1) * p.stride_h + 3;
         const size_t stage = (static_cast<size_t>(kK3WeightElems) + static_cast<size_t>(IH) * q.IWp * kK3CH) * sizeof(T);
         const uint64_t microblocks = 4ull * (p.W / 8) * IH;
-        if (2 * stage > budget || microblocks > kK3Passes * kK3Threads) break;
         const int t = R * p.WO > 256 ? 4 : 2;
+        const size_t out_bytes = static_cast<size_t>(kK3BCO) * (128 * t + 8) * sizeof(T);
+        if (microblocks > (single ? 1 : kK3Passes) * kK3Threads) return;
+        if (single ? (stage > budget / 2 || out_bytes > budget / 2 || t != 2) : 2 * stage > budget) return;
         const double fill = static_cast<double>(R * p.WO) / (128.0 * t);              // lanes with a pixel
         const double rows = static_cast<double>(p.HO) / (((p.HO + R - 1) / R) * R);    // rows of the last block that exist
         const double halo = static_cast<double>(R * p.stride_h) / IH;                  // input rows read once
-        const double score = fill * rows * (0.5 + 0.5 * halo);
-        if (score >= best) { best = score; q.R = R; q.IH = IH; tn = t; }
-    }
+        const double score = weight * fill * rows * (0.5 + 0.5 * halo);
+        if (score >= best) { best = score; q.R = R; q.IH = IH; tn = t; one_stage = single; }
+    };
+    for (uint32_t R = 1; R <= p.HO && R * p.WO <= 512; ++R) consider(R, false, 1.0);
+    // Few chunks: one stage per block and tiles of at most 256 pixels, so that two blocks share a compute unit and
+    // one block's loads, LDS writes and result rows run under the other's MFMAs.  With more than four chunks the
+    // LDS writes between the chunks, which a single stage cannot hide inside a block, cost more than that gains.
+    if (p.C <= 4 * kK3CH)
+        for (uint32_t R = 1; R <= p.HO && R * p.WO <= 256; ++R) consider(R, true, 1.25);
     if (best == 0.0) return TANNIC_UNSUPPORTED_DTYPE;
     q.row_blocks = (p.HO + q.R - 1) / q.R;
     q.co_tiles = (p.O + kK3BCO - 1) / kK3BCO;
@@ -355,9 +385,11 @@ int run_k3(const ConvProblem& p, const void* x, const void* w, const void* bias,
     if (blocks >= (1ull << 31)) return TANNIC_UNSUPPORTED_DTYPE;
     const size_t stage_bytes = static_cast<size_t>(q.stage_elems) * sizeof(T);
     const size_t out_bytes = static_cast<size_t>(kK3BCO) * (128 * tn + 8) * sizeof(T);
-    const size_t lds = 2 * stage_bytes > out_bytes ? 2 * stage_bytes : out_bytes;
-    if (tn == 4) return launch_k3<T, 4>(p, q, lds, static_cast<uint32_t>(blocks), x, w, bias, y, stream);
-    return launch_k3<T, 2>(p, q, lds, static_cast<uint32_t>(blocks), x, w, bias, y, stream);
+    const size_t held = (one_stage ? 1 : 2) * stage_bytes;
+    const size_t lds = held > out_bytes ? held : out_bytes;
+    if (one_stage) return launch_k3<T, 2, true>(p, q, lds, static_cast<uint32_t>(blocks), x, w, bias, y, stream);
+    if (tn == 4) return launch_k3<T, 4, false>(p, q, lds, static_cast<uint32_t>(blocks), x, w, bias, y, stream);
+    return launch_k3<T, 2, false>(p, q, lds, static_cast<uint32_t>(blocks), x, w, bias, y, stream);
 }
 
 int conv2d_k3(const ConvProblem& p, int dtype, const void* x, const void* w, const void* bias, void* y, hipStream_t stream) {

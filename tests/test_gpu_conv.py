@@ -45,6 +45,10 @@ CASES = {
     "stem_c4_k5x8_s3x2": ((1, 4, 17, 32), (8, 4, 5, 8), (3, 2), (0, 4)),
     "stem_c2_k7_s2_tall": ((1, 2, 64, 16), (5, 2, 7, 7), (2, 2), (3, 3)),
     "k3_rect_stride_pad": ((1, 96, 13, 24), (64, 96, 3, 3), (2, 1), (0, 2)),
+    # more than four chunks: two LDS stages per block (up to four chunks a block has one stage and shares its compute unit)
+    "k3_two_stages_160ch": ((1, 160, 12, 16), (64, 160, 3, 3), (1, 1), (1, 1)),
+    "k3_two_stages_256ch_s2": ((2, 256, 16, 16), (40, 256, 3, 3), (2, 2), (1, 1)),
+    "k3_one_stage_ragged_rows": ((2, 64, 19, 56), (64, 64, 3, 3), (1, 1), (1, 1)),
     # 1x1 kernels with the weights resident in registers: 64..256 channels in, multiples of 256 out, stride 1 and 2,
     # pixel counts that end inside a 64-pixel tile, several images per worker
     "k1_s2_256ch": ((2, 256, 24, 24), (256, 256, 1, 1), (2, 2), (0, 0)),
