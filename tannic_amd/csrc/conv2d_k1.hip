@@ -76,7 +76,11 @@ __global__ __launch_bounds__(kK1Threads) void conv2d_k1_kernel(const T* x, const
     const int wave = threadIdx.x / 64, lane = threadIdx.x % 64;
     T* stage = lds + 2 * BUFFER + wave * (kK1CoWave * kK1Pitch);
 
-    const uint32_t group = blockIdx.x / q.workers, worker = blockIdx.x % q.workers;
+    const uint32_t group = blockIdx.x / q.workers;
+    // workgroups go round the eight dies in turn: consecutive workers (tiles that share cache lines of the signal
+    // and of the result) are given to workgroups of one die, so that its L2 merges what they share
+    uint32_t worker = blockIdx.x % q.workers;
+    if (q.workers % 8 == 0) worker = (worker % 8) * (q.workers / 8) + worker / 8;
     const uint32_t co0 = group * kK1CoBlock + wave * kK1CoWave;
 
     // ---- this thread's micro-block: 8 channels x 8 pixels ----------------------------------------

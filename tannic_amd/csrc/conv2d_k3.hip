@@ -81,8 +81,12 @@ __global__ __launch_bounds__(kK3Threads, ONE_STAGE ? 2 : 1) void conv2d_k3_kerne
     extern __shared__ __align__(16) unsigned char k3_lds[];
     T* lds = reinterpret_cast<T*>(k3_lds);
 
+    // workgroups go round the eight dies in turn: neighbouring tiles (which share rows of the signal and cache
+    // lines of the result) are given to workgroups of one die, so that its L2 serves what they share
+    uint32_t block = blockIdx.x;
+    if (gridDim.x % 8 == 0) block = (block % 8) * (gridDim.x / 8) + block / 8;
     uint32_t tile, ct;
-    q.div_co_tiles.divmod(blockIdx.x, tile, ct);
+    q.div_co_tiles.divmod(block, tile, ct);
     uint32_t n, rb;
     q.div_row_blocks.divmod(tile, n, rb);
     const uint32_t oh0 = rb * q.R, co0 = ct * kK3BCO;
