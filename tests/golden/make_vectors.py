@@ -98,7 +98,7 @@ case("polar", "tests/cpu/test-complex.cpp:40-62", "polar", [t([2,2],[1,6,2,3]), 
 freq=[1.0,0.0,1.0,0.0,1.0,0.0, 0.5403,0.8415,0.9989,0.0464,1.0,0.0022, -0.4161,0.9093,0.9957,0.0927,1.0,0.0043, -0.99,0.1411,0.9903,0.1388,1.0,0.0065,
       -0.6536,-0.7568,0.9828,0.1846,1.0,0.0086, 0.2837,-0.9589,0.9732,0.23,0.9999,0.0108, 0.9602,-0.2794,0.9615,0.2749,0.9999,0.0129, 0.7539,0.657,0.9477,0.3192,0.9999,0.0151]
 case("llama_freq_cis", "tests/cpu/test-complex.cpp:64-108", "freq_cis", [], t([8,3,2],freq,"float64"), model_dimension=6, sequence_length=8, theta=10000.0, rtol=0.1, atol=0.1)
-# ---- 16-bit conversions (tests/test-types.cpp:45-166) and the survey's native-accumulation known answers
+# ---- 16-bit conversions (tests/test-types.cpp:45-166) and known answers of 16-bit native accumulation (sums of ones stall at 2048)
 case("half_bits", "tests/test-types.cpp:45-166", "half_bits", [], None,
      pairs=[[0.0,0x0000],[-0.0,0x8000],[1.0,0x3C00],[-2.0,0xC000],["inf",0x7C00],["-inf",0xFC00],[5.960464477539063e-08,0x0001],[65504.0,0x7BFF],[1e5,0x7C00]])
 case("bhalf_bits", "tests/test-types.cpp:45-166", "bhalf_bits", [], None,
