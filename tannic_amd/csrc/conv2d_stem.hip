@@ -326,12 +326,14 @@ int run_stem(const ConvProblem& p, const void* x, const void* w, const void* bia
     if (lds < raw_bytes) lds = raw_bytes;
     if (lds > 64 * 1024) return TANNIC_UNSUPPORTED_DTYPE;
     q.co_tiles = (p.O + kStemBCO - 1) / kStemBCO;
-    static int cus = 0;   // compute units of the device, asked once
+    static std::atomic<int> known_cus{0};   // compute units of the device, asked once
+    int cus = known_cus.load(std::memory_order_relaxed);
     if (cus == 0) {
         cus = 256;
         hipDeviceProp_t prop;
         int dev = 0;
         if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess && prop.multiProcessorCount > 0) cus = prop.multiProcessorCount;
+        known_cus.store(cus, std::memory_order_relaxed);
     }
     // strips: about two blocks per compute unit, at least KH rows each so that the first tile's rows pay off
     const uint64_t want = static_cast<uint64_t>(2 * cus);
