@@ -561,12 +561,14 @@ int run16(const GemmProblem& p, const void* a, const void* b, void* c, hipStream
     uint32_t best_splits = 1;
     for (int bm : {256, 128, 64}) {
         if ((bm == 128 && !tall) || (bm == 256 && p.M <= 192)) continue;
-        const double step_us = bm == 256 ? 1.0 : bm == 128 ? 0.55 : 0.40;
         const uint64_t tiles = static_cast<uint64_t>((p.M + bm - 1) / bm) * ((p.N + 127) / 128) * p.batches;
         for (uint32_t splits : {1u, 2u, 4u, 8u, 16u}) {
             if (splits > 1 && (bm == 256 || p.row_bias || splits > p.K / 256)) break;
             const double blocks = static_cast<double>(tiles) * splits;
             const double rounds = static_cast<double>((static_cast<uint64_t>(blocks) + 255) / 256);
+            // a step costs more the more compute units pull operands through the L2s at the same time
+            const double busy = blocks < 256.0 ? blocks / 256.0 : 1.0;
+            const double step_us = bm == 256 ? 1.0 : bm == 128 ? 0.375 + 0.175 * busy : 0.30 + 0.075 * busy;
             double cost = rounds * (steps_all / splits) * step_us + 5.0;
             if (splits > 1) cost += 4.0 + (splits + 0.5) * static_cast<double>(p.M) * p.N * p.batches * 4.0 / 5.0e6;
             if (cost < best_cost) { best_cost = cost; best_bm = bm; best_splits = splits; }
