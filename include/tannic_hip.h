@@ -277,8 +277,10 @@ int tannic_hip_argmean(const tannic_tensor_t* src, tannic_tensor_t* dst, tannic_
 int tannic_hip_argmax(const tannic_tensor_t* src, tannic_tensor_t* dst, tannic_stream_t stream, uint8_t axis);
 int tannic_hip_argmin(const tannic_tensor_t* src, tannic_tensor_t* dst, tannic_stream_t stream, uint8_t axis);
 /* Value max / min over an axis.  No counterpart in the reference (it has only
- * argmax/argmin, include/tannic/reductions.hpp:101-193); defined as
- * src[argmax(src, axis)] resp. src[argmin(src, axis)], dst dtype = src dtype. */
+ * argmax/argmin, include/tannic/reductions.hpp:101-193).  The largest resp.
+ * smallest number of the slice, +0 counting as larger than -0 and NaNs as
+ * absent; a slice in which nothing exceeds -inf (+inf, the integer limits)
+ * yields its first element, i.e. src[argmax].  dst dtype = src dtype. */
 int tannic_hip_max(const tannic_tensor_t* src, tannic_tensor_t* dst, tannic_stream_t stream, uint8_t axis);
 int tannic_hip_min(const tannic_tensor_t* src, tannic_tensor_t* dst, tannic_stream_t stream, uint8_t axis);
 
@@ -305,7 +307,7 @@ int tannic_hip_conv2d_biased(const tannic_tensor_t* signal, const tannic_tensor_
 /* ------------------------------------------------------------------ *
  * Operators with no counterpart in the reference.  A Tannic program
  * spells them today as chains of the operators above (there is no
- * division, no cast, no softmax in include/tannic/*.hpp); each is one
+ * division, no cast, no softmax in the headers under include/tannic); each is one
  * pass here.  16- and 32-bit types are evaluated in float, float64 in
  * double, and rounded once.
  * ------------------------------------------------------------------ */

@@ -33,7 +33,9 @@
  *   two known answers "fp16 dot of 4096 ones = 2048" and "fp16 sum of 4096
  *   ones = 2048" for native mode; native mode is otherwise PARITY UNPINNED and
  *   only informational.
- *   max/min: not in the reference; defined as src[argmax]/src[argmin].
+ *   max/min: not in the reference; defined as the largest/smallest number of the
+ *   slice with +0 above -0 and NaNs absent (IEEE 754-2019 maximumNumber), and the
+ *   slice's first element where nothing exceeds -inf/+inf (the integer limits).
  */
 #include <cmath>
 #include <complex>
@@ -441,6 +443,30 @@ int arg_run(const tannic_tensor_t* src, tannic_tensor_t* dst, uint8_t ax, bool v
         }
         if (values) static_cast<T*>(dst->address)[slot] = ps[base + best * step];
         else static_cast<int64_t*>(dst->address)[slot] = best;
+    });
+    return TANNIC_SUCCESS;
+}
+
+/* value max/min (not in the reference): IEEE 754-2019 maximumNumber / minimumNumber folded over the slice from
+ * -inf / +inf (the integer limits): numbers by value, +0 above -0, NaNs skipped; where no element beats the start
+ * the slice's first element is the answer (what src[argmax] would be). */
+template <class T, bool MAX>
+int extreme_run(const tannic_tensor_t* src, tannic_tensor_t* dst, uint8_t ax) {
+    const T* ps = static_cast<const T*>(src->address);
+    for_each_slice(src, ax, [&](size_t slot, int64_t base, int64_t step, size_t R) {
+        const T start = arg_init<T, MAX>();
+        T acc = start;
+        bool beaten = false;
+        for (size_t r = 0; r < R; ++r) {
+            const T v = ps[base + static_cast<int64_t>(r) * step];
+            bool wins = MAX ? (v > acc) : (v < acc);
+            if constexpr (!is_int<T>) {
+                const double dv = static_cast<double>(static_cast<float>(v)) , da = static_cast<double>(static_cast<float>(acc));
+                if (dv == 0.0 && da == 0.0) wins = MAX ? (std::signbit(da) && !std::signbit(dv)) : (!std::signbit(da) && std::signbit(dv));
+            }
+            if (wins) { acc = v; beaten = true; }
+        }
+        static_cast<T*>(dst->address)[slot] = beaten ? acc : ps[base];
     });
     return TANNIC_SUCCESS;
 }
@@ -856,15 +882,15 @@ int oracle_argmin(const tannic_tensor_t* s, tannic_tensor_t* d, uint8_t ax) {
     with_type(s->dtype, [&](auto t) { using T = typename decltype(t)::type; if constexpr (!is_cplx<T>) st = arg_run<T, false>(s, d, ax, false); });
     return st;
 }
-/* value max/min: src[argmax], src[argmin] (not in the reference) */
+/* value max/min (not in the reference): extreme_run above */
 int oracle_max(const tannic_tensor_t* s, tannic_tensor_t* d, uint8_t ax) {
     int st = TANNIC_UNSUPPORTED_DTYPE;
-    with_type(s->dtype, [&](auto t) { using T = typename decltype(t)::type; if constexpr (!is_cplx<T>) st = arg_run<T, true>(s, d, ax, true); });
+    with_type(s->dtype, [&](auto t) { using T = typename decltype(t)::type; if constexpr (!is_cplx<T>) st = extreme_run<T, true>(s, d, ax); });
     return st;
 }
 int oracle_min(const tannic_tensor_t* s, tannic_tensor_t* d, uint8_t ax) {
     int st = TANNIC_UNSUPPORTED_DTYPE;
-    with_type(s->dtype, [&](auto t) { using T = typename decltype(t)::type; if constexpr (!is_cplx<T>) st = arg_run<T, false>(s, d, ax, true); });
+    with_type(s->dtype, [&](auto t) { using T = typename decltype(t)::type; if constexpr (!is_cplx<T>) st = extreme_run<T, false>(s, d, ax); });
     return st;
 }
 

@@ -111,9 +111,24 @@ struct ArgOp {
     __device__ static inline int64_t finish(A acc, uint32_t) { return static_cast<int64_t>(acc.index); }
 };
 
-// Value max / min = src[argmax] / src[argmin] without carrying the index: the strict maximum from the
-// -inf (lowest) start IS that element's value whenever anything beats the start; when nothing does
-// (a slice of NaN, of -inf, of the integer minimum) argmax is 0 and the answer is the slice's first element.
+// The larger (smaller) of two values the way the hardware's maximum instructions order them: numbers by value,
+// +0 above -0, a NaN loses against a number.  The order of the operands does not matter, so partial results may meet
+// in any order and still give the same bits.
+template <class T, bool MAX> __device__ inline T extreme(T a, T b) {
+    if constexpr (std::is_same_v<T, float>) return MAX ? __builtin_fmaxf(a, b) : __builtin_fminf(a, b);
+    else if constexpr (std::is_same_v<T, double>) return MAX ? __builtin_fmax(a, b) : __builtin_fmin(a, b);
+    else if constexpr (std::is_same_v<T, f16>) {
+        const float r = MAX ? __builtin_fmaxf(static_cast<float>(a), static_cast<float>(b)) : __builtin_fminf(static_cast<float>(a), static_cast<float>(b));
+        return static_cast<f16>(r);   // one of the operands: exact
+    } else if constexpr (std::is_same_v<T, bf16>) {
+        const float r = MAX ? __builtin_fmaxf(to_float(a), to_float(b)) : __builtin_fminf(to_float(a), to_float(b));
+        return bf16{static_cast<uint16_t>(__builtin_bit_cast(uint32_t, r) >> 16)};   // one of the operands: exact
+    } else return (MAX ? a > b : b > a) ? a : b;
+}
+
+// Value max / min: the largest (smallest) number of the slice, +0 counting as larger than -0 and NaNs as absent.
+// The fold starts from -inf / +inf (the lowest / highest integer); when nothing beats the start (a slice of NaN,
+// of -inf, of the integer minimum) the answer is the slice's first element, which is also what argmax points at.
 template <class T, bool MAX>
 struct ValueOp {
     using S = T;
@@ -122,8 +137,8 @@ struct ValueOp {
     static constexpr bool needs_source = true;
     static constexpr bool value_only = true;
     __device__ static inline A init() { return arg_start<T, MAX>(); }
-    __device__ static inline A step(A acc, T v, uint32_t) { return (MAX ? gt(v, acc) : gt(acc, v)) ? v : acc; }
-    __device__ static inline A combine(A x, A y) { return (MAX ? gt(y, x) : gt(x, y)) ? y : x; }
+    __device__ static inline A step(A acc, T v, uint32_t) { return extreme<T, MAX>(acc, v); }
+    __device__ static inline A combine(A x, A y) { return extreme<T, MAX>(x, y); }
 };
 
 template <class Op, class = void> struct is_value_only { static constexpr bool value = false; };

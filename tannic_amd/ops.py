@@ -274,12 +274,14 @@ def argmin(x, axis=-1, keepdim=False):
 
 
 def max(x, axis=-1, keepdim=False):
-    """Largest value along ``axis``; the reference has no such reduction."""
+    """Largest number along ``axis`` (+0 above -0, NaNs skipped; the first element where nothing exceeds -inf);
+    the reference has no such reduction."""
     return _reduce("max", x, axis, keepdim, x.dtype)
 
 
 def min(x, axis=-1, keepdim=False):
-    """Smallest value along ``axis``; the reference has no such reduction."""
+    """Smallest number along ``axis`` (-0 below +0, NaNs skipped; the first element where nothing is below +inf);
+    the reference has no such reduction."""
     return _reduce("min", x, axis, keepdim, x.dtype)
 
 

@@ -111,6 +111,29 @@ def test_argmax_with_nan_and_infinities(device):
     support.assert_bit_exact(ops.argmax(di, 1).storage(), ops.argmax(hi, 1).storage(), "int8 all lowest")
 
 
+@pytest.mark.parametrize("dtype", [ta.float32, ta.float64, ta.float16, ta.bfloat16], ids=str)
+def test_value_max_min_order_signed_zeros_and_skip_nan(device, dtype):
+    """max / min are the largest / smallest NUMBER of a slice with +0 above -0, whichever lane, wavefront or block
+    holds which zero; NaNs only show where nothing exceeds the start value (then the slice's first element comes back)."""
+    rows, n = 6, 5000
+    x = np.zeros((rows, n))
+    x[0, :] = 0.0; x[0, 4321] = -0.0           # one -0 among +0
+    x[1, :] = -0.0; x[1, 77] = 0.0             # one +0 among -0
+    x[2, ::2] = -0.0                           # alternating
+    x[3, :] = np.nan; x[3, 1234] = -0.0; x[3, 4000] = 0.0
+    x[4, :] = np.nan                           # nothing but NaN: the first element
+    x[5, :] = -3.0; x[5, 9] = np.nan; x[5, 4999] = -0.0
+    h, d = support.both(x, dtype, device)
+    for axis in (1, 0):
+        for op in ("max", "min"):
+            want, got = getattr(ops, op)(h, axis), getattr(ops, op)(d, axis)
+            support.assert_bit_exact(got.storage(), want.storage(), f"{op} axis={axis} {dtype}")
+    got_max, got_min = ops.max(d, 1).numpy().astype(np.float64), ops.min(d, 1).numpy().astype(np.float64)
+    assert not np.signbit(got_max[:4]).any() and np.signbit(got_min[:4]).all()      # +0 is the maximum, -0 the minimum
+    assert np.isnan(got_max[4]) and np.isnan(got_min[4])
+    assert got_max[5] == 0 and np.signbit(got_max[5]) and got_min[5] == -3.0
+
+
 @pytest.mark.parametrize("dtype", [ta.float32, ta.int32, ta.float16], ids=str)
 def test_strided_sources(device, dtype):
     h, d = support.both(np.round(support.values_for(dtype, SEED, 6, (12, 30, 20)).astype(np.float64)), dtype, device)

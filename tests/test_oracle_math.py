@@ -173,7 +173,7 @@ def test_conv1x1_is_a_gemm_and_padding_taps_add_nothing(oracle):
 
 
 @pytest.mark.parametrize("dtype", [ta.float32, ta.int32, ta.float16], ids=str)
-def test_value_max_min_are_the_elements_at_argmax_argmin(oracle, dtype):
+def test_value_max_min_against_numpy(oracle, dtype):
     x = support.values_for(dtype, SEED, 27, (4, 9, 5), -3, 3)
     X = support.host_tensor(x, dtype)
     for axis in (0, 1, 2):
@@ -182,6 +182,21 @@ def test_value_max_min_are_the_elements_at_argmax_argmin(oracle, dtype):
         idx = ops.argmax(X, axis).storage()
         support.assert_bit_exact(idx, x.argmax(axis=axis), f"argmax {axis}")  # numpy also returns the first occurrence
         support.assert_bit_exact(ops.argmin(X, axis).storage(), x.argmin(axis=axis), f"argmin {axis}")
+
+
+def test_value_max_min_signed_zeros_and_nan(oracle):
+    """+0 is above -0 wherever they stand, NaNs are skipped, and a slice where nothing exceeds the start gives back its
+    first element: checked against the definition written out by hand."""
+    x = np.array([[0.0, -0.0, 0.0], [-0.0, 0.0, -0.0], [np.nan, -0.0, 0.0], [np.nan, np.nan, np.nan], [-np.inf, np.nan, -np.inf],
+                  [np.nan, -2.0, 5.0], [np.inf, np.nan, np.inf]], dtype=np.float32)
+    X = support.host_tensor(x, ta.float32)
+    got_max, got_min = ops.max(X, 1).storage().view(np.uint32), ops.min(X, 1).storage().view(np.uint32)
+    bits = lambda v: np.array(v, dtype=np.float32).view(np.uint32)
+    assert (got_max[:3] == bits(0.0)).all() and (got_min[:3] == bits(-0.0)).all()
+    assert got_max[3] == x[3, 0].view(np.uint32) and got_min[3] == x[3, 0].view(np.uint32)      # all NaN: the first element
+    assert got_max[4] == bits(-np.inf) and got_min[4] == bits(-np.inf)
+    assert got_max[5] == bits(5.0) and got_min[5] == bits(-2.0)
+    assert got_max[6] == bits(np.inf) and got_min[6] == bits(np.inf)                            # nothing below +inf: the first element
 
 
 def test_polar_has_the_radius_as_modulus(oracle):
