@@ -61,6 +61,21 @@ template <class T> constexpr bool is16 = std::is_same_v<T, f16> || std::is_same_
 template <class T> constexpr bool is_int = std::is_integral_v<T>;
 template <class T> constexpr bool is_cplx = std::is_same_v<T, c64> || std::is_same_v<T, c128>;
 
+/* the dtype code of a C++ element type */
+template <class T> constexpr int code_of() {
+    if constexpr (std::is_same_v<T, int8_t>) return TANNIC_INT8;
+    else if constexpr (std::is_same_v<T, int16_t>) return TANNIC_INT16;
+    else if constexpr (std::is_same_v<T, int32_t>) return TANNIC_INT32;
+    else if constexpr (std::is_same_v<T, int64_t>) return TANNIC_INT64;
+    else if constexpr (std::is_same_v<T, f16>) return TANNIC_FLOAT16;
+    else if constexpr (std::is_same_v<T, b16>) return TANNIC_BFLOAT16;
+    else if constexpr (std::is_same_v<T, float>) return TANNIC_FLOAT32;
+    else if constexpr (std::is_same_v<T, double>) return TANNIC_FLOAT64;
+    else if constexpr (std::is_same_v<T, c64>) return TANNIC_COMPLEX64;
+    else if constexpr (std::is_same_v<T, c128>) return TANNIC_COMPLEX128;
+    else return -1;
+}
+
 /* Calls f(tag<T>) for the C++ type behind a dtype code; returns false if none. */
 template <class F> bool with_type(int dtype, F&& f) {
     switch (dtype) {
@@ -218,7 +233,12 @@ int binary_dispatch(const tannic_tensor_t* a, const tannic_tensor_t* b, tannic_t
             using S0 = typename decltype(ta)::type;
             using S1 = typename decltype(tb)::type;
             using D = typename Result<S0, S1>::type;
-            if constexpr (!std::is_void_v<D>) st = binary_run<S0, S1, D, Op>(a, b, dst);
+            /* The reference's table writes elements of type D, the front end sizes the destination by promotion
+             * (include/tannic/operations.hpp): for the pairs where the two differ (an integer with a 16-bit float:
+             * the table says float) the reference overruns the destination; those are refused here, as on the device. */
+            if constexpr (!std::is_void_v<D>) {
+                if (code_of<D>() == static_cast<int>(dst->dtype)) st = binary_run<S0, S1, D, Op>(a, b, dst);
+            }
         });
     });
     return st;
@@ -355,6 +375,9 @@ int cmp_run(const tannic_tensor_t* a, const tannic_tensor_t* b, tannic_tensor_t*
 
 template <int K> int cmp_dispatch(const tannic_tensor_t* a, const tannic_tensor_t* b, tannic_tensor_t* dst) {
     int st = TANNIC_UNSUPPORTED_DTYPE; /* :108-202: ints and real floats */
+    /* the reference dispatches on the first operand and reads the second as the same type, past the end of a
+     * narrower one: operands of different dtypes are refused here, as on the device */
+    if (a->dtype != b->dtype) return st;
     with_type(a->dtype, [&](auto t) {
         using T = typename decltype(t)::type;
         if constexpr (!is_cplx<T>) st = cmp_run<T, K>(a, b, dst);
@@ -901,7 +924,12 @@ int oracle_gemm(const tannic_tensor_t* a, const tannic_tensor_t* b, tannic_tenso
             using S0 = typename decltype(ta)::type;
             using S1 = typename decltype(tb)::type;
             using D = typename GemmResult<S0, S1>::type;
-            if constexpr (!std::is_void_v<D>) st = gemm_run<S0, S1, D>(a, b, c);
+            /* as for the binary operations: a pair whose table type is not the dtype the front end gives the product
+             * (int8/int16 with a 16-bit float: the table says float, include/tannic/transformations.hpp:112-139 says
+             * the 16-bit type) overruns the destination in the reference and is refused here */
+            if constexpr (!std::is_void_v<D>) {
+                if (code_of<D>() == static_cast<int>(c->dtype)) st = gemm_run<S0, S1, D>(a, b, c);
+            }
         });
     });
     return st;
@@ -974,6 +1002,8 @@ int oracle_concat(const tannic_tensor_t* a, const tannic_tensor_t* b, tannic_ten
 int oracle_outer(const tannic_tensor_t* a, const tannic_tensor_t* b, tannic_tensor_t* d) {
     const int x = a->dtype, y = b->dtype;
 #define OUTER(X, Y, TA, TB, TD) if (x == X && y == Y) return outer_run<TA, TB, TD>(a, b, d);
+    OUTER(TANNIC_INT8, TANNIC_INT32, int8_t, int32_t, int32_t) OUTER(TANNIC_INT32, TANNIC_INT8, int32_t, int8_t, int32_t)
+    OUTER(TANNIC_INT16, TANNIC_INT32, int16_t, int32_t, int32_t) OUTER(TANNIC_INT32, TANNIC_INT16, int32_t, int16_t, int32_t)
     OUTER(TANNIC_INT8, TANNIC_INT64, int8_t, int64_t, int64_t) OUTER(TANNIC_INT64, TANNIC_INT8, int64_t, int8_t, int64_t)
     OUTER(TANNIC_INT16, TANNIC_INT64, int16_t, int64_t, int64_t) OUTER(TANNIC_INT64, TANNIC_INT16, int64_t, int16_t, int64_t)
     OUTER(TANNIC_INT32, TANNIC_INT64, int32_t, int64_t, int64_t) OUTER(TANNIC_INT64, TANNIC_INT32, int64_t, int32_t, int64_t)
@@ -1009,6 +1039,7 @@ int oracle_tril(const tannic_tensor_t* s, tannic_tensor_t* d, int k) {
 
 /* 1 close, 0 not close, -1 unsupported dtype (the reference throws, src/cpu/val.cpp:81) */
 int oracle_allclose(const tannic_tensor_t* a, const tannic_tensor_t* b, double rtol, double atol) {
+    if (a->dtype != b->dtype) return -1; /* src/cpu/val.cpp:73-83 would read b as a's type */
     switch (a->dtype) {
         case TANNIC_FLOAT16: return allclose_run<f16>(a, b, rtol, atol);
         case TANNIC_BFLOAT16: return allclose_run<b16>(a, b, rtol, atol);

@@ -122,7 +122,10 @@ int binary(const tannic_tensor_t* a, const tannic_tensor_t* b, tannic_tensor_t* 
             using A = typename decltype(ta)::type;
             using B = typename decltype(tb)::type;
             using R = typename BinaryResult<A, B, K>::type;
-            if constexpr (!std::is_void_v<R>) status = run_binary<A, B, R, K>(a, b, dst, as_stream(stream));
+            if constexpr (!std::is_void_v<R>) {
+                if (!destination_is(dst, dtype_code<R>(), "binary op: the destination's dtype is not the pair's result type")) status = TANNIC_ERROR;
+                else status = run_binary<A, B, R, K>(a, b, dst, as_stream(stream));
+            }
         });
     });
     return status;

@@ -136,6 +136,29 @@ template <class F> inline bool with_type(int dtype, F&& f) {
     }
 }
 
+// The dtype code of an element type (the inverse of with_type).
+template <class T> constexpr int dtype_code() {
+    if constexpr (std::is_same_v<T, int8_t>) return TANNIC_INT8;
+    else if constexpr (std::is_same_v<T, int16_t>) return TANNIC_INT16;
+    else if constexpr (std::is_same_v<T, int32_t>) return TANNIC_INT32;
+    else if constexpr (std::is_same_v<T, int64_t>) return TANNIC_INT64;
+    else if constexpr (std::is_same_v<T, f16>) return TANNIC_FLOAT16;
+    else if constexpr (std::is_same_v<T, bf16>) return TANNIC_BFLOAT16;
+    else if constexpr (std::is_same_v<T, float>) return TANNIC_FLOAT32;
+    else if constexpr (std::is_same_v<T, double>) return TANNIC_FLOAT64;
+    else if constexpr (std::is_same_v<T, c64>) return TANNIC_COMPLEX64;
+    else if constexpr (std::is_same_v<T, c128>) return TANNIC_COMPLEX128;
+    else return -1;
+}
+
+// A kernel writes elements of one type; a destination described with another dtype would be over- or under-run.
+// (The reference's kernels take the front end's word for it; here a descriptor that does not fit is refused.)
+inline bool destination_is(const tannic_tensor_t* dst, int dtype, const char* who) {
+    if (static_cast<int>(dst->dtype) == dtype) return true;
+    set_error_text(who);
+    return false;
+}
+
 inline size_t dtype_size(int dtype) {
     switch (dtype) {
         case TANNIC_INT8: return 1;

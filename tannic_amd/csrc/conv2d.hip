@@ -63,6 +63,11 @@ static int conv2d_entry(const tannic_tensor_t* x, const tannic_tensor_t* w, cons
         default: return TANNIC_UNSUPPORTED_DTYPE;
     }
     if (x->rank != 4 || w->rank != 4 || y->rank != 4 || (bias && bias->rank != 1)) return TANNIC_ERROR;
+    if (!destination_is(y, x->dtype, "conv2d: the result's dtype is not the signal's")) return TANNIC_ERROR;
+    if (bias && bias->dtype != x->dtype) {
+        set_error_text("conv2d: the bias's dtype is not the signal's");
+        return TANNIC_ERROR;
+    }
     if (stride[0] == 0 || stride[1] == 0) return TANNIC_ERROR;
     const size_t N = x->shape.sizes[0], C = x->shape.sizes[1], H = x->shape.sizes[2], W = x->shape.sizes[3];
     const size_t O = w->shape.sizes[0], KC = w->shape.sizes[1], KH = w->shape.sizes[2], KW = w->shape.sizes[3];
@@ -134,6 +139,7 @@ static int conv1d_entry(const tannic_tensor_t* x, const tannic_tensor_t* w, tann
         default: return TANNIC_UNSUPPORTED_DTYPE;
     }
     if (x->rank != 3 || w->rank != 3 || y->rank != 3) return TANNIC_ERROR;
+    if (!destination_is(y, x->dtype, "conv1d: the result's dtype is not the signal's")) return TANNIC_ERROR;
     auto with_row = [](const tannic_tensor_t* t) {
         tannic_tensor_t r = *t;
         r.rank = 4;

@@ -180,7 +180,10 @@ int tannic_hip_div(const tannic_tensor_t* a, const tannic_tensor_t* b, tannic_te
             using B = typename decltype(tb)::type;
             if constexpr (!std::is_same_v<A, c64> && !std::is_same_v<A, c128> && !std::is_same_v<B, c64> && !std::is_same_v<B, c128>) {
                 using R = typename QuotientType<A, B>::type;
-                if constexpr (!std::is_void_v<R>) status = run_pair<DivF<A, B, R>, A, B, R>(a, b, dst, as_stream(stream));
+                if constexpr (!std::is_void_v<R>) {
+                    if (!destination_is(dst, dtype_code<R>(), "div: the destination's dtype is not the pair's quotient type")) status = TANNIC_ERROR;
+                    else status = run_pair<DivF<A, B, R>, A, B, R>(a, b, dst, as_stream(stream));
+                }
             }
         });
     });

@@ -178,6 +178,10 @@ extern "C" int tannic_hip_gemm(const tannic_tensor_t* a, const tannic_tensor_t* 
             using B = typename decltype(tb)::type;
             using D = typename GemmResult<A, B>::type;
             if constexpr (!std::is_void_v<D>) {
+                if (!destination_is(dst, dtype_code<D>(), "gemm: the destination's dtype is not the pair's product type")) {
+                    status = TANNIC_ERROR;
+                    return;
+                }
                 GemmProblem p;
                 status = describe_gemm(a, b, dst, p);
                 if (status != TANNIC_SUCCESS) return;

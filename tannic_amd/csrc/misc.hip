@@ -157,7 +157,10 @@ int complex_entry(const tannic_tensor_t* a, const tannic_tensor_t* b, tannic_ten
                                    (std::is_integral_v<B> || std::is_floating_point_v<B>);
             if constexpr (plain) {
                 using C = typename ComplexResult<A, B>::type;
-                if constexpr (!std::is_void_v<C>) status = run_complex<A, B, C, POLAR>(a, b, dst, as_stream(stream));
+                if constexpr (!std::is_void_v<C>) {
+                    if (!destination_is(dst, dtype_code<cplx<C>>(), "complex: the destination's dtype is not the pair's complex type")) status = TANNIC_ERROR;
+                    else status = run_complex<A, B, C, POLAR>(a, b, dst, as_stream(stream));
+                }
             }
         });
     });
@@ -274,8 +277,13 @@ template <int K>
 int compare_entry(const tannic_tensor_t* a, const tannic_tensor_t* b, tannic_tensor_t* dst, tannic_stream_t stream) {
     if (!a || !b || !dst) return TANNIC_ERROR;
     int status = TANNIC_UNSUPPORTED_DTYPE;
-    // dispatch on the first source only; the second is read as the same type
-    // (src/cpu/cmps.cpp:108-202)
+    // The CPU path dispatches on the first source only and reads the second as the same type (src/cpu/cmps.cpp:108-202),
+    // which runs past the end of a narrower second operand: operands of different dtypes are refused here.
+    if (a->dtype != b->dtype) {
+        set_error_text("comparison: operands of different dtypes");
+        return TANNIC_UNSUPPORTED_DTYPE;
+    }
+    if (!destination_is(dst, TANNIC_BOOLEAN, "comparison: the destination is not boolean")) return TANNIC_ERROR;
     with_type(a->dtype, [&](auto t) {
         using T = typename decltype(t)::type;
         if constexpr (!std::is_same_v<T, c64> && !std::is_same_v<T, c128>)
@@ -353,6 +361,7 @@ extern "C" {
 int tannic_hip_scale(const tannic_tensor_t* src, const tannic_scalar_t* sc, tannic_tensor_t* dst, tannic_stream_t stream) {
     if (!src || !sc || !dst || !sc->address) return TANNIC_ERROR;
     if (src->dtype != sc->dtype) return TANNIC_UNSUPPORTED_DTYPE;
+    if (!destination_is(dst, src->dtype, "scale: the destination's dtype is not the source's")) return TANNIC_ERROR;
     hipStream_t s = as_stream(stream);
     switch (src->dtype) {
         case TANNIC_INT8: return run_scale<uint8_t>(src, sc, dst, s);
@@ -369,6 +378,10 @@ int tannic_hip_scale(const tannic_tensor_t* src, const tannic_scalar_t* sc, tann
 
 int tannic_hip_cpy(const tannic_tensor_t* src, tannic_tensor_t* dst, tannic_stream_t stream) {
     if (!src || !dst) return TANNIC_ERROR;
+    if (dtype_size(dst->dtype) != dtype_size(src->dtype)) {   // elements move as bits of the source's width
+        set_error_text("cpy: source and destination elements differ in size");
+        return TANNIC_ERROR;
+    }
     hipStream_t s = as_stream(stream);
     switch (dtype_size(src->dtype)) {
         case 1: return run_cpy<uint8_t>(src, dst, s);
@@ -396,6 +409,10 @@ int tannic_hip_le(const tannic_tensor_t* a, const tannic_tensor_t* b, tannic_ten
 
 int tannic_hip_allclose(const tannic_tensor_t* a, const tannic_tensor_t* b, tannic_stream_t stream, double rtol, double atol) {
     if (!a || !b) return -1;
+    if (a->dtype != b->dtype) {   // the second operand would be read as the first's type (src/cpu/val.cpp:73-83 does)
+        set_error_text("allclose: operands of different dtypes");
+        return -1;
+    }
     hipStream_t s = as_stream(stream);
     switch (a->dtype) {
         case TANNIC_FLOAT16: return run_allclose<f16>(a, b, s, rtol, atol);

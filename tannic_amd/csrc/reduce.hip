@@ -531,6 +531,12 @@ int reduce_entry(const tannic_tensor_t* src, tannic_tensor_t* dst, tannic_stream
         constexpr bool cplx = std::is_same_v<T, c64> || std::is_same_v<T, c128>;
         if constexpr (!cplx) {
             hipStream_t s = as_stream(stream);
+            // indices leave as int64, everything else in the source's type
+            const int out = (K == R_ARGMAX || K == R_ARGMIN) ? static_cast<int>(TANNIC_INT64) : dtype_code<T>();
+            if (!destination_is(dst, out, "reduction: the destination's dtype does not fit the result")) {
+                status = TANNIC_ERROR;
+                return;
+            }
             // coverage: src/cpu/argred.cpp:289-347 (mean: floating types only)
             if constexpr (K == R_SUM) status = run_reduce<SumOp<T, false>>(src, dst, s, axis);
             else if constexpr (K == R_MEAN) { if constexpr (!std::is_integral_v<T>) status = run_reduce<SumOp<T, true>>(src, dst, s, axis); }

@@ -53,6 +53,7 @@ int run_repeat(const tannic_tensor_t* src, tannic_tensor_t* dst, int axis, int r
         default: return TANNIC_UNSUPPORTED_DTYPE;
     }
     const int rank = src->rank;
+    if (!destination_is(dst, src->dtype, "repeat: the destination's dtype is not the source's")) return TANNIC_ERROR;
     if (rank < 1 || rank > 8 || dst->rank != rank || axis < 0 || axis >= rank || reps < 1) {
         set_error_text("repeat: rank, axis or count out of range");
         return TANNIC_ERROR;
@@ -219,6 +220,7 @@ int run_triangular(const tannic_tensor_t* src, tannic_tensor_t* dst, int k, hipS
         default: return TANNIC_UNSUPPORTED_DTYPE;
     }
     if (src->rank != 2) return TANNIC_UNSUPPORTED_DTYPE;   // src/cpu/triang.cpp:58
+    if (!destination_is(dst, src->dtype, "triu/tril: the destination's dtype is not the source's")) return TANNIC_ERROR;
     if (dst->rank != 2 || dst->shape.sizes[0] != src->shape.sizes[0] || dst->shape.sizes[1] != src->shape.sizes[1]) {
         set_error_text("triu/tril: destination shape does not match");
         return TANNIC_ERROR;

@@ -111,7 +111,10 @@ int unary(const tannic_tensor_t* src, tannic_tensor_t* dst, tannic_stream_t stre
         constexpr bool ok = (K == U_NEG || K == U_CPY) ? true
                           : K == U_ABS ? (flt || std::is_same_v<T, int32_t> || std::is_same_v<T, int64_t>)
                           : (flt && !cplx);
-        if constexpr (ok) status = run_unary<T, K>(src, dst, as_stream(stream), eps);
+        if constexpr (ok) {
+            if (!destination_is(dst, dtype_code<T>(), "unary op: the destination's dtype is not the source's")) status = TANNIC_ERROR;
+            else status = run_unary<T, K>(src, dst, as_stream(stream), eps);
+        }
     });
     return status;
 }

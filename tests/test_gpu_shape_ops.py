@@ -117,7 +117,7 @@ def test_concat_leading_axes_follow_numpy(device, axis):
     np.testing.assert_array_equal(got, np.concatenate([a, b], axis=axis))
 
 
-OUTER = [(ta.int8, ta.int64), (ta.int64, ta.int32), (ta.int64, ta.int64), (ta.float32, ta.float32), (ta.float32, ta.float64),
+OUTER = [(ta.int8, ta.int64), (ta.int64, ta.int32), (ta.int64, ta.int64), (ta.int8, ta.int32), (ta.int32, ta.int8), (ta.int16, ta.int32), (ta.int32, ta.int16), (ta.float32, ta.float32), (ta.float32, ta.float64),
          (ta.float64, ta.float64), (ta.int32, ta.float32), (ta.float64, ta.int32), (ta.float16, ta.float32), (ta.float32, ta.bfloat16)]
 
 

@@ -75,3 +75,61 @@ def test_reduction_destination_must_hold_one_element_per_slice(device, name):
     assert status == abi.SUCCESS
     status, _ = call(name, device, [src], zeros((4, 1, 8), dtype, device), (C.c_uint8(1),))   # kept dimension
     assert status == abi.SUCCESS
+
+
+# ---- dtypes that do not fit each other -----------------------------------------------------------------------------------
+# A kernel writes elements of one type: a destination described with another dtype would be over- or under-run, and a
+# second operand read as the first's type (what the reference's comparison and allclose do) would be read past its end.
+def test_destination_dtype_must_be_the_result_type(device):
+    f32, f16, i32 = (lambda s: zeros(s, ta.float32, device)), (lambda s: zeros(s, ta.float16, device)), (lambda s: zeros(s, ta.int32, device))
+    cases = [
+        ("exp", [f32((4, 8))], f16((4, 8)), ()),
+        ("neg", [i32((4, 8))], zeros((4, 8), ta.int64, device), ()),
+        ("add", [f32((4, 8)), f32((4, 8))], zeros((4, 8), ta.float64, device), ()),
+        ("mul", [i32((4, 8)), f32((4, 8))], i32((4, 8)), ()),
+        ("div", [f32((4, 8)), f32((4, 8))], f16((4, 8)), ()),
+        ("argsum", [f32((4, 8))], f16((4,)), (C.c_uint8(1),)),
+        ("argmax", [f32((4, 8))], zeros((4,), ta.int32, device), (C.c_uint8(1),)),
+        ("max", [f16((4, 8))], f32((4,)), (C.c_uint8(1),)),
+        ("gemm", [f16((8, 8)), f16((8, 8))], f32((8, 8)), ()),
+        ("gemm", [f32((8, 8)), f32((8, 8))], f16((8, 8)), ()),
+        ("conv2d", [f16((1, 2, 6, 6)), f16((3, 2, 3, 3))], f32((1, 3, 4, 4)), (abi.SIZE2(0, 0), abi.SIZE2(1, 1))),
+        ("repeat", [f32((4, 8))], f16((8, 8)), (C.c_int(0), C.c_int(2))),
+        ("triu", [f32((4, 8))], zeros((4, 8), ta.float64, device), (C.c_int(0),)),
+        ("gt", [f32((4, 8)), f32((4, 8))], zeros((4, 8), ta.int8, device), ()),
+        ("cpy", [f32((4, 8))], f16((4, 8)), ()),
+        ("view_as_polar", [f32((4, 8)), f32((4, 8))], zeros((4, 8), ta.complex128, device), ()),
+    ]
+    for name, sources, dst, extra in cases:
+        status, message = call(name, device, sources, dst, extra)
+        assert status == abi.ERROR and message, (name, status, message)
+
+
+def test_scale_destination_dtype(device):
+    lib = ta.library()
+    dvc = device.structure()
+    stream = lib.pop_stream(C.byref(dvc))
+    src, dst = zeros((4, 8), ta.float32, device).descriptor(), zeros((4, 8), ta.float16, device).descriptor()
+    value = C.c_float(2.0)
+    scalar = abi.scalar_t(C.cast(C.pointer(value), C.c_void_p), ta.float32.code)
+    status = lib.kernels["scale"](C.byref(src), C.byref(scalar), C.byref(dst), stream)
+    lib.put_stream(C.byref(dvc), stream)
+    assert status == abi.ERROR
+
+
+def test_comparison_and_allclose_want_one_dtype(device):
+    """The reference reads the second operand as the first's type (src/cpu/cmps.cpp:108-202, src/cpu/val.cpp:73-83): with
+    a narrower second operand that runs past its end, so the pair is refused."""
+    wide, narrow = zeros((64, 64), ta.int64, device), zeros((64, 64), ta.int8, device)
+    for name in ("eq", "ne", "gt", "ge", "lt", "le"):
+        status, message = call(name, device, [wide, narrow], zeros((64, 64), ta.boolean, device))
+        assert status == abi.UNSUPPORTED_DTYPE and "different dtypes" in message, name
+    lib = ta.library()
+    dvc = device.structure()
+    stream = lib.pop_stream(C.byref(dvc))
+    a, b = zeros((64, 64), ta.float64, device).descriptor(), zeros((64, 64), ta.float16, device).descriptor()
+    r = lib.kernels["allclose"](C.byref(a), C.byref(b), stream, 1e-5, 1e-8)
+    lib.put_stream(C.byref(dvc), stream)
+    assert r == -1
+    with pytest.raises(ta.TannicError):
+        ops.gt(wide, narrow)

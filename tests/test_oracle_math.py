@@ -261,3 +261,27 @@ def test_outer_is_numpy_outer_and_unsupported_pairs_say_so(oracle):
         # int8 x int8: the reference's kernel writes int32 into the int8 destination the front end made
         with pytest.raises(ops.TannicError):
             ops.outer(support.host_tensor(np.ones(3), ta.int8), support.host_tensor(np.ones(3), ta.int8))
+
+
+def test_pairs_whose_table_type_is_not_the_destinations_are_refused(oracle):
+    """The reference's tables write float for an integer with a 16-bit float (binary operations, matmul with int8 / int16)
+    while its front end sizes the destination as the 16-bit type: it overruns the destination.  The checker refuses
+    those pairs, like the device; so it does a comparison or allclose of two dtypes, whose second operand the
+    reference reads as the first's type."""
+    i8 = support.host_tensor(np.ones((2, 2)), ta.int8)
+    i64 = support.host_tensor(np.ones((2, 2)), ta.int64)
+    f16 = support.host_tensor(np.ones((2, 2)), ta.float16)
+    bf16 = support.host_tensor(np.ones((2, 2)), ta.bfloat16)
+    f64 = support.host_tensor(np.ones((2, 2)), ta.float64)
+    for op in (ops.add, ops.sub, ops.mul):
+        for a, b in ((i8, f16), (f16, i64), (bf16, i8), (i64, bf16)):
+            with pytest.raises(ta.TannicError):
+                op(a, b)
+    with pytest.raises(ta.TannicError):
+        ops.matmul(i8, f16)
+    for cmp in (ops.eq, ops.gt, ops.le):
+        with pytest.raises(ta.TannicError):
+            cmp(i64, i8)
+    with pytest.raises(ta.TannicError):
+        ops.allclose(f64, f16)
+    assert ops.allclose(f64, f64)

@@ -351,6 +351,7 @@ def test_concat_transposed_operands(oracle, reference):
 
 
 OUTER_PAIRS = [(ta.int8, ta.int64), (ta.int64, ta.int16), (ta.int32, ta.int64), (ta.int64, ta.int64),
+               (ta.int8, ta.int32), (ta.int32, ta.int8), (ta.int16, ta.int32), (ta.int32, ta.int16),
                (ta.float32, ta.float32), (ta.float32, ta.float64), (ta.float64, ta.float32), (ta.float64, ta.float64),
                (ta.int32, ta.float32), (ta.float32, ta.int32), (ta.int32, ta.float64), (ta.float64, ta.int32)]
 
