@@ -22,7 +22,10 @@
  *   - `address` already includes the view offset; strides are in ELEMENTS and
  *     may be 0 (expanded dims) or permuted; boolean tensors are bit-packed,
  *     LSB first, (size+7)/8 bytes; complex tensors are interleaved (re,im);
- *   - the destination is pre-allocated by the caller on the same device;
+ *   - the destination is pre-allocated by the caller on the same device, with
+ *     the shape and the dtype of the call's result: descriptors that do not
+ *     fit each other are refused with TANNIC_ERROR before anything is launched
+ *     (the reference's kernels take them on trust);
  *   - work is enqueued on `stream` and the call returns without waiting;
  *   - nothing is thrown across this boundary: the status says what happened
  *     and tannic_hip_last_error() holds a message for TANNIC_ERROR.
@@ -224,7 +227,9 @@ int tannic_hip_scale(const tannic_tensor_t* src, const tannic_scalar_t* scalar, 
 /* ------------------------------------------------------------------ *
  * Comparisons -> bit-packed boolean.  The reference has a CPU kernel only
  * (src/cpu/cmps.cpp:85-202) and throwing device stubs (src/comparisons.cpp:18-29);
- * these are the device twins of cpu::eq..le.
+ * these are the device twins of cpu::eq..le.  Both operands must have one
+ * dtype (UNSUPPORTED_DTYPE otherwise): cpu::eq..le read the second operand
+ * as the first's type, past the end of a narrower one.
  * ------------------------------------------------------------------ */
 int tannic_hip_eq(const tannic_tensor_t* a, const tannic_tensor_t* b, tannic_tensor_t* dst, tannic_stream_t stream);
 int tannic_hip_ne(const tannic_tensor_t* a, const tannic_tensor_t* b, tannic_tensor_t* dst, tannic_stream_t stream);
@@ -263,8 +268,8 @@ int tannic_hip_tril(const tannic_tensor_t* src, tannic_tensor_t* dst, tannic_str
  * ------------------------------------------------------------------ */
 /* cuda::cpy: strided -> strided, size-1 dims broadcast (CPU: src/cpu/cpy.cpp:18-80) */
 int tannic_hip_cpy(const tannic_tensor_t* src, tannic_tensor_t* dst, tannic_stream_t stream);
-/* cuda::allclose: 1 close, 0 not close, -1 unsupported dtype (the reference throws
- * there, src/cuda/val.cu:82-89); waits for the stream (CPU: src/cpu/val.cpp:17-83) */
+/* cuda::allclose: 1 close, 0 not close, -1 unsupported dtype or operands of two dtypes (the
+ * reference throws there, src/cuda/val.cu:82-89); waits for the stream (CPU: src/cpu/val.cpp:17-83) */
 int tannic_hip_allclose(const tannic_tensor_t* a, const tannic_tensor_t* b, tannic_stream_t stream, double rtol, double atol);
 
 /* ------------------------------------------------------------------ *
