@@ -489,7 +489,8 @@ int extreme_run(const tannic_tensor_t* src, tannic_tensor_t* dst, uint8_t ax) {
             }
             if (wins) { acc = v; beaten = true; }
         }
-        static_cast<T*>(dst->address)[slot] = beaten ? acc : ps[base];
+        /* an empty slice has no first element: it yields the start value */
+        static_cast<T*>(dst->address)[slot] = (beaten || R == 0) ? acc : ps[base];
     });
     return TANNIC_SUCCESS;
 }

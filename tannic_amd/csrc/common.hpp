@@ -182,7 +182,8 @@ inline size_t element_count(const tannic_tensor_t* t) {
 struct FastDiv {
     uint32_t d, magic, shift;
     FastDiv() : d(1), magic(1), shift(0) {}
-    explicit FastDiv(uint32_t divisor) : d(divisor) {
+    // (a divisor of 0 only comes from an empty index space, where nothing is ever divided: it is taken as 1)
+    explicit FastDiv(uint32_t divisor) : d(divisor ? divisor : 1) {
         for (shift = 0; shift < 32; ++shift)
             if ((1u << shift) >= d) break;
         const uint64_t one = 1;

@@ -169,7 +169,7 @@ __device__ inline Vec<T, N> load_vec(const T* p) {
 template <class Op>
 __device__ inline void emit(typename Op::A acc, uint32_t count, typename Op::Out* dst, size_t slot,
                             const typename Op::S* src, size_t first, size_t step) {
-    if constexpr (is_value_only<Op>::value) dst[slot] = same(acc, Op::init()) ? src[first] : acc;
+    if constexpr (is_value_only<Op>::value) dst[slot] = (count != 0 && same(acc, Op::init())) ? src[first] : acc;   // an empty slice yields the start value
     else if constexpr (Op::needs_source) dst[slot] = src[first + static_cast<size_t>(acc.index) * step];
     else dst[slot] = Op::finish(acc, count);
 }
@@ -392,7 +392,7 @@ __global__ __launch_bounds__(kThreads) void reduce_strided_kernel(const typename
     const int64_t step = w.stride[w.axis];
     typename Op::A acc = Op::init();
     for (uint32_t r = 0; r < R; ++r) acc = Op::step(acc, src[base + static_cast<int64_t>(r) * step], r);
-    if constexpr (is_value_only<Op>::value) dst[slot] = same(acc, Op::init()) ? src[base] : acc;
+    if constexpr (is_value_only<Op>::value) dst[slot] = (R != 0 && same(acc, Op::init())) ? src[base] : acc;
     else if constexpr (Op::needs_source) dst[slot] = src[base + static_cast<int64_t>(acc.index) * step];
     else dst[slot] = Op::finish(acc, R);
 }

@@ -133,3 +133,30 @@ def test_comparison_and_allclose_want_one_dtype(device):
     assert r == -1
     with pytest.raises(ta.TannicError):
         ops.gt(wide, narrow)
+
+
+# ---- nothing to do ------------------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("shape", [(0,), (3, 0), (0, 4), (2, 0, 5)])
+def test_empty_tensors_go_through_every_family(device, oracle, shape):
+    """A tensor without elements is a valid operand: the call succeeds, launches nothing and agrees with the CPU path
+    (an empty index space once divided by zero on the host while the launch was planned)."""
+    import support
+    for dtype in (ta.float32, ta.float16, ta.int32):
+        h, d = support.both(np.zeros(shape), dtype, device)
+        for op in (ops.neg, ops.repack, lambda t: ops.add(t, t), lambda t: ops.mul(t, t), lambda t: ops.scale(t, 2), lambda t: ops.gt(t, t)):
+            want, got = op(h), op(d)
+            assert got.shape == want.shape and got.dtype is want.dtype
+        for axis in range(len(shape)):
+            for name in ("sum", "argmax", "max", "min"):
+                want, got = getattr(ops, name)(h, axis), getattr(ops, name)(d, axis)
+                assert got.shape == want.shape
+                support.assert_bit_exact(got.storage(), want.storage(), f"{name} {dtype} {shape} axis={axis}")
+    # value max / min over an axis without elements: the start value of the fold
+    h, d = support.both(np.zeros((0, 4)), ta.float32, device)
+    assert np.isneginf(ops.max(d, 0).numpy()).all() and np.isposinf(ops.min(d, 0).numpy()).all()
+    for sa, sb in (((0, 4), (4, 3)), ((3, 4), (4, 0)), ((3, 0), (0, 5))):
+        ha, da = support.both(np.ones(sa), ta.float16, device)
+        hb, db = support.both(np.ones(sb), ta.float16, device)
+        want, got = ops.matmul(ha, hb), ops.matmul(da, db)
+        assert got.shape == want.shape
+        support.assert_bit_exact(got.storage(), want.storage(), f"matmul {sa} x {sb}")
