@@ -204,3 +204,24 @@ def test_reductions_full_size(device, oracle, dtype):
     np.testing.assert_array_equal(ops.max(dx, 0).numpy(), x[0])
     np.testing.assert_array_equal(ops.argmax(dx, 0).numpy(), np.zeros(SHAPE[1:], dtype=np.int64))
     support.assert_close(ops.sum(dx, 0).numpy(), x[0].astype(np.float64) * SHAPE[0], *sum_tol, "sum axis 0 against float64")
+
+
+def test_byte_offsets_beyond_4_gib(device):
+    """Tensors of 4.4 GB (element counts under 2^31, byte offsets over 2^32): elementwise, broadcast, both reduction
+    directions, argmax and a transposing copy index them with 64-bit offsets."""
+    n = 1_100_000_000
+    x = (np.arange(n, dtype=np.int64) % 1000).astype(np.float32)
+    dx = ta.tensor(x, ta.float32, device)
+    got = ops.add(dx, dx).numpy()
+    assert (got[-1_000_000:] == 2 * x[-1_000_000:]).all() and (got[::4097] == 2 * x[::4097]).all()
+    del got
+    cube = dx.view(1100, 1000, 1000)
+    got = ops.mul(cube, ta.tensor(np.full((1, 1000, 1), 3.0), ta.float32, device)).numpy().reshape(-1)
+    assert (got[-1_000_000:] == 3 * x[-1_000_000:]).all() and (got[::4099] == 3 * x[::4099]).all()
+    del got
+    blocks = x.reshape(1100, 1000, 1000)
+    np.testing.assert_allclose(ops.sum(cube, 2).numpy(), blocks.sum(axis=2, dtype=np.float64), rtol=1e-6)
+    np.testing.assert_allclose(ops.sum(cube, 0).numpy(), blocks.sum(axis=0, dtype=np.float64), rtol=1e-6)
+    assert (ops.argmax(cube, 1).numpy() == blocks.argmax(axis=1)).all()
+    turned = ops.repack(cube.transpose(0, 2)).numpy()
+    assert (turned[:, :, -3:] == blocks.transpose(2, 1, 0)[:, :, -3:]).all() and (turned[::7, ::11] == blocks.transpose(2, 1, 0)[::7, ::11]).all()
