@@ -500,14 +500,10 @@ int extreme_run(const tannic_tensor_t* src, tannic_tensor_t* dst, uint8_t ax) {
  *                                         :87-123 (transposition, batch offsets),
  *                                         :126-176 (launcher)
  * ------------------------------------------------------------------ */
-bool is_transposed(const tannic_tensor_t* t) { /* :87-94 */
-    if (t->rank < 2) return false;
-    return t->strides.sizes[t->rank - 1] > t->strides.sizes[t->rank - 2];
-}
 
 template <class S0, class S1, class D>
-void gemm_kernel(bool at, bool bt, const S0* A, const S1* B, D* C, size_t M, size_t N, size_t K,
-                 size_t lda, size_t ldb, size_t ldc) {
+void gemm_kernel(const S0* A, const S1* B, D* C, size_t M, size_t N, size_t K,
+                 int64_t a_rs, int64_t a_cs, int64_t b_rs, int64_t b_cs, size_t ldc) {
     constexpr bool sixteen = is16<D>;
     for (size_t i = 0; i < M; ++i)
         for (size_t j = 0; j < N; ++j) {
@@ -515,15 +511,16 @@ void gemm_kernel(bool at, bool bt, const S0* A, const S1* B, D* C, size_t M, siz
                 if (g_wide) {
                     float acc = 0.0f;
                     for (size_t k = 0; k < K; ++k)
-                        acc += static_cast<float>(A[at ? k * lda + i : i * lda + k]) *
-                               static_cast<float>(B[bt ? j * ldb + k : k * ldb + j]);
+                        acc += static_cast<float>(A[static_cast<int64_t>(i) * a_rs + static_cast<int64_t>(k) * a_cs]) *
+                               static_cast<float>(B[static_cast<int64_t>(k) * b_rs + static_cast<int64_t>(j) * b_cs]);
                     C[i * ldc + j] = static_cast<D>(acc);
                     continue;
                 }
             }
             D sum = D(0);
             for (size_t k = 0; k < K; ++k)
-                sum += static_cast<D>(A[at ? k * lda + i : i * lda + k]) * static_cast<D>(B[bt ? j * ldb + k : k * ldb + j]);
+                sum += static_cast<D>(A[static_cast<int64_t>(i) * a_rs + static_cast<int64_t>(k) * a_cs]) *
+                       static_cast<D>(B[static_cast<int64_t>(k) * b_rs + static_cast<int64_t>(j) * b_cs]);
             C[i * ldc + j] = sum;
         }
 }
@@ -532,16 +529,19 @@ template <class S0, class S1, class D>
 int gemm_run(const tannic_tensor_t* a, const tannic_tensor_t* b, tannic_tensor_t* c) {
     const size_t M = c->shape.sizes[c->rank - 2], N = c->shape.sizes[c->rank - 1];
     const size_t K = a->shape.sizes[a->rank - 1];
-    const bool at = is_transposed(a), bt = is_transposed(b);
-    /* leading dimensions are narrowed to int in the reference (:135-137) */
-    const int lda = static_cast<int>(at ? a->strides.sizes[a->rank - 1] : a->strides.sizes[a->rank - 2]);
-    const int ldb = static_cast<int>(bt ? b->strides.sizes[b->rank - 1] : b->strides.sizes[b->rank - 2]);
+    /* The reference takes the larger of an operand's two matrix strides as its leading dimension and the other one to
+     * be 1 (:87-94, :135-137).  Whenever the other one IS 1 (a slab or its transpose: everything its tests hold) that
+     * is the element a view means; here, as on the device, both strides are always used, so a view whose inner
+     * stride is not 1 (one half of an interleaved tensor, an expanded column) multiplies the elements it shows.
+     * Leading dimensions are narrowed to int in the reference (:135-137). */
+    const int64_t a_rs = static_cast<int>(a->strides.sizes[a->rank - 2]), a_cs = static_cast<int>(a->strides.sizes[a->rank - 1]);
+    const int64_t b_rs = static_cast<int>(b->strides.sizes[b->rank - 2]), b_cs = static_cast<int>(b->strides.sizes[b->rank - 1]);
     const int ldc = static_cast<int>(c->strides.sizes[c->rank - 2]);
     const S0* A = static_cast<const S0*>(a->address);
     const S1* B = static_cast<const S1*>(b->address);
     D* C = static_cast<D*>(c->address);
     if (c->rank <= 2) {
-        gemm_kernel<S0, S1, D>(at, bt, A, B, C, M, N, K, lda, ldb, ldc);
+        gemm_kernel<S0, S1, D>(A, B, C, M, N, K, a_rs, a_cs, b_rs, b_cs, ldc);
         return TANNIC_SUCCESS;
     }
     const int batch_rank = c->rank - 2;
@@ -566,7 +566,7 @@ int gemm_run(const tannic_tensor_t* a, const tannic_tensor_t* b, tannic_tensor_t
             if (d < b->rank) ob += coord(b) * b->strides.sizes[d];
             oc += idx[d] * c->strides.sizes[d];
         }
-        gemm_kernel<S0, S1, D>(at, bt, A + oa, B + ob, C + oc, M, N, K, lda, ldb, ldc);
+        gemm_kernel<S0, S1, D>(A + oa, B + ob, C + oc, M, N, K, a_rs, a_cs, b_rs, b_cs, ldc);
     }
     return TANNIC_SUCCESS;
 }

@@ -10,15 +10,12 @@
 //     path accumulates in the 16-bit type);
 //   - fp32 sums are formed in a different order (tiles of K);
 //   - batch counts above 255 are handled (the CPU path narrows the batch
-//     counter to uint8_t, src/cpu/matmul.cpp:102).
+//     counter to uint8_t, src/cpu/matmul.cpp:102);
+//   - an operand is addressed by both of its matrix strides (the CPU path
+//     takes the smaller one to be 1, src/cpu/matmul.cpp:87-94).
 #include "gemm_common.hpp"
 
 namespace th {
-
-static bool is_transposed(const tannic_tensor_t* t) {
-    if (t->rank < 2) return false;
-    return t->strides.sizes[t->rank - 1] > t->strides.sizes[t->rank - 2];
-}
 
 int describe_gemm(const tannic_tensor_t* a, const tannic_tensor_t* b, const tannic_tensor_t* c, GemmProblem& p) {
     if (a->rank < 2 || b->rank < 2 || c->rank < 2 || c->rank > 8) {
@@ -33,15 +30,13 @@ int describe_gemm(const tannic_tensor_t* a, const tannic_tensor_t* b, const tann
     p.M = static_cast<uint32_t>(M);
     p.N = static_cast<uint32_t>(N);
     p.K = static_cast<uint32_t>(K);
-    // a transposed view is recognised by its strides; its leading dimension is
-    // the larger stride and the other one is taken to be 1
-    const bool at = is_transposed(a), bt = is_transposed(b);
-    const int64_t lda = at ? a->strides.sizes[a->rank - 1] : a->strides.sizes[a->rank - 2];
-    const int64_t ldb = bt ? b->strides.sizes[b->rank - 1] : b->strides.sizes[b->rank - 2];
-    p.a_rs = at ? 1 : lda;
-    p.a_cs = at ? lda : 1;
-    p.b_rs = bt ? 1 : ldb;
-    p.b_cs = bt ? ldb : 1;
+    // Both matrix strides of an operand are used as they are.  (The CPU path takes the larger one as the leading
+    // dimension and the other one to be 1, src/cpu/matmul.cpp:87-94,135-137: the same thing for a slab or its
+    // transpose, and the wrong elements for a view whose inner stride is not 1.)
+    p.a_rs = a->strides.sizes[a->rank - 2];
+    p.a_cs = a->strides.sizes[a->rank - 1];
+    p.b_rs = b->strides.sizes[b->rank - 2];
+    p.b_cs = b->strides.sizes[b->rank - 1];
     p.c_rs = c->strides.sizes[c->rank - 2];
     p.row_bias = nullptr;
     p.batch_rank = c->rank - 2;

@@ -121,3 +121,29 @@ def test_fp32_matmul_512_seed0(device):
     support.assert_close(got, want, 1e-5, 512 * 2.0 ** -24, "fp32 512^3")
     exact = a.astype(np.float64) @ b.astype(np.float64)
     assert np.abs(got - exact).max() <= np.abs(want - exact).max() * 1.5 + 1e-6  # no worse than the sequential sum
+
+
+@pytest.mark.parametrize("dtype", [ta.float16, ta.float32, ta.int32, ta.float64], ids=str)
+def test_operands_whose_inner_stride_is_not_one(device, oracle, dtype):
+    """Views with both matrix strides different from 1 (every other column, one half of an interleaved tensor, an
+    expanded column) multiply the elements they show: checked against numpy on small integers, where every type is
+    exact.  (The reference's CPU path takes the smaller stride to be 1, src/cpu/matmul.cpp:87-94.)"""
+    rng = np.random.default_rng(5)
+    a = rng.integers(-3, 4, (40, 70)).astype(np.float64)
+    b = rng.integers(-3, 4, (70, 50)).astype(np.float64)
+    ha, da = support.both(a, dtype, device)
+    hb, db = support.both(b, dtype, device)
+    index_a, index_b = (slice(3, 35, 2), slice(1, 61, 2)), (slice(10, 40), slice(2, 50, 3))
+    want = a[index_a] @ b[index_b]
+    for x, y in ((da, db), (ha, hb)):
+        np.testing.assert_array_equal(ops.matmul(x[index_a], y[index_b]).numpy().astype(np.float64), want)
+    pairs = rng.integers(-3, 4, (16, 24, 2)).astype(np.float64)          # [M, K, 2]: the "real parts" are a stride-2 view
+    hp, dp = support.both(pairs, dtype, device)
+    w = rng.integers(-3, 4, (24, 8)).astype(np.float64)
+    hw, dw = support.both(w, dtype, device)
+    for x, y in ((dp, dw), (hp, hw)):
+        np.testing.assert_array_equal(ops.matmul(x[:, :, 0], y).numpy().astype(np.float64), pairs[:, :, 0] @ w)
+    column = rng.integers(-3, 4, (16, 1)).astype(np.float64)
+    hc, dc = support.both(column, dtype, device)
+    for x, y in ((dc, dw), (hc, hw)):
+        np.testing.assert_array_equal(ops.matmul(x.expand(16, 24), y).numpy().astype(np.float64), np.broadcast_to(column, (16, 24)) @ w)
