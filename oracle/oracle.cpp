@@ -597,7 +597,9 @@ int conv2d_run(const tannic_tensor_t* x, const tannic_tensor_t* w, const tannic_
       for (size_t co = 0; co < Co; ++co)
         for (size_t oh = 0; oh < Ho; ++oh)
           for (size_t ow = 0; ow < Wo; ++ow) {
-            T acc = pb ? pb[co] : T(0);      /* :37 / :90: bias seeds the accumulator */
+            /* :37 / :90: bias seeds the accumulator.  The reference reads b[co]; here, as on the device, the bias is read
+             * through its stride, so that a column of a matrix is a valid bias */
+            T acc = pb ? pb[static_cast<int64_t>(co) * bias->strides.sizes[0]] : T(0);
             Acc wacc = static_cast<Acc>(acc);
             const int64_t bh = static_cast<int64_t>(oh * stride[0]) - static_cast<int64_t>(pad[0]);
             const int64_t bw = static_cast<int64_t>(ow * stride[1]) - static_cast<int64_t>(pad[1]);
@@ -800,7 +802,8 @@ template <class T> int concat_run(const tannic_tensor_t* a, const tannic_tensor_
 
 /* ------------------------------------------------------------------ *
  * outer product of two vectors             src/cpu/outer.cpp:18-110
- * dst[i][j] = a[i] * b[j] with C++'s own conversions of the pair, stored in the table's type D; contiguous vectors
+ * dst[i][j] = a[i] * b[j] with C++'s own conversions of the pair, stored in the table's type D.  The reference reads
+ * both vectors as contiguous; here, as on the device, through their strides (every other element of a vector is a vector)
  * ------------------------------------------------------------------ */
 template <class A, class B, class D> int outer_run(const tannic_tensor_t* a, const tannic_tensor_t* b, tannic_tensor_t* dst) {
     const A* pa = static_cast<const A*>(a->address);
@@ -808,7 +811,7 @@ template <class A, class B, class D> int outer_run(const tannic_tensor_t* a, con
     D* pd = static_cast<D*>(dst->address);
     const size_t n1 = a->shape.sizes[0], n2 = b->shape.sizes[0];
     for (size_t i = 0; i < n1; ++i)
-        for (size_t j = 0; j < n2; ++j) pd[i * n2 + j] = static_cast<D>(pa[i] * pb[j]);
+        for (size_t j = 0; j < n2; ++j) pd[i * n2 + j] = static_cast<D>(pa[static_cast<int64_t>(i) * a->strides.sizes[0]] * pb[static_cast<int64_t>(j) * b->strides.sizes[0]]);
     return TANNIC_SUCCESS;
 }
 

@@ -20,7 +20,7 @@ __global__ __launch_bounds__(256) void conv2d_direct_kernel(const T* x, const T*
     const uint32_t oh = rem % p.HO; rem /= p.HO;
     const uint32_t co = rem % p.O;
     const uint32_t n = rem / p.O;
-    Acc acc = p.has_bias ? static_cast<Acc>(widen(bias[co])) : Acc(0);
+    Acc acc = p.has_bias ? static_cast<Acc>(widen(bias[static_cast<int64_t>(co) * p.bs])) : Acc(0);
     const int64_t bh = static_cast<int64_t>(oh) * p.stride_h - p.pad_h;
     const int64_t bw = static_cast<int64_t>(ow) * p.stride_w - p.pad_w;
     for (uint32_t ci = 0; ci < p.C; ++ci)
@@ -91,7 +91,8 @@ static int conv2d_entry(const tannic_tensor_t* x, const tannic_tensor_t* w, cons
         p.ys[d] = y->strides.sizes[d];
     }
     p.has_bias = bias != nullptr;
-    // the bias is read as b[co]: element stride 1 (src/cpu/conv2d.cpp:90)
+    // the bias is read through its stride (a column of a matrix is a valid bias; the CPU path reads b[co], src/cpu/conv2d.cpp:86)
+    p.bs = bias ? bias->strides.sizes[0] : 0;
     const void* pb = bias ? bias->address : nullptr;
     hipStream_t s = as_stream(stream);
     // Kernels in order of preference.  A 1x1 kernel has no tap to amortise a staged patch over: its weights stay in

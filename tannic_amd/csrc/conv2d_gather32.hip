@@ -162,7 +162,7 @@ __global__ __launch_bounds__(kG32Threads) void conv2d_gather32_kernel(const floa
 #pragma unroll
         for (int v = 0; v < 16; ++v) {
             const uint32_t co = co0 + wco + i * 32 + 8 * (v / 4) + 4 * (lane / 32) + v % 4;
-            const float b = (p.has_bias && co < p.O) ? bias[co] : 0.0f;
+            const float b = (p.has_bias && co < p.O) ? bias[static_cast<int64_t>(co) * p.bs] : 0.0f;
 #pragma unroll
             for (int j = 0; j < TN; ++j) acc[i][j][v] = b;
         }

@@ -164,7 +164,7 @@ __global__ __launch_bounds__(kK1Threads) void conv2d_k1_kernel(const T* x, const
         const T* row = w + static_cast<int64_t>(co) * p.ws[0] + 8 * (lane / 32);
 #pragma unroll
         for (int ks = 0; ks < KSTEPS; ++ks) afrag[i][ks] = *reinterpret_cast<const uint4p*>(row + ks * 16);
-        start[i] = bias ? static_cast<float>(widen(bias[co])) : 0.0f;
+        start[i] = bias ? static_cast<float>(widen(bias[static_cast<int64_t>(co) * p.bs])) : 0.0f;
     }
 
     k1_static_for<4>([&](auto m_) { commit_pair(Zero{}, m_, lds); });

@@ -187,7 +187,7 @@ __global__ __launch_bounds__(kK3Threads, ONE_STAGE ? 2 : 1) void conv2d_k3_kerne
 #pragma unroll
     for (int i = 0; i < TM; ++i) {
         const uint32_t co = co0 + i * 32 + lane % 32;
-        bias_v[i] = (p.has_bias && co < p.O) ? static_cast<float>(widen(bias[co])) : 0.0f;
+        bias_v[i] = (p.has_bias && co < p.O) ? static_cast<float>(widen(bias[static_cast<int64_t>(co) * p.bs])) : 0.0f;
     }
 #pragma unroll
     for (int k = 0; k < kK3Taps; ++k) commit_w(k, lds);

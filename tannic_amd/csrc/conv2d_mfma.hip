@@ -195,7 +195,7 @@ __global__ __launch_bounds__(kConvThreads) void conv2d_mfma16_kernel(const T* x,
 #pragma unroll
         for (int v = 0; v < 16; ++v) {
             const uint32_t co = co0 + wco + i * 32 + 8 * (v / 4) + 4 * (lane / 32) + v % 4;
-            const float b = (p.has_bias && co < p.O) ? static_cast<float>(widen(bias[co])) : 0.0f;
+            const float b = (p.has_bias && co < p.O) ? static_cast<float>(widen(bias[static_cast<int64_t>(co) * p.bs])) : 0.0f;
 #pragma unroll
             for (int j = 0; j < TN; ++j) acc[i][j][v] = b;
         }

@@ -109,7 +109,7 @@ __global__ __launch_bounds__(kPatchThreads, 2) void conv2d_patch_kernel(const T*
 #pragma unroll
         for (int v = 0; v < 16; ++v) {
             const uint32_t co = co0 + i * 32 + 8 * (v / 4) + 4 * (lane / 32) + v % 4;
-            const float bv = (p.has_bias && co < p.O) ? static_cast<float>(widen(bias[co])) : 0.0f;
+            const float bv = (p.has_bias && co < p.O) ? static_cast<float>(widen(bias[static_cast<int64_t>(co) * p.bs])) : 0.0f;
             acc[i][0][v] = bv;
             acc[i][1][v] = bv;
         }

@@ -51,6 +51,7 @@ int product(const GemmProblem& g, int dtype, const void* a, const void* b, void*
 template <class T>
 int run_pointwise(const ConvProblem& p, int dtype, const void* x, const void* w, const void* bias, void* y, hipStream_t stream) {
     if (p.KH != 1 || p.KW != 1 || p.pad_h != 0 || p.pad_w != 0) return TANNIC_UNSUPPORTED_DTYPE;
+    if (p.has_bias && p.bs != 1 && p.O > 1) return TANNIC_UNSUPPORTED_DTYPE;   // the product reads its row bias as a dense vector
     if (p.N == 0 || p.O == 0 || p.HO == 0 || p.WO == 0) return TANNIC_SUCCESS;
     if (p.C == 0) return TANNIC_UNSUPPORTED_DTYPE;
     // the kernel tensor as a K-contiguous O x C matrix; the result as row-major O x (HO*WO) per image

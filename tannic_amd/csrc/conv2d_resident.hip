@@ -121,7 +121,7 @@ __global__ __launch_bounds__(kResThreads) void conv2d_resident_kernel(const T* x
 #pragma unroll
         for (int v = 0; v < 16; ++v) {
             const uint32_t co = co0 + wco + i * 32 + 8 * (v / 4) + 4 * (lane / 32) + v % 4;
-            bias_v[i][v] = (p.has_bias && co < p.O) ? static_cast<float>(widen(bias[co])) : 0.0f;
+            bias_v[i][v] = (p.has_bias && co < p.O) ? static_cast<float>(widen(bias[static_cast<int64_t>(co) * p.bs])) : 0.0f;
         }
 
     // ---- patch staging: global -> registers (fetch), registers -> LDS (commit) ------------------

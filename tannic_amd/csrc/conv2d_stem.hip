@@ -135,7 +135,7 @@ __global__ __launch_bounds__(kStemThreads, 2) void conv2d_stem_kernel(const T* x
 #pragma unroll
         for (int i = 0; i < 2; ++i) {
             const uint32_t co = co0 + i * 32 + lane % 32;
-            bias_v[i] = (p.has_bias && co < p.O) ? static_cast<float>(widen(bias[co])) : 0.0f;
+            bias_v[i] = (p.has_bias && co < p.O) ? static_cast<float>(widen(bias[static_cast<int64_t>(co) * p.bs])) : 0.0f;
         }
 #pragma unroll
         for (int j = 0; j < kStemWeightPieces; ++j) {

@@ -57,6 +57,7 @@ __global__ __launch_bounds__(256) void conv_pad_weights_kernel(const float* w, f
 
 int conv2d_unfold(const ConvProblem& p, int dtype, const void* x, const void* w, const void* bias, void* y, hipStream_t stream) {
     if (dtype != TANNIC_FLOAT32) return TANNIC_UNSUPPORTED_DTYPE;
+    if (p.has_bias && p.bs != 1 && p.O > 1) return TANNIC_UNSUPPORTED_DTYPE;   // the product reads its row bias as a dense vector
     if (p.N == 0 || p.O == 0 || p.HO == 0 || p.WO == 0) return TANNIC_SUCCESS;
     const uint64_t K64 = static_cast<uint64_t>(p.C) * p.KH * p.KW, P64 = static_cast<uint64_t>(p.HO) * p.WO;
     // the product's conditions, checked before anything is queued: whole 16-byte groups of pixels, dense result rows

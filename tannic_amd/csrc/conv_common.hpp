@@ -13,6 +13,7 @@ struct ConvProblem {
     uint32_t HO, WO;           // output spatial size
     uint32_t pad_h, pad_w, stride_h, stride_w;
     int64_t xs[4], ws[4], ys[4];
+    int64_t bs;                // element stride of the bias (the CPU path reads it as 1, src/cpu/conv2d.cpp:86)
     bool has_bias;
 };
 

@@ -182,3 +182,26 @@ def test_conv1d(device, dtype, name):
     else:
         eps = 2.0 ** -24 if dtype is ta.float32 else 2.0 ** -53
         support.assert_close(got.numpy(), want.numpy(), 1e-5 if dtype is ta.float32 else 1e-13, fan_in * eps * 4, f"conv1d {dtype} {name}")
+
+
+@pytest.mark.parametrize("dtype", [ta.float32, ta.float16, ta.int32], ids=str)
+@pytest.mark.parametrize("kernel", [1, 3], ids=lambda k: f"k{k}")
+def test_bias_and_kernel_seen_through_views(device, oracle, dtype, kernel):
+    """A column of a matrix is a valid bias and every other output channel of a kernel tensor a valid kernel: both are
+    read through their strides by every kernel path (the reference reads the bias as b[co], src/cpu/conv2d.cpp:86).
+    Small integers, so every type is exact and numpy decides."""
+    rng = np.random.default_rng(17)
+    x = rng.integers(-2, 3, (2, 8, 10, 16)).astype(np.float64)
+    w = rng.integers(-2, 3, (12, 8, kernel, kernel)).astype(np.float64)
+    table = rng.integers(-2, 3, (6, 5)).astype(np.float64)
+    pad = kernel // 2
+    padded = np.pad(x, ((0, 0), (0, 0), (pad, pad), (pad, pad)))
+    want = np.zeros((2, 6, 10, 16))
+    for kh in range(kernel):
+        for kw in range(kernel):
+            want += np.einsum("nchw,oc->nohw", padded[:, :, kh:kh + 10, kw:kw + 16], w[::2, :, kh, kw])
+    want += table[:, 3].reshape(1, 6, 1, 1)
+    for make in (lambda a: support.both(a, dtype, device)[1], lambda a: support.host_tensor(a, dtype)):
+        tx, tw, tb = make(x), make(w), make(table)
+        got = ops.convolve2d(tx, tw[::2], tb[:, 3], 1, pad).numpy().astype(np.float64)
+        np.testing.assert_array_equal(got, want)

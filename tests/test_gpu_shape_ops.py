@@ -134,3 +134,14 @@ def test_outer_pairs_that_overrun_their_destination_are_refused(device):
     a = ta.tensor(np.ones(4), ta.float16, device)
     with pytest.raises(ops.TannicError):
         ops.outer(a, a)     # the table says fp32, the destination is fp16
+
+
+def test_outer_of_strided_vectors(device, oracle):
+    """Every other element of a vector is a vector: both operands are read through their strides (the reference reads
+    them as contiguous, src/cpu/outer.cpp:18-40)."""
+    a, b = np.arange(40, dtype=np.float64) - 20, np.arange(30, dtype=np.float64) - 7
+    for dtype in (ta.float32, ta.float64, ta.int64):
+        want = np.outer(a[::2], b[1::3])
+        (ha, da), (hb, db) = support.both(a, dtype, device), support.both(b, dtype, device)
+        np.testing.assert_array_equal(ops.outer(da[::2], db[1::3]).numpy().astype(np.float64), want)
+        np.testing.assert_array_equal(ops.outer(ha[::2], hb[1::3]).numpy().astype(np.float64), want)
