@@ -344,3 +344,33 @@ def test_random_moves_and_the_rest(device, oracle):
             want, got = ops.polar(h1, h2).numpy(), ops.polar(d1, d2).numpy()
             tol = 1e-12 if kind_of_float is ta.float64 else 2e-6
             assert got.shape == want.shape and (np.abs(got - want) <= tol * (np.abs(want) + 1)).all(), what
+
+
+def test_random_matrix_products_of_sliced_views(device):
+    """Operands cut out of larger matrices with offsets and steps (so that neither matrix stride need be 1), one of them
+    possibly transposed: small integers, every type is exact and numpy decides."""
+    rng = np.random.default_rng(105)
+
+    def cut(n):
+        first = int(rng.integers(0, max(1, n // 3)))
+        last = int(rng.integers(first + 1, n + 1))
+        return slice(first, last, int(rng.choice([1, 1, 1, 2])))
+
+    for done in range(150):
+        dtype = [ta.float16, ta.bfloat16, ta.float32, ta.int32, ta.float64][int(rng.integers(0, 5))]
+        m, k, n = (int(rng.choice([1, 7, 16, 33, 64, 100, 130, 257])) for _ in range(3))
+        a = rng.integers(-3, 4, (m + 5, k + 9)).astype(np.float64)
+        b = rng.integers(-3, 4, (k + 9, n + 6)).astype(np.float64)
+        index_a = (cut(m + 5), cut(k + 9))
+        depth = a[index_a].shape[1]
+        start = int(rng.integers(0, k + 9 - depth + 1))
+        index_b = (slice(start, start + depth), cut(n + 6))
+        turned = bool(rng.random() < 0.3)
+        what = f"{done}: {dtype} A{a.shape}{index_a} B{b.shape}{index_b} A stored transposed: {turned}"
+        print(what, flush=True)
+        da = ta.tensor(a.T.copy() if turned else a, dtype, device)
+        db = ta.tensor(b, dtype, device)
+        va = da[(index_a[1], index_a[0])].transpose(0, 1) if turned else da[index_a]
+        got = ops.matmul(va, db[index_b]).numpy().astype(np.float64)
+        want = a[index_a] @ b[index_b]
+        assert got.shape == want.shape and (got == want).all(), what
