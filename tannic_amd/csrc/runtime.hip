@@ -278,6 +278,8 @@ void* tannic_hip_deallocate(const tannic_device_t* device, void* address) {
 
 int tannic_hip_copy_from_host(const tannic_device_t* device, const void* host, void* dev, size_t nbytes) {
     if (!device) return TANNIC_NULL_ALLOCATOR;
+    if (nbytes == 0) return TANNIC_SUCCESS;
+    if (!host || !dev) { set_error_text("copy_from_host: null address"); return TANNIC_ERROR; }
     TH_TRY(hipSetDevice(device->id));
     Streams& streams = Streams::instance();
     hipStream_t stream = streams.pop(device->id);
@@ -292,6 +294,8 @@ int tannic_hip_copy_from_host(const tannic_device_t* device, const void* host, v
 
 int tannic_hip_copy_device_to_host(const tannic_device_t* device, const void* dev, void* host, size_t nbytes) {
     if (!device) return TANNIC_NULL_ALLOCATOR;
+    if (nbytes == 0) return TANNIC_SUCCESS;
+    if (!host || !dev) { set_error_text("copy_device_to_host: null address"); return TANNIC_ERROR; }
     TH_TRY(hipSetDevice(device->id));
     Streams& streams = Streams::instance();
     hipStream_t stream = streams.pop(device->id);
@@ -303,7 +307,7 @@ int tannic_hip_copy_device_to_host(const tannic_device_t* device, const void* de
 }
 
 int tannic_hip_compare_from_host(const tannic_device_t* device, const void* host, const void* dev, size_t nbytes) {
-    if (!device) return -1;
+    if (!device || (nbytes && (!host || !dev))) return -1;
     void* buffer = std::malloc(nbytes ? nbytes : 1);
     if (!buffer) return -1;
     int rc = tannic_hip_copy_device_to_host(device, dev, buffer, nbytes);
@@ -313,6 +317,12 @@ int tannic_hip_compare_from_host(const tannic_device_t* device, const void* host
 }
 
 int tannic_hip_copy(const tannic_tensor_t* src, tannic_tensor_t* dst, size_t nbytes, tannic_stream_t s) {
+    if (!src || !dst) return TANNIC_ERROR;
+    if (nbytes == 0) return TANNIC_SUCCESS;
+    if (!src->address || !dst->address) {
+        set_error_text("copy: a tensor without storage");
+        return TANNIC_ERROR;
+    }
     hipStream_t stream = as_stream(s);
     const bool src_dev = src->environment.kind == TANNIC_DEVICE;
     const bool dst_dev = dst->environment.kind == TANNIC_DEVICE;
@@ -325,6 +335,8 @@ int tannic_hip_copy(const tannic_tensor_t* src, tannic_tensor_t* dst, size_t nby
         if (dst->environment.resource.host.traits != TANNIC_PINNED) TH_TRY(hipStreamSynchronize(stream));
     } else if (src_dev && dst_dev) {
         TH_TRY(hipMemcpyAsync(dst->address, src->address, nbytes, hipMemcpyDeviceToDevice, stream));
+    } else {
+        std::memmove(dst->address, src->address, nbytes);   // host to host: the front end never asks, a caller of the C ABI may
     }
     return TANNIC_SUCCESS;
 }

@@ -152,3 +152,24 @@ def test_temporaries_reusing_blocks_keep_results_right(device, oracle):
         want = ops.add(ops.mul(want, hx), ops.neg(want)) if step % 2 else ops.sub(ops.abs(want), hx)
         got, want = ops.tanh(got), ops.tanh(want)
     support.assert_close(got.numpy(), want.numpy(), 1e-5, 1e-6, "forty operators over reused blocks")
+
+
+def test_copies_with_nothing_to_copy_or_nowhere_to_go(device):
+    """Zero bytes succeed without touching the addresses; a null address with bytes to move is an error, not a crash."""
+    lib = ta.library()
+    dvc = device.structure()
+    assert lib.copy_from_host(C.byref(dvc), None, None, 0) == abi.SUCCESS
+    assert lib.copy_device_to_host(C.byref(dvc), None, None, 0) == abi.SUCCESS
+    assert lib.compare_from_host(C.byref(dvc), None, None, 0) == 1
+    ptr = lib.allocate(C.byref(dvc), 0)          # an empty tensor still owns an address
+    assert ptr
+    buf = (C.c_char * 16)()
+    assert lib.copy_from_host(C.byref(dvc), None, ptr, 16) == abi.ERROR
+    assert lib.copy_device_to_host(C.byref(dvc), ptr, None, 16) == abi.ERROR
+    assert lib.compare_from_host(C.byref(dvc), None, ptr, 16) == -1
+    assert lib.copy_from_host(C.byref(dvc), buf, ptr, 16) == abi.SUCCESS
+    lib.deallocate(C.byref(dvc), ptr)
+    assert lib.deallocate(C.byref(dvc), None) is None
+    assert lib.allocate(None, 64) is None
+    empty = ta.Tensor(ta.float32, (0, 4)).initialize(device)
+    assert empty.numpy().shape == (0, 4) and empty.to(ta.Host()).numpy().shape == (0, 4)
