@@ -24,8 +24,9 @@
  *     LSB first, (size+7)/8 bytes; complex tensors are interleaved (re,im);
  *   - the destination is pre-allocated by the caller on the same device, with
  *     the shape and the dtype of the call's result: descriptors that do not
- *     fit each other are refused with TANNIC_ERROR before anything is launched
- *     (the reference's kernels take them on trust);
+ *     fit each other, or that have elements but a null address, are refused
+ *     with TANNIC_ERROR before anything is launched (the reference's kernels
+ *     take them on trust);
  *   - work is enqueued on `stream` and the call returns without waiting;
  *   - nothing is thrown across this boundary: the status says what happened
  *     and tannic_hip_last_error() holds a message for TANNIC_ERROR.

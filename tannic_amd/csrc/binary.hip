@@ -116,6 +116,7 @@ int run_binary(const tannic_tensor_t* a, const tannic_tensor_t* b, tannic_tensor
 template <int K>
 int binary(const tannic_tensor_t* a, const tannic_tensor_t* b, tannic_tensor_t* dst, tannic_stream_t stream) {
     if (!a || !b || !dst) return TANNIC_ERROR;
+    if (!have_storage(a, b, dst)) return TANNIC_ERROR;
     int status = TANNIC_UNSUPPORTED_DTYPE;
     with_type(a->dtype, [&](auto ta) {
         with_type(b->dtype, [&](auto tb) {

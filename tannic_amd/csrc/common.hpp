@@ -177,6 +177,13 @@ inline size_t element_count(const tannic_tensor_t* t) {
     return n;
 }
 
+// Every given tensor either has storage or no elements (a kernel handed a null address faults the device).
+template <class... Ts> inline bool have_storage(const Ts*... t) {
+    const bool ok = ((t == nullptr || t->address != nullptr || element_count(t) == 0) && ...);
+    if (!ok) set_error_text("a tensor with elements has no storage (null address)");
+    return ok;
+}
+
 // ---- 32-bit division by a launch-time constant ------------------------------
 // q = n / d for n < 2^31 with one multiply-high, one add and one shift.
 struct FastDiv {

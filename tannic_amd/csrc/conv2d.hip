@@ -54,6 +54,7 @@ int run_direct(const ConvProblem& p, const void* x, const void* w, const void* b
 static int conv2d_entry(const tannic_tensor_t* x, const tannic_tensor_t* w, const tannic_tensor_t* bias, tannic_tensor_t* y,
                         tannic_stream_t stream, const size_t pad[2], const size_t stride[2]) {
     if (!x || !w || !y || !pad || !stride) return TANNIC_ERROR;
+    if (!have_storage(x, w, bias, y)) return TANNIC_ERROR;
     // dispatch on (signal, kernel) dtype first: unsupported pairs report
     // UNSUPPORTED_DTYPE before any shape check, as the table lookup does
     if (x->dtype != w->dtype) return TANNIC_UNSUPPORTED_DTYPE;
@@ -133,6 +134,7 @@ static int conv2d_entry(const tannic_tensor_t* x, const tannic_tensor_t* w, cons
 // [O,C,1,K], same loops in the same order (channel, tap), same status rules with rank 3 in place of 4.
 static int conv1d_entry(const tannic_tensor_t* x, const tannic_tensor_t* w, tannic_tensor_t* y, tannic_stream_t stream, size_t pad, size_t stride) {
     if (!x || !w || !y) return TANNIC_ERROR;
+    if (!have_storage(x, w, y)) return TANNIC_ERROR;
     if (x->dtype != w->dtype) return TANNIC_UNSUPPORTED_DTYPE;
     switch (x->dtype) {
         case TANNIC_INT8: case TANNIC_INT16: case TANNIC_INT32: case TANNIC_INT64:

@@ -173,6 +173,7 @@ extern "C" {
 #if !defined(TH_EXTENDED_ONLY) || TH_EXTENDED_ONLY == 0
 int tannic_hip_div(const tannic_tensor_t* a, const tannic_tensor_t* b, tannic_tensor_t* dst, tannic_stream_t stream) {
     if (!a || !b || !dst) return TANNIC_ERROR;
+    if (!have_storage(a, b, dst)) return TANNIC_ERROR;
     int status = TANNIC_UNSUPPORTED_DTYPE;
     with_real_type(a->dtype, [&](auto ta) {
         with_real_type(b->dtype, [&](auto tb) {
@@ -192,6 +193,7 @@ int tannic_hip_div(const tannic_tensor_t* a, const tannic_tensor_t* b, tannic_te
 
 int tannic_hip_swiglu(const tannic_tensor_t* gate, const tannic_tensor_t* up, tannic_tensor_t* dst, tannic_stream_t stream) {
     if (!gate || !up || !dst) return TANNIC_ERROR;
+    if (!have_storage(gate, up, dst)) return TANNIC_ERROR;
     if (gate->dtype != up->dtype || gate->dtype != dst->dtype) return TANNIC_UNSUPPORTED_DTYPE;
     int status = TANNIC_UNSUPPORTED_DTYPE;
     with_real_type(gate->dtype, [&](auto t) {
@@ -205,6 +207,7 @@ int tannic_hip_swiglu(const tannic_tensor_t* gate, const tannic_tensor_t* up, ta
 #if !defined(TH_EXTENDED_ONLY) || TH_EXTENDED_ONLY == 1
 int tannic_hip_cast(const tannic_tensor_t* src, tannic_tensor_t* dst, tannic_stream_t stream) {
     if (!src || !dst) return TANNIC_ERROR;
+    if (!have_storage(src, dst)) return TANNIC_ERROR;
     int status = TANNIC_UNSUPPORTED_DTYPE;
     with_real_type(src->dtype, [&](auto ta) {
         with_real_type(dst->dtype, [&](auto tb) {

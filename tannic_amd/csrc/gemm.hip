@@ -165,6 +165,7 @@ using namespace th;
 
 extern "C" int tannic_hip_gemm(const tannic_tensor_t* a, const tannic_tensor_t* b, tannic_tensor_t* dst, tannic_stream_t stream) {
     if (!a || !b || !dst) return TANNIC_ERROR;
+    if (!have_storage(a, b, dst)) return TANNIC_ERROR;
     int status = TANNIC_UNSUPPORTED_DTYPE;
     hipStream_t s = as_stream(stream);
     with_type(a->dtype, [&](auto ta) {

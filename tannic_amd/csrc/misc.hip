@@ -148,6 +148,7 @@ int run_complex(const tannic_tensor_t* a, const tannic_tensor_t* b, tannic_tenso
 template <bool POLAR>
 int complex_entry(const tannic_tensor_t* a, const tannic_tensor_t* b, tannic_tensor_t* dst, tannic_stream_t stream) {
     if (!a || !b || !dst) return TANNIC_ERROR;
+    if (!have_storage(a, b, dst)) return TANNIC_ERROR;
     int status = TANNIC_UNSUPPORTED_DTYPE;
     with_type(a->dtype, [&](auto ta) {
         with_type(b->dtype, [&](auto tb) {
@@ -276,6 +277,7 @@ int run_compare(const tannic_tensor_t* a, const tannic_tensor_t* b, tannic_tenso
 template <int K>
 int compare_entry(const tannic_tensor_t* a, const tannic_tensor_t* b, tannic_tensor_t* dst, tannic_stream_t stream) {
     if (!a || !b || !dst) return TANNIC_ERROR;
+    if (!have_storage(a, b, dst)) return TANNIC_ERROR;
     int status = TANNIC_UNSUPPORTED_DTYPE;
     // The CPU path dispatches on the first source only and reads the second as the same type (src/cpu/cmps.cpp:108-202),
     // which runs past the end of a narrower second operand: operands of different dtypes are refused here.
@@ -360,6 +362,7 @@ extern "C" {
 
 int tannic_hip_scale(const tannic_tensor_t* src, const tannic_scalar_t* sc, tannic_tensor_t* dst, tannic_stream_t stream) {
     if (!src || !sc || !dst || !sc->address) return TANNIC_ERROR;
+    if (!have_storage(src, dst)) return TANNIC_ERROR;
     if (src->dtype != sc->dtype) return TANNIC_UNSUPPORTED_DTYPE;
     if (!destination_is(dst, src->dtype, "scale: the destination's dtype is not the source's")) return TANNIC_ERROR;
     hipStream_t s = as_stream(stream);
@@ -378,6 +381,7 @@ int tannic_hip_scale(const tannic_tensor_t* src, const tannic_scalar_t* sc, tann
 
 int tannic_hip_cpy(const tannic_tensor_t* src, tannic_tensor_t* dst, tannic_stream_t stream) {
     if (!src || !dst) return TANNIC_ERROR;
+    if (!have_storage(src, dst)) return TANNIC_ERROR;
     if (dtype_size(dst->dtype) != dtype_size(src->dtype)) {   // elements move as bits of the source's width
         set_error_text("cpy: source and destination elements differ in size");
         return TANNIC_ERROR;
@@ -408,7 +412,7 @@ int tannic_hip_lt(const tannic_tensor_t* a, const tannic_tensor_t* b, tannic_ten
 int tannic_hip_le(const tannic_tensor_t* a, const tannic_tensor_t* b, tannic_tensor_t* d, tannic_stream_t s) { return compare_entry<C_LE>(a, b, d, s); }
 
 int tannic_hip_allclose(const tannic_tensor_t* a, const tannic_tensor_t* b, tannic_stream_t stream, double rtol, double atol) {
-    if (!a || !b) return -1;
+    if (!a || !b || !have_storage(a, b)) return -1;
     if (a->dtype != b->dtype) {   // the second operand would be read as the first's type (src/cpu/val.cpp:73-83 does)
         set_error_text("allclose: operands of different dtypes");
         return -1;

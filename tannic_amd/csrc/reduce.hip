@@ -525,6 +525,7 @@ enum ReduceKind { R_SUM, R_MEAN, R_ARGMAX, R_ARGMIN, R_MAX, R_MIN };
 template <int K>
 int reduce_entry(const tannic_tensor_t* src, tannic_tensor_t* dst, tannic_stream_t stream, uint8_t axis) {
     if (!src || !dst) return TANNIC_ERROR;
+    if (!have_storage(src, dst)) return TANNIC_ERROR;
     int status = TANNIC_UNSUPPORTED_DTYPE;
     with_type(src->dtype, [&](auto t) {
         using T = typename decltype(t)::type;

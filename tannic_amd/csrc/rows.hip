@@ -420,6 +420,7 @@ extern "C" {
 
 int tannic_hip_rms_norm(const tannic_tensor_t* x, const tannic_tensor_t* gain, tannic_tensor_t* dst, tannic_stream_t stream, float eps) {
     if (!x || !gain || !dst) return TANNIC_ERROR;
+    if (!have_storage(x, gain, dst)) return TANNIC_ERROR;
     if (x->dtype != gain->dtype || x->dtype != dst->dtype) return TANNIC_UNSUPPORTED_DTYPE;
     if (x->rank < 1 || !same_shape(x, dst) || !is_contiguous(x) || !is_contiguous(dst) || !is_contiguous(gain) ||
         element_count(gain) != x->shape.sizes[x->rank - 1]) {
@@ -434,6 +435,7 @@ int tannic_hip_rms_norm(const tannic_tensor_t* x, const tannic_tensor_t* gain, t
 
 int tannic_hip_softmax(const tannic_tensor_t* x, const tannic_tensor_t* mask, tannic_tensor_t* dst, tannic_stream_t stream, float scale) {
     if (!x || !dst) return TANNIC_ERROR;
+    if (!have_storage(x, mask, dst)) return TANNIC_ERROR;
     if (x->dtype != dst->dtype || (mask && mask->dtype != x->dtype)) return TANNIC_UNSUPPORTED_DTYPE;
     if (x->rank < 1 || !same_shape(x, dst) || !is_contiguous(x) || !is_contiguous(dst)) {
         set_error_text("softmax: x and dst must be contiguous with one shape");
@@ -455,6 +457,7 @@ int tannic_hip_softmax(const tannic_tensor_t* x, const tannic_tensor_t* mask, ta
 
 int tannic_hip_rope(const tannic_tensor_t* x, const tannic_tensor_t* cos, const tannic_tensor_t* sin, tannic_tensor_t* dst, tannic_stream_t stream) {
     if (!x || !cos || !sin || !dst) return TANNIC_ERROR;
+    if (!have_storage(x, cos, sin, dst)) return TANNIC_ERROR;
     if (x->dtype != dst->dtype || cos->dtype != x->dtype || sin->dtype != x->dtype) return TANNIC_UNSUPPORTED_DTYPE;
     bool ok = x->rank >= 2 && same_shape(x, dst) && is_contiguous(dst) && is_contiguous(cos) && is_contiguous(sin) && same_shape(cos, sin) && cos->rank == 2;
     if (ok) {

@@ -246,14 +246,17 @@ int run_triangular(const tannic_tensor_t* src, tannic_tensor_t* dst, int k, hipS
 extern "C" {
 int tannic_hip_repeat(const tannic_tensor_t* src, tannic_tensor_t* dst, tannic_stream_t stream, int axis, int reps) {
     if (!src || !dst) return TANNIC_ERROR;
+    if (!th::have_storage(src, dst)) return TANNIC_ERROR;
     return th::run_repeat(src, dst, axis, reps, th::as_stream(stream));
 }
 int tannic_hip_concat(const tannic_tensor_t* a, const tannic_tensor_t* b, tannic_tensor_t* dst, tannic_stream_t stream, int axis) {
     if (!a || !b || !dst) return TANNIC_ERROR;
+    if (!th::have_storage(a, b, dst)) return TANNIC_ERROR;
     return th::run_concat(a, b, dst, axis, th::as_stream(stream));
 }
 int tannic_hip_outer(const tannic_tensor_t* a, const tannic_tensor_t* b, tannic_tensor_t* dst, tannic_stream_t stream) {
     if (!a || !b || !dst) return TANNIC_ERROR;
+    if (!th::have_storage(a, b, dst)) return TANNIC_ERROR;
     const int result = th::outer_table(a->dtype, b->dtype);
     const int sized_as = a->dtype > b->dtype ? a->dtype : b->dtype;
     if (result < 0 || result != sized_as || dst->dtype != result) return TANNIC_UNSUPPORTED_DTYPE;
@@ -274,10 +277,12 @@ int tannic_hip_outer(const tannic_tensor_t* a, const tannic_tensor_t* b, tannic_
 }
 int tannic_hip_triu(const tannic_tensor_t* src, tannic_tensor_t* dst, tannic_stream_t stream, int k) {
     if (!src || !dst) return TANNIC_ERROR;
+    if (!th::have_storage(src, dst)) return TANNIC_ERROR;
     return th::run_triangular<true>(src, dst, k, th::as_stream(stream));
 }
 int tannic_hip_tril(const tannic_tensor_t* src, tannic_tensor_t* dst, tannic_stream_t stream, int k) {
     if (!src || !dst) return TANNIC_ERROR;
+    if (!th::have_storage(src, dst)) return TANNIC_ERROR;
     return th::run_triangular<false>(src, dst, k, th::as_stream(stream));
 }
 }

@@ -102,6 +102,7 @@ int run_unary(const tannic_tensor_t* src, tannic_tensor_t* dst, hipStream_t stre
 template <int K>
 int unary(const tannic_tensor_t* src, tannic_tensor_t* dst, tannic_stream_t stream, double eps = 0.0) {
     if (!src || !dst) return TANNIC_ERROR;
+    if (!have_storage(src, dst)) return TANNIC_ERROR;
     int status = TANNIC_UNSUPPORTED_DTYPE;
     with_type(src->dtype, [&](auto t) {
         using T = typename decltype(t)::type;

@@ -160,3 +160,24 @@ def test_empty_tensors_go_through_every_family(device, oracle, shape):
         want, got = ops.matmul(ha, hb), ops.matmul(da, db)
         assert got.shape == want.shape
         support.assert_bit_exact(got.storage(), want.storage(), f"matmul {sa} x {sb}")
+
+
+def test_a_tensor_without_storage_is_refused(device):
+    """A descriptor with elements and a null address is turned away at the entry (a kernel reading it would fault the
+    device); one without elements needs no storage."""
+    good = zeros((4, 8), ta.float32, device)
+    for name, n_sources, extra in (("exp", 1, ()), ("add", 2, ()), ("gt", 2, ()), ("argsum", 1, (C.c_uint8(1),)), ("gemm", 2, ()), ("cpy", 1, ()), ("div", 2, ())):
+        lib = ta.library()
+        dvc = device.structure()
+        stream = lib.pop_stream(C.byref(dvc))
+        sources = [zeros((8, 8) if name == "gemm" else (4, 8), ta.float32, device) for _ in range(n_sources)]
+        shape = {"gt": (4, 8), "argsum": (4,), "gemm": (8, 8)}.get(name, (4, 8))
+        dst = zeros(shape, ta.boolean if name == "gt" else ta.float32, device)
+        descs = [s.descriptor() for s in sources]
+        out = dst.descriptor()
+        descs[0].address = None
+        status = lib.kernels[name](*[C.byref(d) for d in descs], C.byref(out), stream, *extra)
+        message = lib.error_message()
+        lib.put_stream(C.byref(dvc), stream)
+        assert status == abi.ERROR and "no storage" in message, (name, status, message)
+    del good
