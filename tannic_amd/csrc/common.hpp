@@ -177,8 +177,13 @@ inline size_t element_count(const tannic_tensor_t* t) {
     return n;
 }
 
-// Every given tensor either has storage or no elements (a kernel handed a null address faults the device).
+// Every given tensor has at most TANNIC_DIMENSIONS dims and either storage or no elements (a kernel handed a null
+// address faults the device; a rank beyond the descriptor's arrays would be read past them).
 template <class... Ts> inline bool have_storage(const Ts*... t) {
+    if (!((t == nullptr || t->rank <= TANNIC_DIMENSIONS) && ...)) {
+        set_error_text("a tensor's rank is beyond what a descriptor holds");
+        return false;
+    }
     const bool ok = ((t == nullptr || t->address != nullptr || element_count(t) == 0) && ...);
     if (!ok) set_error_text("a tensor with elements has no storage (null address)");
     return ok;
