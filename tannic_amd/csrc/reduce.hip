@@ -228,9 +228,6 @@ __global__ __launch_bounds__(kThreads) void reduce_rows_kernel(const typename Op
 // the -inf / +inf start kept when nothing beats it), then the lowest index holding it.  Same answers as
 // the strict comparison from the start value: ties go to the lowest index, NaN never wins, and a row in
 // which nothing beats the start gives 0 (src/cpu/argred.cpp:95-101, :317-347).
-struct MinIndexOp {
-    __device__ static inline uint32_t combine(uint32_t x, uint32_t y) { return x < y ? x : y; }
-};
 template <bool MAX> struct ExtremeOp {
     __device__ static inline float combine(float x, float y) { return MAX ? fmaxf(x, y) : fminf(x, y); }
 };
@@ -259,28 +256,40 @@ __global__ __launch_bounds__(kThreads) void arg_rows16_kernel(const T* src, int6
     }
 #pragma unroll
     for (int r = 0; r < kArgRows; ++r) {
-        float f[NCH][8];
+        float f[NCH][8], piece_best[NCH];
         float best = start;
 #pragma unroll
         for (int i = 0; i < NCH; ++i) {
-            const bool present = lane + i * kWave < chunks;
+            float m = start;
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
-                f[i][e] = present ? widen(raw[r][i].v[e]) : __builtin_nanf("");   // an absent piece equals nothing
-                best = ExtremeOp<MAX>::combine(best, f[i][e]);
+                f[i][e] = widen(raw[r][i].v[e]);
+                m = ExtremeOp<MAX>::combine(m, f[i][e]);
             }
+            piece_best[i] = lane + i * kWave < chunks ? m : __builtin_nanf("");   // an absent piece equals nothing
+            best = ExtremeOp<MAX>::combine(best, piece_best[i]);
         }
         best = wave_reduce<ExtremeOp<MAX>>(best);
-        // the lane's first position holding the extreme, walking backwards so that the lowest one stays
-        uint32_t pos = 0xFFu;
+        // Nothing beat the start (all NaN, or only the start value itself): the strict comparison never moved off 0.
+        // Otherwise the lowest index holding the extreme is in the first piece (pieces are 64 lanes apart) that any
+        // lane found it in, in the lowest such lane: a ballot names both, and only that piece is searched.
+        uint32_t index = 0;
+        if (best != start) {
+            bool found = false;
 #pragma unroll
-        for (int i = NCH - 1; i >= 0; --i)
+            for (int i = 0; i < NCH; ++i) {
+                const uint64_t holders = __ballot(piece_best[i] == best);
+                if (!found && holders != 0) {
+                    found = true;
+                    const int holder = __builtin_ctzll(holders);
+                    int pos = 7;
 #pragma unroll
-            for (int e = 7; e >= 0; --e) pos = f[i][e] == best ? static_cast<uint32_t>(i * 8 + e) : pos;
-        uint32_t index = pos == 0xFFu ? 0xFFFFFFFFu : ((pos / 8) * kWave + lane) * 8 + pos % 8;
-        index = wave_reduce<MinIndexOp>(index);
-        // nothing beat the start (all NaN, or only the start value itself): the strict comparison never moved off 0
-        if (lane == 0 && row0 + r < rows) dst[row0 + r] = (best == start || index == 0xFFFFFFFFu) ? 0 : static_cast<int64_t>(index);
+                    for (int e = 6; e >= 0; --e) pos = f[i][e] == best ? e : pos;
+                    index = (static_cast<uint32_t>(i) * kWave + holder) * 8 + __builtin_amdgcn_readlane(pos, holder);
+                }
+            }
+        }
+        if (lane == 0 && row0 + r < rows) dst[row0 + r] = static_cast<int64_t>(index);
     }
 }
 

@@ -111,6 +111,38 @@ def test_argmax_with_nan_and_infinities(device):
     support.assert_bit_exact(ops.argmax(di, 1).storage(), ops.argmax(hi, 1).storage(), "int8 all lowest")
 
 
+@pytest.mark.parametrize("extent", [8, 64, 504, 512, 520, 1024, 1032, 1536, 2048])
+@pytest.mark.parametrize("dtype", [ta.float16, ta.bfloat16], ids=str)
+def test_index_of_extreme_in_many_short_rows_of_16_bit_floats(device, dtype, extent):
+    """Thousands of rows of at most 2048 16-bit floats (whole 16-byte pieces) are searched by a kernel of their own:
+    ties, NaNs, infinities, signed zeros and rows in which nothing beats the start value, at every piece count."""
+    rows = 1027
+    x = np.round(support.values_for(dtype, SEED, 40 + extent, (rows, extent), -4, 4).astype(np.float64))
+    rng = np.random.default_rng(extent)
+    x[0, :] = np.nan                                   # nothing but NaN: index 0
+    x[1, :] = -np.inf                                  # argmax never leaves 0; argmin ties everywhere
+    x[2, :] = np.inf
+    x[3, :] = np.nan; x[3, extent - 1] = -7.0          # the only number is the last element
+    x[4, :] = 0.0; x[4, ::3] = -0.0                    # zeros of both signs tie
+    x[5, :] = 1.0; x[5, extent // 2] = np.nan          # the same value everywhere: lowest index
+    x[6, :] = -2.0; x[6, extent - 1] = 9.0; x[6, extent // 2] = 9.0   # two holders in different lanes or pieces
+    x[7, :] = np.nan; x[7, extent - 3:] = [-np.inf, np.inf, -np.inf][:3]
+    for row in range(8, 200):                          # one or two planted extremes at random places
+        where = rng.integers(0, extent, 2)
+        x[row, where] = 50.0
+        x[row, rng.integers(0, extent, 2)] = -50.0
+        if row % 5 == 0:
+            x[row, rng.integers(0, extent, max(1, extent // 7))] = np.nan
+    h, d = support.both(x, dtype, device)
+    for op in ("argmax", "argmin"):
+        want, got = getattr(ops, op)(h, 1), getattr(ops, op)(d, 1)
+        assert got.dtype is ta.int64 and got.shape == want.shape
+        support.assert_bit_exact(got.storage(), want.storage(), f"{op} {dtype} [{rows},{extent}]")
+    clean = ~np.isnan(x).any(axis=1)                   # and against numpy where its answer is defined the same way
+    np.testing.assert_array_equal(ops.argmax(d, 1).numpy()[clean & (x.max(axis=1) > -np.inf)],
+                                  x.argmax(axis=1)[clean & (x.max(axis=1) > -np.inf)])
+
+
 @pytest.mark.parametrize("dtype", [ta.float32, ta.float64, ta.float16, ta.bfloat16], ids=str)
 def test_value_max_min_order_signed_zeros_and_skip_nan(device, dtype):
     """max / min are the largest / smallest NUMBER of a slice with +0 above -0, whichever lane, wavefront or block
