@@ -118,18 +118,21 @@ class Bench:
         return self.lib.event_elapsed_ms(self.e0, self.e1) / iters
 
 
-def gemm_entry(b, dtype, M, N, K, iters):
+def gemm_entry(b, dtype, M, N, K, iters, layout="NT"):
+    """layout: how the operands lie in memory. "NT": X[M,K] . W[N,K]^T (a linear layer); "NN": X[M,K] . W[K,N];
+    "TN": X[K,M]^T . W[K,N]."""
     ta = b.ta
-    x = b.filled(dtype, (M, K), "normal", 0, 1, 1.0)
-    w = b.filled(dtype, (N, K), "normal", 0, 2, 0.02)
+    x = b.filled(dtype, (K, M) if layout[0] == "T" else (M, K), "normal", 0, 1, 1.0)
+    w = b.filled(dtype, (N, K) if layout[1] == "T" else (K, N), "normal", 0, 2, 0.02)
     y = ta.Tensor(dtype, (M, N)).initialize(b.device)
-    ms = b.event_time(b.raw_call("gemm", [x, w.transpose()], y), iters)
+    ms = b.event_time(b.raw_call("gemm", [x.transpose() if layout[0] == "T" else x, w.transpose() if layout[1] == "T" else w], y), iters)
     flops = 2.0 * M * N * K
     nbytes = (M * K + N * K + M * N) * dtype.itemsize
     tflops, gbs = flops / ms / 1e9, nbytes / ms / 1e6
     peak = MFMA_PEAK_TFLOPS["f32" if dtype is ta.float32 else "f16"]
     hbm_bound = flops / nbytes < peak * 1e3 / HBM_PEAK_GBS   # below the ridge of the matrix peak over 8 TB/s
-    return {"op": f"gemm {dtype} X[{M},{K}].W[{N},{K}]^T", "us": round(ms * 1e3, 2), "tflops": round(tflops, 2), "gbs": round(gbs, 1),
+    name = {"NT": f"X[{M},{K}].W[{N},{K}]^T", "NN": f"X[{M},{K}].W[{K},{N}]", "TN": f"X[{K},{M}]^T.W[{K},{N}]"}[layout]
+    return {"op": f"gemm {dtype} {name}", "us": round(ms * 1e3, 2), "tflops": round(tflops, 2), "gbs": round(gbs, 1),
             "bound": "hbm" if hbm_bound else "mfma",
             "frac": round(gbs / HBM_PEAK_GBS if hbm_bound else tflops / peak, 4)}
 
@@ -316,6 +319,8 @@ def secondary(b, only):
     if only in (None, "gemm"):
         for (m, n) in [(2048, 4096), (2048, 14336), (128, 4096), (128, 14336), (16, 4096), (16, 14336), (1, 4096), (1, 14336)]:
             work.append(gemm_entry(b, ta.float16, m, n, 4096, 20))
+        work.append(gemm_entry(b, ta.float16, 4096, 4096, 4096, 20, "NN"))
+        work.append(gemm_entry(b, ta.float16, 4096, 4096, 4096, 20, "TN"))
         work.append(gemm_entry(b, ta.bfloat16, 4096, 4096, 4096, 20))
         work.append(gemm_entry(b, ta.float32, 512, 512, 512, 20))
         work.append(gemm_entry(b, ta.float32, 4096, 4096, 4096, 5))

@@ -12,8 +12,8 @@
 //   two MFMAs; one barrier per step, placed where the fragments of the next 16
 //   MFMAs are in registers already.  An operand that is contiguous along K is copied chunk by chunk;
 //   an operand that is contiguous along its row index (a transposed view of A,
-//   a plain row-major B) is read as 8x8 micro-blocks and transposed in
-//   registers on its way to LDS.
+//   a plain row-major B) goes to LDS as it lies in memory, [k][row], and is
+//   transposed on the way out by ds_read_b64_tr_b16, two per fragment.
 //
 // fp32 operands: v_mfma_f32_32x32x2f32 (true fp32), the same kernel with K steps
 //   of 32 (rows of a tile stay 128 bytes): a 16-byte fragment feeds four MFMAs,
@@ -141,7 +141,7 @@ struct KMajorLoader {
     static constexpr int index_of(int o) { return o / 2; }
 };
 
-// ---- operand contiguous along its row index: E x E micro-blocks (E elements per 16 bytes), transposed --------
+// ---- fp32 operand contiguous along its row index: E x E micro-blocks (E elements per 16 bytes), transposed ----
 template <class T, int ROWS, int THREADS>
 struct RowMajorLoader {
     static constexpr int E = kChunkOf<T>;
@@ -190,8 +190,55 @@ struct RowMajorLoader {
     static constexpr int index_of(int o) { return (o / (2 * E)) * E + o % E; }
 };
 
+// ---- 16-bit operand contiguous along its row index: the tile goes to LDS as it lies in memory -----------------
+// [k][row] with a pitch of ROWS + 32 elements.  The transposition happens on the way out: gfx950's
+// ds_read_b64_tr_b16 hands lane i of a group of 16 lanes, whose lanes 4e+q point at four elements each, element i % 4
+// of the four pointers with q = i / 4 - that is, pointed at k-row e and rows 4q..4q+3, it returns to lane i four
+// consecutive k of row i.  Two such reads make the 8 k of a lane's MFMA fragment.  The 64 bytes added to the pitch put
+// the four k-rows that 32 lanes read together on different banks.
+template <class T, int ROWS, int THREADS>
+struct AsIsLoader {
+    static constexpr int PITCH = ROWS + 32;
+    static constexpr int CHUNKS = ROWS / 8;                    // 16-byte chunks per k-row
+    static constexpr int LOADS = kBKof<T> * CHUNKS / THREADS, STORES = LOADS;
+    static_assert(kBKof<T> * CHUNKS % THREADS == 0, "whole passes");
+    uint4v regs[LOADS];
+    uint32_t k0_, K_;
+    __device__ inline void begin_fetch(const Operand&, uint32_t k0, uint32_t K) { k0_ = k0; K_ = K; }
+    __device__ inline void fetch_one(int i, const Operand& op, uint32_t row0) {
+        const uint32_t id = threadIdx.x + THREADS * i, k = k0_ + id / CHUNKS, row = row0 + (id % CHUNKS) * 8;
+        regs[i] = *reinterpret_cast<const uint4v*>(static_cast<const T*>(op.base) + static_cast<int64_t>(k < K_ ? k : 0) * op.k_stride + (row < op.rows ? row : 0));
+    }
+    template <bool MASK>
+    __device__ inline void commit_one(int i, T* tile) const {
+        const uint32_t id = threadIdx.x + THREADS * i, k = id / CHUNKS;
+        *reinterpret_cast<uint4v*>(tile + k * PITCH + (id % CHUNKS) * 8) = (!MASK || k0_ + k < K_) ? regs[i] : uint4v{0, 0, 0, 0};
+    }
+    static constexpr int OPS = STORES + LOADS;
+    static constexpr bool is_commit(int o) { return o % 2 == 0; }
+    static constexpr int index_of(int o) { return o / 2; }
+};
+
+typedef short short4v __attribute__((ext_vector_type(4)));
+// the lane's fragment of k-slice ks for the 32 rows starting at row0; lane_offset: see the kernel
+template <class T, int PITCH> __device__ inline uint4v read_transposed(const T* tile, uint32_t row0, int ks, uint32_t lane_offset) {
+    using Lds = __attribute__((address_space(3))) short4v;
+    const T* at = tile + lane_offset + static_cast<uint32_t>(ks) * 16 * PITCH + row0;
+    const short4v lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((Lds*)at);
+    const short4v hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((Lds*)(at + 4 * PITCH));
+    uint4v out;
+    __builtin_memcpy(&out, &lo, 8);
+    __builtin_memcpy(reinterpret_cast<char*>(&out) + 8, &hi, 8);
+    return out;
+}
+
+template <class T, bool K_MAJOR> constexpr bool kAsIs = !K_MAJOR && sizeof(T) == 2;
+// elements of LDS that one buffer of an operand's tile takes
+template <class T, int ROWS, bool K_MAJOR> constexpr uint32_t kTileElements = kAsIs<T, K_MAJOR> ? kBKof<T> * (ROWS + 32) : ROWS * kBKof<T>;
+
 template <class T, int ROWS, int THREADS, bool K_MAJOR>
-using Loader = std::conditional_t<K_MAJOR, KMajorLoader<T, ROWS, THREADS>, RowMajorLoader<T, ROWS, THREADS>>;
+using Loader = std::conditional_t<K_MAJOR, KMajorLoader<T, ROWS, THREADS>,
+                                  std::conditional_t<sizeof(T) == 2, AsIsLoader<T, ROWS, THREADS>, RowMajorLoader<T, ROWS, THREADS>>>;
 
 // WAVES_N: wavefronts along N (2 -> 256 threads, one wavefront per SIMD; 4 -> 512 threads, two per SIMD, so that
 // one wavefront's waits are covered by the other's MFMAs); always two wavefronts along M.
@@ -212,7 +259,7 @@ __global__ __launch_bounds__(128 * WAVES_N) void gemm16_kernel(const T* A, const
     // layout: A buffer 0, A buffer 1, B buffer 0, B buffer 1 (offsets in elements)
     T* lds = reinterpret_cast<T*>(lds_raw);
     constexpr int kBK = kBKof<T>;   // K elements per step
-    constexpr uint32_t A_TILE = BM * kBK, B_TILE = BN * kBK, B_BASE = 2 * A_TILE;
+    constexpr uint32_t A_TILE = kTileElements<T, BM, A_KMAJOR>, B_TILE = kTileElements<T, BN, B_KMAJOR>, B_BASE = 2 * A_TILE;
 
     uint32_t tm, tn;
     const uint32_t tile_id = SPLIT ? blockIdx.x / sk.splits : blockIdx.x, split = SPLIT ? blockIdx.x % sk.splits : 0;
@@ -229,6 +276,8 @@ __global__ __launch_bounds__(128 * WAVES_N) void gemm16_kernel(const T* A, const
     const int wave = threadIdx.x / 64, lane = threadIdx.x % 64;
     const int wm = (wave / WAVES_N) * WM, wn = (wave % WAVES_N) * WN;
     const uint32_t frag_row = lane % 32, frag_chunk = lane / 32;
+    // transposing reads: lane 16b + 4e + q points at k-row 8 * (b / 2) + e, rows 16 * (b % 2) + 4q .. + 3 of the fragment
+    const uint32_t tr_k = 8 * (lane / 32) + (lane % 16) / 4, tr_row = 16 * ((lane / 16) % 2) + 4 * (lane % 4);
 
     // an accumulator holds C transposed: the lane's row of C is lane % 32, so a per-row bias is one value per lane
     float16v acc[TM][TN];
@@ -281,9 +330,15 @@ __global__ __launch_bounds__(128 * WAVES_N) void gemm16_kernel(const T* A, const
     uint4v fa[2][TM], fb[2][TN];
     auto read_fragments = [&](const T* a_tile, const T* b_tile, int ks, int into) {
 #pragma unroll
-        for (int x = 0; x < TM; ++x) fa[into][x] = *reinterpret_cast<const uint4v*>(a_tile + tile_offset<T>(wm + x * 32 + frag_row, ks * 2 + frag_chunk));
+        for (int x = 0; x < TM; ++x) {
+            if constexpr (kAsIs<T, A_KMAJOR>) fa[into][x] = read_transposed<T, BM + 32>(a_tile, wm + x * 32, ks, tr_k * (BM + 32) + tr_row);
+            else fa[into][x] = *reinterpret_cast<const uint4v*>(a_tile + tile_offset<T>(wm + x * 32 + frag_row, ks * 2 + frag_chunk));
+        }
 #pragma unroll
-        for (int y = 0; y < TN; ++y) fb[into][y] = *reinterpret_cast<const uint4v*>(b_tile + tile_offset<T>(wn + y * 32 + frag_row, ks * 2 + frag_chunk));
+        for (int y = 0; y < TN; ++y) {
+            if constexpr (kAsIs<T, B_KMAJOR>) fb[into][y] = read_transposed<T, BN + 32>(b_tile, wn + y * 32, ks, tr_k * (BN + 32) + tr_row);
+            else fb[into][y] = *reinterpret_cast<const uint4v*>(b_tile + tile_offset<T>(wn + y * 32 + frag_row, ks * 2 + frag_chunk));
+        }
     };
     // (for tile 0 the "previous tile's" fragments are zeros: 16 MFMAs that add nothing keep the loop free of a
     // peeled first iteration, whose extra copy of the code costs more than it saves)
@@ -449,7 +504,7 @@ template <class T, int BM, int BN, int WAVES_N, bool AK, bool BK_, bool SPLIT = 
 int launch16(const GemmProblem& p, const void* a, const void* b, void* c, hipStream_t stream, SplitK sk = SplitK{1, 0, nullptr}) {
     const uint32_t tiles_m = (p.M + BM - 1) / BM, tiles_n = (p.N + BN - 1) / BN;
     // operand tiles (two buffers each); the same memory later stages the output, BM*BN elements in padded rows
-    constexpr size_t tile_bytes = sizeof(T) * 2 * (BM + BN) * kBKof<T>;
+    constexpr size_t tile_bytes = sizeof(T) * 2 * (kTileElements<T, BM, AK> + kTileElements<T, BN, BK_>);
     constexpr size_t stage_bytes = sizeof(T) * 2 * WAVES_N * (BM / 2) * (BN / WAVES_N + 8);
     constexpr size_t lds_bytes = (sizeof(T) == 2 && stage_bytes > tile_bytes) ? stage_bytes : tile_bytes;   // fp32 results are not staged
     auto kernel = gemm16_kernel<T, BM, BN, WAVES_N, AK, BK_, SPLIT>;
