@@ -42,6 +42,11 @@ LAYOUTS = {
     "skinny_batched": ((3, 5, 64), (3, 24, 64), [], [("transpose", (-1, -2))]),
     "split_k_nt": ((128, 1096), (136, 1096), [], [("transpose", (-1, -2))]),
     "split_k_nn": ((72, 2048), (2048, 64), [], []),
+    # operands contiguous along M / N with ragged tiles and a K tail, in every tile size (the largest needs 200 tiles)
+    "tn_tiles_ragged": ((200, 520), (200, 264), [("transpose", (-1, -2))], []),
+    "tt_tiles_ragged": ((136, 264), (520, 136), [("transpose", (-1, -2))], [("transpose", (-1, -2))]),
+    "tn_large_tiles_batched": ((50, 24, 264), (50, 24, 264), [("transpose", (-1, -2))], []),
+    "nn_large_tiles_batched": ((50, 264, 72), (50, 72, 264), [], []),
 }
 
 
