@@ -195,6 +195,13 @@ int tannic_hip_event_record(void* event, tannic_stream_t stream);
 /* milliseconds between two recorded events; waits for `stop`; <0 on failure */
 float tannic_hip_event_elapsed_ms(void* start, void* stop);
 
+/* Rate probe of the matrix pipe, for benchmark harnesses (no reference twin): `blocks` workgroups of four wavefronts
+ * issue nothing but MFMAs, `iterations` x 2^21 multiply-adds per wavefront, on operand values the caller supplies
+ * (`operands`: 64 KiB of device memory, 16 x 256 vectors of 16 bytes, read once; `sink`: 1 KiB per block, written
+ * once).  shape 0: v_mfma_f32_32x32x16, shape 1: v_mfma_f32_16x16x32; dtype TANNIC_FLOAT16 or TANNIC_BFLOAT16.
+ * What it sustains on given values is the ceiling of a product of such values on this device. */
+int tannic_hip_probe_mfma(int shape, int dtype, const void* operands, void* sink, uint32_t blocks, uint32_t iterations, tannic_stream_t stream);
+
 /* ------------------------------------------------------------------ *
  * Unary elementwise                 replaces src/cuda/ops.cuh:11-24
  *                                   (CPU semantics: src/cpu/ops-unary.cpp:202-370)
@@ -294,6 +301,10 @@ int tannic_hip_min(const tannic_tensor_t* src, tannic_tensor_t* dst, tannic_stre
  * Matrix multiply                   replaces src/cuda/matmul.cuh:12
  *                                   (CPU: src/cpu/matmul.cpp:126-176,254)
  * f16xf16 and bf16xbf16 accumulate in fp32 on MFMA and round once.
+ * Operand extents must fit the destination ([.., M, K] x [.., K, N] -> [.., M, N], batch extents 1 or the
+ * destination's): TANNIC_ERROR otherwise (the reference takes M, N from the destination and K from `a` on trust).
+ * The batch coordinate of an operand with fewer batch dims is multiplied by the stride of the dim it is looked up in;
+ * the reference multiplies it by the stride at the left-aligned position (src/cpu/matmul.cpp:107-118).
  * ------------------------------------------------------------------ */
 int tannic_hip_gemm(const tannic_tensor_t* a, const tannic_tensor_t* b, tannic_tensor_t* dst, tannic_stream_t stream);
 

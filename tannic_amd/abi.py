@@ -149,4 +149,5 @@ def runtime_signatures():
         "event_destroy": (None, [C.c_void_p]),
         "event_record": (C.c_int, [C.c_void_p, stream_t]),
         "event_elapsed_ms": (C.c_float, [C.c_void_p, C.c_void_p]),
+        "probe_mfma": (C.c_int, [C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_uint32, C.c_uint32, stream_t]),
     }

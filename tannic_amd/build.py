@@ -42,6 +42,8 @@ UNITS = [
     ("gemm.hip", "gemm.o", []),
     ("gemm_mfma.hip", "gemm_mfma.o", []),
     ("gemm_skinny.hip", "gemm_skinny.o", []),
+    ("gemm_dtl.hip", "gemm_dtl.o", []),
+    ("probes.hip", "probes.o", []),
     ("conv2d.hip", "conv2d.o", []),
     ("conv2d_mfma.hip", "conv2d_mfma.o", []),
     ("conv2d_patch.hip", "conv2d_patch.o", []),

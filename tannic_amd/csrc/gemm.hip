@@ -12,7 +12,15 @@
 //   - batch counts above 255 are handled (the CPU path narrows the batch
 //     counter to uint8_t, src/cpu/matmul.cpp:102);
 //   - an operand is addressed by both of its matrix strides (the CPU path
-//     takes the smaller one to be 1, src/cpu/matmul.cpp:87-94).
+//     takes the smaller one to be 1, src/cpu/matmul.cpp:87-94);
+//   - the batch coordinate of an operand with fewer batch dims than the
+//     destination is multiplied by the stride of the dim it was looked up in
+//     (right-aligned).  The CPU path looks the coordinate up right-aligned and
+//     multiplies it by the stride at the left-aligned position
+//     (src/cpu/matmul.cpp:107-118), which steps a[3,M,K] in a[3,M,K] x
+//     b[2,3,K,N] by its row stride;
+//   - operand extents are checked against the destination's (the CPU path
+//     takes M and N from the destination and K from the first operand on trust).
 #include "gemm_common.hpp"
 
 namespace th {
@@ -27,6 +35,24 @@ int describe_gemm(const tannic_tensor_t* a, const tannic_tensor_t* b, const tann
         set_error_text("gemm: dimension of 2^31 or more");
         return TANNIC_ERROR;
     }
+    // The kernels index both operands by the destination's M, N and batch coordinates and by the first operand's K:
+    // anything that does not fit would be read outside its storage.
+    if (a->shape.sizes[a->rank - 2] != M || b->shape.sizes[b->rank - 2] != K || b->shape.sizes[b->rank - 1] != N) {
+        set_error_text("gemm: operand extents do not fit the destination ([.., M, K] x [.., K, N] -> [.., M, N])");
+        return TANNIC_ERROR;
+    }
+    if (a->rank > c->rank || b->rank > c->rank) {
+        set_error_text("gemm: an operand has more dims than the destination");
+        return TANNIC_ERROR;
+    }
+    for (const tannic_tensor_t* s : {a, b})
+        for (int sd = 0; sd < s->rank - 2; ++sd) {
+            const size_t extent = s->shape.sizes[sd];
+            if (extent != 1 && extent != c->shape.sizes[sd + (c->rank - s->rank)]) {
+                set_error_text("gemm: a batch extent of an operand is neither 1 nor the destination's");
+                return TANNIC_ERROR;
+            }
+        }
     p.M = static_cast<uint32_t>(M);
     p.N = static_cast<uint32_t>(N);
     p.K = static_cast<uint32_t>(K);
@@ -50,13 +76,12 @@ int describe_gemm(const tannic_tensor_t* a, const tannic_tensor_t* b, const tann
         p.batch_extent[d] = static_cast<uint32_t>(c->shape.sizes[d]);
         batches *= c->shape.sizes[d];
         p.c_bs[d] = c->strides.sizes[d];
-        // src/cpu/matmul.cpp:107-118: the coordinate of an operand is looked up
-        // right-aligned (size-1 and missing dims give 0) and multiplied by the
-        // stride stored at position d of that operand
+        // the coordinate of an operand is looked up right-aligned (size-1 and missing dims give 0,
+        // src/cpu/matmul.cpp:107-112) and multiplied by the stride of that same dim
         auto stride_of = [&](const tannic_tensor_t* s) -> int64_t {
             const int sd = d + (s->rank - c->rank);
-            if (sd < 0 || s->shape.sizes[sd] == 1 || d >= s->rank) return 0;
-            return s->strides.sizes[d];
+            if (sd < 0 || s->shape.sizes[sd] == 1) return 0;
+            return s->strides.sizes[sd];
         };
         p.a_bs[d] = stride_of(a);
         p.b_bs[d] = stride_of(b);

@@ -43,5 +43,7 @@ int describe_gemm(const tannic_tensor_t* a, const tannic_tensor_t* b, const tann
 int gemm_skinny_16bit(const GemmProblem& p, int dtype, const void* a, const void* b, void* c, hipStream_t stream);
 int gemm_mfma_16bit(const GemmProblem& p, int dtype, const void* a, const void* b, void* c, hipStream_t stream);
 int gemm_mfma_f32(const GemmProblem& p, const float* a, const float* b, float* c, hipStream_t stream);
+// 256 x 256 tiles filled by direct global -> LDS loads (gemm_dtl.hip); T is f16 or bf16
+template <class T> int gemm16_dtl(const GemmProblem& p, const void* a, const void* b, void* c, hipStream_t stream);
 
 }  // namespace th

@@ -26,61 +26,9 @@
 // one XCD share A and B panels.
 #include "gemm_common.hpp"
 
+#include "gemm_tiles.hpp"
+
 namespace th {
-
-typedef _Float16 half8 __attribute__((ext_vector_type(8)));
-typedef __bf16 bfloat8 __attribute__((ext_vector_type(8)));
-typedef float float16v __attribute__((ext_vector_type(16)));
-typedef unsigned int uint4v __attribute__((ext_vector_type(4)));
-
-template <class T> struct Mfma16;
-template <> struct Mfma16<f16> {
-    __device__ static inline float16v run(uint4v a, uint4v b, float16v c) {
-        half8 x, y;
-        __builtin_memcpy(&x, &a, 16);
-        __builtin_memcpy(&y, &b, 16);
-        return __builtin_amdgcn_mfma_f32_32x32x16_f16(x, y, c, 0, 0, 0);
-    }
-};
-template <> struct Mfma16<bf16> {
-    __device__ static inline float16v run(uint4v a, uint4v b, float16v c) {
-        bfloat8 x, y;
-        __builtin_memcpy(&x, &a, 16);
-        __builtin_memcpy(&y, &b, 16);
-        return __builtin_amdgcn_mfma_f32_32x32x16_bf16(x, y, c, 0, 0, 0);
-    }
-};
-
-// A tile row is 128 bytes = eight 16-byte chunks for every element type.
-template <class T> constexpr int kBKof = 128 / sizeof(T);      // K elements per step: 64 (16-bit), 32 (fp32)
-template <class T> constexpr int kChunkOf = 16 / sizeof(T);    // elements per 16-byte chunk
-template <> struct Mfma16<float> {
-    // element e of both fragments is one k: four 32x32x2 MFMAs (lanes 0-31 hold one k of the pair, lanes 32-63 the other)
-    __device__ static inline float16v run(uint4v a, uint4v b, float16v c) {
-        float x[4], y[4];
-        __builtin_memcpy(x, &a, 16);
-        __builtin_memcpy(y, &b, 16);
-#pragma unroll
-        for (int e = 0; e < 4; ++e) c = __builtin_amdgcn_mfma_f32_32x32x2f32(x[e], y[e], c, 0, 0, 0);
-        return c;
-    }
-};
-
-constexpr int kBK = 64;          // K granule the host splits by (a multiple of every type's step)
-
-// Maps the hardware workgroup id to a tile: XCD folding, then grouped rows.
-__device__ inline void tile_of(uint32_t wg, uint32_t tiles_m, uint32_t tiles_n, uint32_t& tm, uint32_t& tn) {
-    const uint32_t total = tiles_m * tiles_n;
-    uint32_t id = wg;
-    if (total % 8 == 0) id = (wg % 8) * (total / 8) + wg / 8;
-    constexpr uint32_t GROUP = 4;
-    const uint32_t width = GROUP * tiles_n;
-    const uint32_t group = id / width;
-    const uint32_t first = group * GROUP;
-    const uint32_t rows = tiles_m - first < GROUP ? tiles_m - first : GROUP;
-    tm = first + (id % width) % rows;
-    tn = (id % width) / rows;
-}
 
 // One operand of the product seen as rows x K: element (r, k) at
 // base[r * row_stride + k * k_stride]; exactly one of the strides is 1.
@@ -90,20 +38,6 @@ struct Operand {
     uint32_t rows;  // M for A, N for B
 };
 
-// Calls f(std::integral_constant<int, 0>{}) ... f(std::integral_constant<int, N-1>{}).
-template <int N, class F, int I = 0>
-__device__ inline void static_for(F&& f) {
-    if constexpr (I < N) {
-        f(std::integral_constant<int, I>{});
-        static_for<N, F, I + 1>(static_cast<F&&>(f));
-    }
-}
-
-// Swizzled element offset of (row, chunk) inside a [ROWS][128 bytes] tile.
-// LDS serves 16 lanes of a 16-byte read per clock out of a 256-byte bank window,
-// i.e. two 128-byte rows: consecutive row PAIRS get different chunk rotations so
-// that 16 consecutive rows of one logical chunk land in 16 different slots.
-template <class T> __device__ inline uint32_t tile_offset(uint32_t row, uint32_t chunk) { return row * kBKof<T> + ((chunk ^ ((row >> 1) & 7u)) * kChunkOf<T>); }
 
 // ---- global -> registers -> LDS, operand contiguous along K -------------------
 // Rows past the operand's end read a clamped (valid) address: they only feed
@@ -589,6 +523,9 @@ int run16_split(const GemmProblem& p, bool ak, bool bk, uint32_t splits, const v
 template <class T>
 int run16(const GemmProblem& p, const void* a, const void* b, void* c, hipStream_t stream) {
     if (p.M == 0 || p.N == 0 || p.batches == 0) return TANNIC_SUCCESS;
+    // No products to add: the operands hold no elements (their addresses may be null) and the tile loaders would still
+    // fetch a first tile.  The scalar kernel, whose K loop then does not run, writes the zeros.
+    if (p.K == 0) return TANNIC_UNSUPPORTED_DTYPE;
     // layout of each operand: along which index is it contiguous?
     const bool ak = p.a_cs == 1, bk = p.b_rs == 1;
     if (!ak && p.a_rs != 1) return TANNIC_UNSUPPORTED_DTYPE;
@@ -604,7 +541,16 @@ int run16(const GemmProblem& p, const void* a, const void* b, void* c, hipStream
     if (p.batches > 65535) return TANNIC_UNSUPPORTED_DTYPE;
     // Tile height by M (a tile taller than M multiplies padding), large tiles only when they still give every CU work.
     const uint64_t big = static_cast<uint64_t>((p.M + 255) / 256) * ((p.N + 255) / 256) * p.batches;
-    if (p.M > 192 && big >= 200) return pick_layout16<T, 256, 256, 2>(p, ak, bk, a, b, c, stream);
+    if (p.M > 192 && big >= 200) {
+        if constexpr (sizeof(T) == 2) {
+            static const bool direct = [] { const char* e = getenv("TANNIC_GEMM_DTL"); return !e || atoi(e) != 0; }();
+            if (direct) {
+                const int rc = gemm16_dtl<T>(p, a, b, c, stream);
+                if (rc != TANNIC_UNSUPPORTED_DTYPE) return rc;
+            }
+        }
+        return pick_layout16<T, 256, 256, 2>(p, ak, bk, a, b, c, stream);
+    }
     // Fewer large tiles than compute units: choose between the smaller tiles (256 x 128, 128 x 128, 64 x 128) and between
     // whole K per block and a share of it, by a model of the time (microseconds): blocks on the busiest compute unit x
     // steps per block x the measured time of one 64-wide step of that tile, a fixed start-up and write-out, and for

@@ -64,6 +64,11 @@ template <class T>
 int run_cpy(const tannic_tensor_t* src, tannic_tensor_t* dst, hipStream_t stream) {
     int64_t strides[kMaxOperands][TANNIC_DIMENSIONS] = {};
     const int rank = src->rank;
+    // the copy walks the destination's index space: a source dim must have that extent or 1 (pinned to index 0)
+    if (dst->rank != rank) return shape_mismatch("cpy: source and destination differ in rank");
+    for (int d = 0; d < rank; ++d)
+        if (src->shape.sizes[d] != 1 && src->shape.sizes[d] != dst->shape.sizes[d])
+            return shape_mismatch("cpy: a source extent is neither 1 nor the destination's");
     for (int d = 0; d < rank; ++d) {
         strides[0][d] = src->shape.sizes[d] == 1 ? 0 : src->strides.sizes[d];
         strides[2][d] = dst->shape.sizes[d] == 1 ? 0 : dst->strides.sizes[d];
@@ -129,6 +134,11 @@ int run_complex(const tannic_tensor_t* a, const tannic_tensor_t* b, tannic_tenso
         set_error_text("complex: operands must have the destination's rank");
         return TANNIC_ERROR;
     }
+    // both parts are indexed by the destination's coordinates: an extent must be the destination's or 1
+    for (int d = 0; d < rank; ++d)
+        for (const tannic_tensor_t* t : {a, b})
+            if (t->shape.sizes[d] != 1 && t->shape.sizes[d] != dst->shape.sizes[d])
+                return shape_mismatch("complex: an operand extent is neither 1 nor the destination's");
     for (int d = 0; d < rank; ++d) {
         strides[0][d] = a->shape.sizes[d] == 1 ? 0 : a->strides.sizes[d];
         strides[1][d] = b->shape.sizes[d] == 1 ? 0 : b->strides.sizes[d];

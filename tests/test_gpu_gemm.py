@@ -47,6 +47,11 @@ LAYOUTS = {
     "tt_tiles_ragged": ((136, 264), (520, 136), [("transpose", (-1, -2))], [("transpose", (-1, -2))]),
     "tn_large_tiles_batched": ((50, 24, 264), (50, 24, 264), [("transpose", (-1, -2))], []),
     "nn_large_tiles_batched": ((50, 264, 72), (50, 72, 264), [], []),
+    # both operands K-contiguous, whole K steps, 200 large tiles: the tiles filled by direct global -> LDS loads
+    # (rows past the end of both operands; one, two and three K steps)
+    "nt_direct_one_step": ((50, 264, 64), (50, 264, 64), [], [("transpose", (-1, -2))]),
+    "nt_direct_two_steps": ((50, 264, 128), (50, 264, 128), [], [("transpose", (-1, -2))]),
+    "nt_direct_ragged_rows": ((10, 1000, 192), (10, 1096, 192), [], [("transpose", (-1, -2))]),
 }
 
 
@@ -100,6 +105,25 @@ def test_mixed_gemm(device, pair):
     want, got = ops.matmul(*host), ops.matmul(*dev)
     assert got.dtype is want.dtype
     support.assert_close(got.numpy(), want.numpy(), 1e-5, k * 9 * 2.0 ** -24, f"gemm {pair}")
+
+
+def test_operand_with_fewer_batch_dims_steps_by_its_own_batch_stride(device):
+    """a[3,M,K] x b[2,3,K,N]: the batch coordinate of `a` is looked up right-aligned and multiplied by the stride of
+    that same dim.  (The reference multiplies it by the stride at the left-aligned position, src/cpu/matmul.cpp:107-118,
+    i.e. steps `a` by its row stride: this is a documented difference, so the expectation here is numpy's.)"""
+    a = support.uniform(SEED, 5, (3, 9, 16))
+    b = support.uniform(SEED, 6, (2, 3, 16, 11))
+    for dtype, rtol, atol in ((ta.float32, 1e-5, 16 * 2.0 ** -24), (ta.float16, 2e-3, 1e-3), (ta.int32, 0, 0)):
+        va = np.floor(a * 50) if dtype.is_integral else a
+        vb = np.floor(b * 50) if dtype.is_integral else b
+        _, da = support.both(va, dtype, device)
+        _, db = support.both(vb, dtype, device)
+        got = ops.matmul(da, db).numpy().astype(np.float64)
+        ra = da.numpy().astype(np.float64)
+        rb = db.numpy().astype(np.float64)
+        support.assert_close(got, np.matmul(ra, rb), rtol, atol, f"rank 3 x rank 4 {dtype}")
+        got = ops.matmul(db.transpose(), da.transpose()).numpy().astype(np.float64)      # [2,3,N,K] x [3,K,M]
+        support.assert_close(got, np.matmul(rb.swapaxes(-1, -2), ra.swapaxes(-1, -2)), rtol, atol, f"rank 4 x rank 3 {dtype}")
 
 
 def test_integer_valued_fp16_gemm_is_exact(device):

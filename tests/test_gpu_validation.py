@@ -77,6 +77,36 @@ def test_reduction_destination_must_hold_one_element_per_slice(device, name):
     assert status == abi.SUCCESS
 
 
+def test_gemm_operand_extents_must_fit_the_destination(device):
+    """The kernels take M and N from the destination and K from the first operand: operands that are smaller than that
+    would be read past their end."""
+    f = lambda *shape: zeros(shape, ta.float16, device)
+    for a, b, dst in ((f(8, 8), f(8, 8), f(16, 16)),                 # destination larger than the product
+                      (f(64, 32), f(64, 64), f(64, 64)),             # K of the second operand
+                      (f(64, 64), f(64, 32), f(64, 64)),             # N of the second operand
+                      (f(32, 64), f(64, 64), f(64, 64)),             # M of the first operand
+                      (f(2, 64, 64), f(64, 64), f(3, 64, 64)),       # batch extent neither 1 nor the destination's
+                      (f(2, 3, 8, 8), f(8, 8), f(3, 8, 8))):         # operand of higher rank than the destination
+        status, message = call("gemm", device, [a, b], dst)
+        assert status == abi.ERROR and "gemm" in message, (a.shape, b.shape, dst.shape, status, message)
+    status, _ = call("gemm", device, [f(1, 64, 32), f(32, 64)], f(3, 64, 64))
+    assert status == abi.SUCCESS
+
+
+def test_copy_and_complex_operands_must_fit_the_destination(device):
+    status, message = call("cpy", device, [zeros((4, 6), ta.float32, device)], zeros((4, 8), ta.float32, device))
+    assert status == abi.ERROR and "cpy" in message
+    status, message = call("cpy", device, [zeros((4, 6), ta.float32, device)], zeros((2, 4, 6), ta.float32, device))
+    assert status == abi.ERROR and "cpy" in message
+    status, _ = call("cpy", device, [zeros((1, 6), ta.float32, device)], zeros((4, 6), ta.float32, device))     # extent 1 repeats
+    assert status == abi.SUCCESS
+    for name in ("view_as_cartesian", "view_as_polar"):
+        status, message = call(name, device, [zeros((4, 6), ta.float32, device), zeros((4, 5), ta.float32, device)], zeros((4, 6), ta.complex64, device))
+        assert status == abi.ERROR and "complex" in message
+        status, _ = call(name, device, [zeros((4, 6), ta.float32, device), zeros((1, 6), ta.float32, device)], zeros((4, 6), ta.complex64, device))
+        assert status == abi.SUCCESS
+
+
 # ---- dtypes that do not fit each other -----------------------------------------------------------------------------------
 # A kernel writes elements of one type: a destination described with another dtype would be over- or under-run, and a
 # second operand read as the first's type (what the reference's comparison and allclose do) would be read past its end.
@@ -154,12 +184,14 @@ def test_empty_tensors_go_through_every_family(device, oracle, shape):
     # value max / min over an axis without elements: the start value of the fold
     h, d = support.both(np.zeros((0, 4)), ta.float32, device)
     assert np.isneginf(ops.max(d, 0).numpy()).all() and np.isposinf(ops.min(d, 0).numpy()).all()
-    for sa, sb in (((0, 4), (4, 3)), ((3, 4), (4, 0)), ((3, 0), (0, 5))):
-        ha, da = support.both(np.ones(sa), ta.float16, device)
-        hb, db = support.both(np.ones(sb), ta.float16, device)
-        want, got = ops.matmul(ha, hb), ops.matmul(da, db)
-        assert got.shape == want.shape
-        support.assert_bit_exact(got.storage(), want.storage(), f"matmul {sa} x {sb}")
+    # (the last two: extents that meet the tiled kernels' alignment conditions, whose loaders would fetch a first tile)
+    for sa, sb in (((0, 4), (4, 3)), ((3, 4), (4, 0)), ((3, 0), (0, 5)), ((64, 0), (0, 512)), ((512, 0), (0, 512))):
+        for dtype in (ta.float16, ta.float32):
+            ha, da = support.both(np.ones(sa), dtype, device)
+            hb, db = support.both(np.ones(sb), dtype, device)
+            want, got = ops.matmul(ha, hb), ops.matmul(da, db)
+            assert got.shape == want.shape
+            support.assert_bit_exact(got.storage(), want.storage(), f"matmul {dtype} {sa} x {sb}")
 
 
 def test_a_tensor_without_storage_is_refused(device):
