@@ -308,6 +308,18 @@ int tannic_hip_min(const tannic_tensor_t* src, tannic_tensor_t* dst, tannic_stre
  * ------------------------------------------------------------------ */
 int tannic_hip_gemm(const tannic_tensor_t* a, const tannic_tensor_t* b, tannic_tensor_t* dst, tannic_stream_t stream);
 
+/* tannic_hip_gemm for callers that must not allocate device memory (code under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc).  No counterpart in the reference.  Same arguments, checks and results as
+ * tannic_hip_gemm, bit for bit; the kernels that share K between workgroups (few output tiles, long K) leave their
+ * fp32 partial sums in a fixed array of TANNIC_GEMM_NOALLOC_SCRATCH_BYTES that is part of the library's device code
+ * (each device the library runs on holds one copy until the process ends) instead of a block from the scratch cache.
+ * A product whose partial sums need more returns TANNIC_ERROR with the sizes in tannic_hip_last_error(); such a caller
+ * uses tannic_hip_gemm.  Nothing is allocated or freed by this call, on the device or through the runtime.  All calls
+ * on one device share the one array: calls that may overlap on a device (different streams, different threads) race;
+ * calls on one stream are ordered by it. */
+#define TANNIC_GEMM_NOALLOC_SCRATCH_BYTES ((size_t)8 << 20)
+int tannic_hip_gemm_noalloc(const tannic_tensor_t* a, const tannic_tensor_t* b, tannic_tensor_t* dst, tannic_stream_t stream);
+
 /* cuda::conv1d(x, w, y, stream, pad, stride): x[N,C,L], w[O,C,K], y[N,O,(L+2*pad-K)/stride+1]; ERROR on rank != 3 or
  * shape mismatch; same dtype for signal and kernel (src/cuda/conv.cuh:11; CPU: src/cpu/conv1d.cpp:17-125) */
 int tannic_hip_conv1d(const tannic_tensor_t* x, const tannic_tensor_t* w, tannic_tensor_t* y, tannic_stream_t stream, size_t pad, size_t stride);

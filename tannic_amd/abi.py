@@ -103,7 +103,7 @@ def kernel_signatures(with_stream):
     for n in UNARY_OPS:
         sig[n] = (C.c_int, [TP, TP] + s)
     sig["rsqrt"] = (C.c_int, [TP, TP] + s + [C.c_float])
-    for n in BINARY_OPS + COMPARE_OPS + COMPLEX_OPS + ["gemm"]:
+    for n in BINARY_OPS + COMPARE_OPS + COMPLEX_OPS + ["gemm"] + (["gemm_noalloc"] if with_stream else []):
         sig[n] = (C.c_int, [TP, TP, TP] + s)
     sig["scale"] = (C.c_int, [TP, SP, TP] + s)
     for n in REDUCE_OPS:

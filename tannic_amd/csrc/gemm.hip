@@ -188,7 +188,9 @@ int run_generic(const GemmProblem& p, const void* a, const void* b, void* c, hip
 
 using namespace th;
 
-extern "C" int tannic_hip_gemm(const tannic_tensor_t* a, const tannic_tensor_t* b, tannic_tensor_t* dst, tannic_stream_t stream) {
+namespace {
+
+int gemm_entry(const tannic_tensor_t* a, const tannic_tensor_t* b, tannic_tensor_t* dst, tannic_stream_t stream, const GemmWorkspace* workspace) {
     if (!a || !b || !dst) return TANNIC_ERROR;
     if (!have_storage(a, b, dst)) return TANNIC_ERROR;
     int status = TANNIC_UNSUPPORTED_DTYPE;
@@ -207,11 +209,11 @@ extern "C" int tannic_hip_gemm(const tannic_tensor_t* a, const tannic_tensor_t* 
                 status = describe_gemm(a, b, dst, p);
                 if (status != TANNIC_SUCCESS) return;
                 if constexpr (std::is_same_v<A, B> && is_16bit<A>::value) {
-                    status = gemm_mfma_16bit(p, a->dtype, a->address, b->address, dst->address, s);
+                    status = gemm_mfma_16bit(p, a->dtype, a->address, b->address, dst->address, s, workspace);
                     if (status != TANNIC_UNSUPPORTED_DTYPE) return;
                 } else if constexpr (std::is_same_v<A, float> && std::is_same_v<B, float>) {
                     status = gemm_mfma_f32(p, static_cast<const float*>(a->address), static_cast<const float*>(b->address),
-                                           static_cast<float*>(dst->address), s);
+                                           static_cast<float*>(dst->address), s, workspace);
                     if (status != TANNIC_UNSUPPORTED_DTYPE) return;
                 }
                 status = run_generic<A, B, D>(p, a->address, b->address, dst->address, s);
@@ -219,4 +221,43 @@ extern "C" int tannic_hip_gemm(const tannic_tensor_t* a, const tannic_tensor_t* 
         });
     });
     return status;
+}
+
+// Partial sums of tannic_hip_gemm_noalloc: device memory that exists from the moment the library's code is loaded on a
+// device until the process ends, one copy per device.
+constexpr size_t kNoAllocScratchBytes = TANNIC_GEMM_NOALLOC_SCRATCH_BYTES;
+__device__ __align__(256) unsigned char scratch[kNoAllocScratchBytes];
+
+// The array's address on the current device.  In host code the name `scratch` is only a handle for this lookup; the
+// kernels are given the address it returns.  Looked up once per device, with that device current.
+constexpr int kMaxDevices = 64;
+std::atomic<void*> g_scratch_address[kMaxDevices];
+
+int scratch_address(void** out) {
+    int device = 0;
+    TH_TRY(hipGetDevice(&device));
+    if (device < 0 || device >= kMaxDevices) {
+        set_error_text("gemm_noalloc: device id beyond the table of scratch addresses");
+        return TANNIC_ERROR;
+    }
+    void* ptr = g_scratch_address[device].load(std::memory_order_acquire);
+    if (!ptr) {
+        TH_TRY(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));
+        g_scratch_address[device].store(ptr, std::memory_order_release);
+    }
+    *out = ptr;
+    return TANNIC_SUCCESS;
+}
+
+}  // namespace
+
+extern "C" int tannic_hip_gemm(const tannic_tensor_t* a, const tannic_tensor_t* b, tannic_tensor_t* dst, tannic_stream_t stream) {
+    return gemm_entry(a, b, dst, stream, nullptr);
+}
+
+extern "C" int tannic_hip_gemm_noalloc(const tannic_tensor_t* a, const tannic_tensor_t* b, tannic_tensor_t* dst, tannic_stream_t stream) {
+    void* base = nullptr;
+    if (int rc = scratch_address(&base)) return rc;
+    const GemmWorkspace workspace{base, kNoAllocScratchBytes};
+    return gemm_entry(a, b, dst, stream, &workspace);
 }

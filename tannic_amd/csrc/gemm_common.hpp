@@ -38,11 +38,18 @@ __host__ __device__ inline void batch_offsets(const GemmProblem& p, uint32_t bat
 // (src/cpu/matmul.cpp:126-176).  Returns a status.
 int describe_gemm(const tannic_tensor_t* a, const tannic_tensor_t* b, const tannic_tensor_t* c, GemmProblem& p);
 
+// Where the kernels that share K between blocks leave their fp32 partial sums.  nullptr: a block from the library's
+// scratch cache (allocated on first need); otherwise caller-supplied memory, and a need beyond `bytes` is an error.
+struct GemmWorkspace {
+    void* base;
+    size_t bytes;
+};
+
 // MFMA paths; each returns TANNIC_UNSUPPORTED_DTYPE when the problem does not
 // meet its layout/alignment conditions so that the caller can fall back.
 int gemm_skinny_16bit(const GemmProblem& p, int dtype, const void* a, const void* b, void* c, hipStream_t stream);
-int gemm_mfma_16bit(const GemmProblem& p, int dtype, const void* a, const void* b, void* c, hipStream_t stream);
-int gemm_mfma_f32(const GemmProblem& p, const float* a, const float* b, float* c, hipStream_t stream);
+int gemm_mfma_16bit(const GemmProblem& p, int dtype, const void* a, const void* b, void* c, hipStream_t stream, const GemmWorkspace* workspace = nullptr);
+int gemm_mfma_f32(const GemmProblem& p, const float* a, const float* b, float* c, hipStream_t stream, const GemmWorkspace* workspace = nullptr);
 // 256 x 256 tiles filled by direct global -> LDS loads (gemm_dtl.hip); T is f16 or bf16
 template <class T> int gemm16_dtl(const GemmProblem& p, const void* a, const void* b, void* c, hipStream_t stream);
 

@@ -495,7 +495,7 @@ __global__ __launch_bounds__(256) void gemm_split_reduce_kernel(const float* par
 
 // Few tiles and a long K: each tile is shared by `splits` blocks.
 template <class T, int BM>
-int run16_split(const GemmProblem& p, bool ak, bool bk, uint32_t splits, const void* a, const void* b, void* c, hipStream_t stream) {
+int run16_split(const GemmProblem& p, bool ak, bool bk, uint32_t splits, const void* a, const void* b, void* c, hipStream_t stream, const GemmWorkspace* workspace) {
     constexpr int BN = 128;
     const uint32_t steps = (p.K + kBK - 1) / kBK;
     SplitK sk{};
@@ -504,7 +504,17 @@ int run16_split(const GemmProblem& p, bool ak, bool bk, uint32_t splits, const v
     const uint64_t rows = static_cast<uint64_t>(p.batches) * p.M, quads_per_row = (p.N + 3) / 4;
     if (rows * quads_per_row >= (1ull << 31)) return TANNIC_UNSUPPORTED_DTYPE;
     const size_t bytes = static_cast<size_t>(sk.splits) * rows * p.N * sizeof(float);
-    if (scratch_acquire(reinterpret_cast<void**>(&sk.partials), bytes, stream) != TANNIC_SUCCESS) return TANNIC_ERROR;
+    if (workspace) {
+        if (bytes > workspace->bytes) {
+            char text[160];
+            snprintf(text, sizeof text, "gemm: this product shares K between blocks and needs %zu bytes for partial sums; the workspace holds %zu", bytes, workspace->bytes);
+            set_error_text(text);
+            return TANNIC_ERROR;
+        }
+        sk.partials = static_cast<float*>(workspace->base);
+    } else if (scratch_acquire(reinterpret_cast<void**>(&sk.partials), bytes, stream) != TANNIC_SUCCESS) {
+        return TANNIC_ERROR;
+    }
     int status;
     if (ak && bk) status = launch16<T, BM, BN, 2, true, true, true>(p, a, b, c, stream, sk);
     else if (ak) status = launch16<T, BM, BN, 2, true, false, true>(p, a, b, c, stream, sk);
@@ -516,12 +526,12 @@ int run16_split(const GemmProblem& p, bool ak, bool bk, uint32_t splits, const v
                            static_cast<uint32_t>(quads_per_row), total);
         status = launch_status("gemm_split_reduce_kernel");
     }
-    scratch_release(sk.partials, stream);
+    if (!workspace) scratch_release(sk.partials, stream);
     return status;
 }
 
 template <class T>
-int run16(const GemmProblem& p, const void* a, const void* b, void* c, hipStream_t stream) {
+int run16(const GemmProblem& p, const void* a, const void* b, void* c, hipStream_t stream, const GemmWorkspace* workspace) {
     if (p.M == 0 || p.N == 0 || p.batches == 0) return TANNIC_SUCCESS;
     // No products to add: the operands hold no elements (their addresses may be null) and the tile loaders would still
     // fetch a first tile.  The scalar kernel, whose K loop then does not run, writes the zeros.
@@ -576,23 +586,23 @@ int run16(const GemmProblem& p, const void* a, const void* b, void* c, hipStream
         }
     }
     if (best_splits > 1) {
-        if (best_bm == 128) return run16_split<T, 128>(p, ak, bk, best_splits, a, b, c, stream);
-        return run16_split<T, 64>(p, ak, bk, best_splits, a, b, c, stream);
+        if (best_bm == 128) return run16_split<T, 128>(p, ak, bk, best_splits, a, b, c, stream, workspace);
+        return run16_split<T, 64>(p, ak, bk, best_splits, a, b, c, stream, workspace);
     }
     if (best_bm == 256) return pick_layout16<T, 256, 128, 2>(p, ak, bk, a, b, c, stream);
     if (best_bm == 128) return pick_layout16<T, 128, 128, 2>(p, ak, bk, a, b, c, stream);
     return pick_layout16<T, 64, 128, 2>(p, ak, bk, a, b, c, stream);
 }
 
-int gemm_mfma_16bit(const GemmProblem& p, int dtype, const void* a, const void* b, void* c, hipStream_t stream) {
+int gemm_mfma_16bit(const GemmProblem& p, int dtype, const void* a, const void* b, void* c, hipStream_t stream, const GemmWorkspace* workspace) {
     // a handful of rows: stream the other operand once, no tiles
     const int skinny = gemm_skinny_16bit(p, dtype, a, b, c, stream);
     if (skinny != TANNIC_UNSUPPORTED_DTYPE) return skinny;
-    if (dtype == TANNIC_FLOAT16) return run16<f16>(p, a, b, c, stream);
-    if (dtype == TANNIC_BFLOAT16) return run16<bf16>(p, a, b, c, stream);
+    if (dtype == TANNIC_FLOAT16) return run16<f16>(p, a, b, c, stream, workspace);
+    if (dtype == TANNIC_BFLOAT16) return run16<bf16>(p, a, b, c, stream, workspace);
     return TANNIC_UNSUPPORTED_DTYPE;
 }
 
-int gemm_mfma_f32(const GemmProblem& p, const float* a, const float* b, float* c, hipStream_t stream) { return run16<float>(p, a, b, c, stream); }
+int gemm_mfma_f32(const GemmProblem& p, const float* a, const float* b, float* c, hipStream_t stream, const GemmWorkspace* workspace) { return run16<float>(p, a, b, c, stream, workspace); }
 
 }  // namespace th
