@@ -50,7 +50,7 @@ struct GemmWorkspace {
 int gemm_skinny_16bit(const GemmProblem& p, int dtype, const void* a, const void* b, void* c, hipStream_t stream);
 int gemm_mfma_16bit(const GemmProblem& p, int dtype, const void* a, const void* b, void* c, hipStream_t stream, const GemmWorkspace* workspace = nullptr);
 int gemm_mfma_f32(const GemmProblem& p, const float* a, const float* b, float* c, hipStream_t stream, const GemmWorkspace* workspace = nullptr);
-// 256 x 256 tiles filled by direct global -> LDS loads (gemm_dtl.hip); T is f16 or bf16
-template <class T> int gemm16_dtl(const GemmProblem& p, const void* a, const void* b, void* c, hipStream_t stream);
+// bm x bn tiles (256 x 256, 256 x 128, 128 x 128) filled by direct global -> LDS loads (gemm_dtl.hip); T is f16 or bf16
+template <class T> int gemm16_dtl(const GemmProblem& p, int bm, int bn, const void* a, const void* b, void* c, hipStream_t stream);
 
 }  // namespace th

@@ -8,9 +8,11 @@
 // no register holds operand data on its way and no ds_write is issued.  Such a load writes the 64 lanes' 16 bytes to
 // consecutive LDS addresses, 1 KB = eight 128-byte tile rows; the swizzle permutes the eight 16-byte chunks inside a row,
 // so it is applied on the global side: the lane that fills slot c of row r fetches chunk c ^ ((r >> 1) & 7) of that row
-// (still whole 128-byte lines).  The loads of tile s+1 are issued between the first MFMAs of step s into the buffer tile
-// s-1 has left; the step ends with vmcnt(0) and one barrier.  Operands are addressed through buffer resources, whose
-// range check returns zeros for rows past the operand's end.
+// (still whole 128-byte lines).  LDS holds STAGES tiles (2 for 256 x 256, 3 for 256 x 128, 4 for 128 x 128): the loads of
+// tile s+STAGES-1 are issued between the first MFMAs of step s into the buffer tile s-1 has left, and a step ends with
+// a wait for the loads of tile s+1 only (loads complete in order, so "at most (STAGES-2) tiles' worth outstanding")
+// and one barrier.  Operands are addressed through buffer resources, whose range check returns zeros for rows past the
+// operand's end.
 //
 // The MFMA: per multiply-add the 16 x 16 x 32 instruction reads and writes half the accumulator registers of the
 // 32 x 32 x 16 one (and twice the operand registers, which are a quarter of the size).  Under the chip's power limit it
@@ -41,14 +43,17 @@ template <class T> __device__ inline void mfma16x16_in_place(float4v& acc, const
     }
 }
 
-template <class T, int LOAD_EVERY>
-__global__ __launch_bounds__(256) void gemm16_dtl16_kernel(const T* A, const T* B, T* C, GemmProblem p, uint32_t tiles_m, uint32_t tiles_n) {
-    constexpr int BM = 256, BN = 256, BK = 64;
-    constexpr int WM = 128, WN = 128, TM = 8, TN = 8, WAVES_N = 2;
-    constexpr uint32_t TILE = 256 * BK;
-    constexpr uint32_t TILE_BYTES = TILE * 2, STAGE_BYTES = 2 * TILE_BYTES;
+// BM x BN: 256 x 256, 256 x 128 or 128 x 128 (2 x 2 wavefronts each).  The smaller tiles are for products with too few
+// large tiles to fill the chip; two workgroups of the smallest share a compute unit.
+template <class T, int BM, int BN, int STAGES, int BLOCKS_PER_CU>
+__global__ __launch_bounds__(256, BLOCKS_PER_CU) void gemm16_dtl_kernel(const T* A, const T* B, T* C, GemmProblem p, uint32_t tiles_m, uint32_t tiles_n) {
+#if defined(__HIP_DEVICE_COMPILE__)   // the host pass needs the launch stub only (and loses it over the body's device-only builtins)
+    constexpr int BK = 64, WAVES_N = 2;
+    constexpr int WM = BM / 2, WN = BN / 2, TM = WM / 16, TN = WN / 16;
+    constexpr uint32_t A_TILE = BM * BK, B_TILE = BN * BK, STAGE = A_TILE + B_TILE;   // elements
+    constexpr int LOADS_A = BM / 32, LOADS_B = BN / 32, LOADS = LOADS_A + LOADS_B;     // 1 KB loads per wavefront and tile
     extern __shared__ __align__(16) unsigned char lds_raw[];
-    T* lds = reinterpret_cast<T*>(lds_raw);
+    T* lds = reinterpret_cast<T*>(lds_raw);           // stage s: A tile at s * STAGE, B tile right behind it
 
     uint32_t tm, tn;
     tile_of(blockIdx.x, tiles_m, tiles_n, tm, tn);
@@ -61,6 +66,7 @@ __global__ __launch_bounds__(256) void gemm16_dtl16_kernel(const T* A, const T* 
     const int wm = (wave / WAVES_N) * WM, wn = (wave % WAVES_N) * WN;
     const uint32_t frag_row = lane % 16, frag_chunk = lane / 16;
 
+    // Buffer resources starting at the tile's first row: offsets stay below 2^31 and rows past the end are out of range.
     const T* a_base = A + oa + static_cast<int64_t>(m0) * p.a_rs;
     const T* b_base = B + ob + static_cast<int64_t>(n0) * p.b_cs;
     auto records = [](uint64_t rows_left, int64_t stride, uint32_t K) -> uint32_t {
@@ -69,17 +75,18 @@ __global__ __launch_bounds__(256) void gemm16_dtl16_kernel(const T* A, const T* 
     };
     const __amdgpu_buffer_rsrc_t rsrc_a = __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(a_base), 0, records(p.M - m0, p.a_rs, p.K), 0x00020000);
     const __amdgpu_buffer_rsrc_t rsrc_b = __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(b_base), 0, records(p.N - n0, p.b_cs, p.K), 0x00020000);
-    uint32_t voff[16];
+    // Load j of a wavefront fills eight rows of a tile (j < LOADS_A: rows 8 * (LOADS_A * wave + j) .. + 7 of A's, then B's
+    // likewise); the lane's byte offset from the tile's first row:
+    uint32_t voff[LOADS];
 #pragma unroll
-    for (int j = 0; j < 8; ++j) {
-        const uint32_t row = (wave * 8 + j) * 8 + lane / 8;
+    for (int j = 0; j < LOADS; ++j) {
+        const uint32_t row = (j < LOADS_A ? wave * LOADS_A + j : wave * LOADS_B + (j - LOADS_A)) * 8 + lane / 8;
         const uint32_t chunk = (lane % 8) ^ ((row >> 1) & 7u);
-        voff[j] = row * static_cast<uint32_t>(p.a_rs) * 2 + chunk * 16;
-        voff[8 + j] = row * static_cast<uint32_t>(p.b_cs) * 2 + chunk * 16;
+        voff[j] = row * static_cast<uint32_t>(j < LOADS_A ? p.a_rs : p.b_cs) * 2 + chunk * 16;
     }
     auto issue_load = [&](int j, uint32_t stage, uint32_t k_bytes) {
-        const uint32_t at = stage * STAGE_BYTES + (j < 8 ? 0 : TILE_BYTES) + (wave * 8 + (j & 7)) * 1024;
-        __builtin_amdgcn_raw_ptr_buffer_load_lds(j < 8 ? rsrc_a : rsrc_b, (lds_void)(lds_raw + at), 16, voff[j], k_bytes, 0, 0);
+        const uint32_t at = stage * (STAGE * 2) + (j < LOADS_A ? (wave * LOADS_A + j) * 1024 : A_TILE * 2 + (wave * LOADS_B + (j - LOADS_A)) * 1024);
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(j < LOADS_A ? rsrc_a : rsrc_b, (lds_void)(lds_raw + at), 16, voff[j], k_bytes, 0, 0);
     };
 
     float4v acc[TM][TN];
@@ -88,12 +95,32 @@ __global__ __launch_bounds__(256) void gemm16_dtl16_kernel(const T* A, const T* 
 #pragma unroll
         for (int j = 0; j < TN; ++j) acc[i][j] = float4v{0.0f, 0.0f, 0.0f, 0.0f};
 
+    // Tile loads complete in the order they were issued: waiting until at most AHEAD of them are outstanding leaves the
+    // tiles that are not needed yet in flight.
+    constexpr int AHEAD = (STAGES - 2) * LOADS;
+    auto wait_loads = [](bool all) {
+        if (all) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        else asm volatile("s_waitcnt vmcnt(%0)" ::"n"(AHEAD) : "memory");
+    };
+    // own LDS traffic done, then everybody's: no fence beyond that (a fence would also wait for the loads in flight)
+    auto meet = [] {
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+    };
+    // prologue: tiles 0 .. STAGES-2 into their stages
 #pragma unroll
-    for (int j = 0; j < 16; ++j) issue_load(j, 0, 0);
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    __syncthreads();
+    for (int t = 0; t < STAGES - 1; ++t) {
+        if (static_cast<uint32_t>(t) < steps) {
+#pragma unroll
+            for (int j = 0; j < LOADS; ++j) issue_load(j, t, t * (BK * 2));
+        }
+    }
+    wait_loads(steps < static_cast<uint32_t>(STAGES - 1));
+    meet();
 
-    constexpr int PER_KS = TM * TN;   // 64 MFMAs per k-slice
+    constexpr int PER_KS = TM * TN;   // MFMAs per k-slice
+    constexpr int LOAD_EVERY = PER_KS / LOADS > 0 ? PER_KS / LOADS : 1;   // the loads of a step go out during its first half
     uint4v fa[2][TM], fb[2][TN];
     auto read_fragments = [&](const T* a_tile, const T* b_tile, int ks, int into) {
 #pragma unroll
@@ -101,20 +128,20 @@ __global__ __launch_bounds__(256) void gemm16_dtl16_kernel(const T* A, const T* 
 #pragma unroll
         for (int y = 0; y < TN; ++y) fb[into][y] = *reinterpret_cast<const uint4v*>(b_tile + tile_offset<T>(wn + y * 16 + frag_row, ks * 4 + frag_chunk));
     };
-
-    // A step issues the MFMAs of the second k-slice of the previous tile (fragments in registers since before the
-    // barrier) and those of the first slice of this tile; the loads of the next tile go between the first of them.
-    // fragment read r of a k-slice: the B fragments and the first A fragment first, in the order the MFMAs want them
+    // fragment read r of a k-slice: the first A fragment and the B fragments first, in the order the MFMAs want them
     auto read_one = [&](const T* a_tile, const T* b_tile, int ks, int into, int r) {
         if (r == 0) fa[into][0] = *reinterpret_cast<const uint4v*>(a_tile + tile_offset<T>(wm + frag_row, ks * 4 + frag_chunk));
         else if (r <= TN) fb[into][r - 1] = *reinterpret_cast<const uint4v*>(b_tile + tile_offset<T>(wn + (r - 1) * 16 + frag_row, ks * 4 + frag_chunk));
         else fa[into][r - TN] = *reinterpret_cast<const uint4v*>(a_tile + tile_offset<T>(wm + (r - TN) * 16 + frag_row, ks * 4 + frag_chunk));
     };
-    auto step = [&](uint32_t s, auto first_tag, auto fetch_tag) {
+    // A step issues the MFMAs of the second k-slice of the previous tile (its fragments are in registers since before
+    // the barrier) and those of the first slice of this tile.  Behind the first MFMAs of each half go the fragment
+    // reads of the slice the NEXT half multiplies (their registers were last read by the half before this one), and,
+    // spread over the first half, the loads of the next tile.
+    auto step = [&](uint32_t s, uint32_t cur, uint32_t fill, auto first_tag, auto fetch_tag) {   // cur: stage of tile s; fill: stage tile s-1 has left
         constexpr bool FIRST = decltype(first_tag)::value, FETCH = decltype(fetch_tag)::value;
-        const uint32_t cur = s & 1;
-        const T* a_tile = lds + cur * 2 * TILE;
-        const T* b_tile = a_tile + TILE;
+        const T* a_tile = lds + cur * STAGE;
+        const T* b_tile = a_tile + A_TILE;
         // the first step has no MFMAs in its first half: its fragment reads go out at once
         if constexpr (FIRST) read_fragments(a_tile, b_tile, 0, 0);
         __builtin_amdgcn_sched_barrier(0);
@@ -124,34 +151,30 @@ __global__ __launch_bounds__(256) void gemm16_dtl16_kernel(const T* A, const T* 
             constexpr int q = m % PER_KS, i = q / TN, j = q % TN;
             constexpr int now = group == 0 ? 1 : 0;
             if constexpr (!(FIRST && group == 0)) mfma16x16_in_place<T>(acc[i][j], fb[now][j], fa[now][i]);
-            // behind the first 16 MFMAs of a half: the fragment reads of the slice the NEXT half multiplies (its registers were
-            // last read by the half before this one)
             if constexpr (q < TM + TN && !(FIRST && group == 0)) read_one(a_tile, b_tile, group == 0 ? 0 : 1, group == 0 ? 0 : 1, q);
             constexpr int slot = FIRST ? m - PER_KS : m;
-            if constexpr (FETCH && slot >= 0 && slot % LOAD_EVERY == LOAD_EVERY / 2 && slot / LOAD_EVERY < 16) issue_load(slot / LOAD_EVERY, cur ^ 1, (s + 1) * (BK * 2));
+            if constexpr (FETCH && slot >= 0 && slot % LOAD_EVERY == LOAD_EVERY / 2 && slot / LOAD_EVERY < LOADS) issue_load(slot / LOAD_EVERY, fill, (s + STAGES - 1) * (BK * 2));
             __builtin_amdgcn_sched_barrier(0);
         });
-        if constexpr (FETCH) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        __syncthreads();
+        wait_loads(!FETCH);    // tile s+1 is in LDS (steps that issue no loads wait for all that are left)
+        meet();
     };
     using Yes = std::true_type;
     using No = std::false_type;
-    if (steps == 1) {
-        step(0, Yes{}, No{});
-    } else {
-        step(0, Yes{}, Yes{});
-        uint32_t s = 1;
-        for (; s + 1 < steps; ++s) step(s, No{}, Yes{});
-        step(s, No{}, No{});
-    }
+    auto next = [](uint32_t stage) { return stage + 1 == STAGES ? 0u : stage + 1; };
+    uint32_t s = 0, cur = 0, fill = STAGES - 1;
+    if (steps > STAGES - 1) step(0, cur, fill, Yes{}, Yes{});
+    else step(0, cur, fill, Yes{}, No{});
+    for (s = 1, cur = next(cur), fill = next(fill); s + STAGES - 1 < steps; ++s, cur = next(cur), fill = next(fill)) step(s, cur, fill, No{}, Yes{});
+    for (; s < steps; ++s, cur = next(cur), fill = next(fill)) step(s, cur, fill, No{}, No{});
     // the second slice of the last tile
 #pragma unroll
     for (int i = 0; i < TM; ++i)
 #pragma unroll
         for (int j = 0; j < TN; ++j) mfma16x16_in_place<T>(acc[i][j], fb[1][j], fa[1][i]);
 
-    // Each wavefront rounds its 128 x 128 block into its own LDS area (no operand tile is read after the last barrier)
-    // and writes it out as whole rows, 16 bytes per lane.
+    // Each wavefront rounds its block into its own LDS area (no operand tile is read after the last barrier) and
+    // writes it out as whole rows, 16 bytes per lane.
     T* c = C + oc;
     constexpr int PITCH = WN + 8;
     T* stage = lds + wave * (WM * PITCH);
@@ -174,23 +197,25 @@ __global__ __launch_bounds__(256) void gemm16_dtl16_kernel(const T* A, const T* 
         const uint4v bits = *reinterpret_cast<const uint4v*>(stage + r * PITCH + (lane % LANES_PER_ROW) * 8);
         if (row < p.M && col < p.N) *reinterpret_cast<uint4v*>(c + static_cast<int64_t>(row) * p.c_rs + col) = bits;
     }
+#endif
 }
 
-template <class T, int LOAD_EVERY>
-static int launch_dtl16(const GemmProblem& p, const void* a, const void* b, void* c, hipStream_t stream) {
-    const uint32_t tiles_m = (p.M + 255) / 256, tiles_n = (p.N + 255) / 256;
-    constexpr size_t lds_bytes = 2 * 4 * 128 * (128 + 8);
-    auto kernel = gemm16_dtl16_kernel<T, LOAD_EVERY>;
+template <class T, int BM, int BN, int STAGES>
+static int launch_dtl(const GemmProblem& p, const void* a, const void* b, void* c, hipStream_t stream) {
+    const uint32_t tiles_m = (p.M + BM - 1) / BM, tiles_n = (p.N + BN - 1) / BN;
+    constexpr size_t tile_bytes = STAGES * (BM + BN) * 128, stage_bytes = 2 * 4 * (BM / 2) * (BN / 2 + 8);   // the operand stages; the output staging
+    constexpr size_t lds_bytes = tile_bytes > stage_bytes ? tile_bytes : stage_bytes;
+    auto kernel = gemm16_dtl_kernel<T, BM, BN, STAGES, (lds_bytes <= 80 * 1024 ? 2 : 1)>;
     static std::atomic<uint64_t> configured{0};
     if (int rc = raise_lds_limit(reinterpret_cast<const void*>(kernel), lds_bytes, configured)) return rc;
     hipLaunchKernelGGL(kernel, dim3(tiles_m * tiles_n, p.batches), dim3(256), lds_bytes, stream, static_cast<const T*>(a), static_cast<const T*>(b),
                        static_cast<T*>(c), p, tiles_m, tiles_n);
-    return launch_status("gemm16_dtl16_kernel");
+    return launch_status("gemm16_dtl_kernel");
 }
 
 // Returns TANNIC_UNSUPPORTED_DTYPE when the problem is not this kernel's: the caller then takes the register-staged one.
 template <class T>
-int gemm16_dtl(const GemmProblem& p, const void* a, const void* b, void* c, hipStream_t stream) {
+int gemm16_dtl(const GemmProblem& p, int bm, int bn, const void* a, const void* b, void* c, hipStream_t stream) {
     if (p.a_cs != 1 || p.b_rs != 1) return TANNIC_UNSUPPORTED_DTYPE;                     // both operands K-contiguous
     if (p.K == 0 || p.K % 64 != 0 || p.row_bias) return TANNIC_UNSUPPORTED_DTYPE;         // whole K steps only, no start values
     if (p.N % 8 != 0 || p.c_rs % 8 != 0 || reinterpret_cast<uintptr_t>(c) % 16 != 0) return TANNIC_UNSUPPORTED_DTYPE;
@@ -199,10 +224,14 @@ int gemm16_dtl(const GemmProblem& p, const void* a, const void* b, void* c, hipS
     // a row's offset inside a tile is a 32-bit byte count; rows must not overlap (the range check relies on it)
     if (p.a_rs < static_cast<int64_t>(p.K) || p.b_cs < static_cast<int64_t>(p.K)) return TANNIC_UNSUPPORTED_DTYPE;
     if (p.a_rs >= (1 << 22) || p.b_cs >= (1 << 22)) return TANNIC_UNSUPPORTED_DTYPE;
-    return launch_dtl16<T, 4>(p, a, b, c, stream);
+    // as many stages as LDS holds (160 KB): the smaller the tile, the shorter its step and the more steps a load needs to arrive
+    if (bm == 256 && bn == 256) return launch_dtl<T, 256, 256, 2>(p, a, b, c, stream);
+    if (bm == 256 && bn == 128) return launch_dtl<T, 256, 128, 3>(p, a, b, c, stream);
+    if (bm == 128 && bn == 128) return launch_dtl<T, 128, 128, 4>(p, a, b, c, stream);
+    return TANNIC_UNSUPPORTED_DTYPE;
 }
 
-template int gemm16_dtl<f16>(const GemmProblem&, const void*, const void*, void*, hipStream_t);
-template int gemm16_dtl<bf16>(const GemmProblem&, const void*, const void*, void*, hipStream_t);
+template int gemm16_dtl<f16>(const GemmProblem&, int, int, const void*, const void*, void*, hipStream_t);
+template int gemm16_dtl<bf16>(const GemmProblem&, int, int, const void*, const void*, void*, hipStream_t);
 
 }  // namespace th

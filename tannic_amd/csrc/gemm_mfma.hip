@@ -553,11 +553,8 @@ int run16(const GemmProblem& p, const void* a, const void* b, void* c, hipStream
     const uint64_t big = static_cast<uint64_t>((p.M + 255) / 256) * ((p.N + 255) / 256) * p.batches;
     if (p.M > 192 && big >= 200) {
         if constexpr (sizeof(T) == 2) {
-            static const bool direct = [] { const char* e = getenv("TANNIC_GEMM_DTL"); return !e || atoi(e) != 0; }();
-            if (direct) {
-                const int rc = gemm16_dtl<T>(p, a, b, c, stream);
-                if (rc != TANNIC_UNSUPPORTED_DTYPE) return rc;
-            }
+            const int rc = gemm16_dtl<T>(p, 256, 256, a, b, c, stream);
+            if (rc != TANNIC_UNSUPPORTED_DTYPE) return rc;
         }
         return pick_layout16<T, 256, 256, 2>(p, ak, bk, a, b, c, stream);
     }
@@ -588,6 +585,12 @@ int run16(const GemmProblem& p, const void* a, const void* b, void* c, hipStream
     if (best_splits > 1) {
         if (best_bm == 128) return run16_split<T, 128>(p, ak, bk, best_splits, a, b, c, stream, workspace);
         return run16_split<T, 64>(p, ak, bk, best_splits, a, b, c, stream, workspace);
+    }
+    if constexpr (sizeof(T) == 2) {
+        if (best_bm >= 128) {
+            const int rc = gemm16_dtl<T>(p, best_bm, 128, a, b, c, stream);
+            if (rc != TANNIC_UNSUPPORTED_DTYPE) return rc;
+        }
     }
     if (best_bm == 256) return pick_layout16<T, 256, 128, 2>(p, ak, bk, a, b, c, stream);
     if (best_bm == 128) return pick_layout16<T, 128, 128, 2>(p, ak, bk, a, b, c, stream);
