@@ -5,7 +5,7 @@ the libraries under oracle/.
 """
 import ctypes as C
 import os
-import subprocess
+import sys
 
 import numpy as np
 
@@ -14,47 +14,10 @@ from tannic_amd import abi, types
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 ORACLE_DIR = os.path.join(ROOT, "oracle")
+sys.path.insert(0, ORACLE_DIR)
 
 
-class HostLibrary:
-    """A library of stream-less entry points with a common prefix."""
-
-    def __init__(self, path, prefix):
-        self.path = path
-        self.cdll = C.CDLL(path)
-        self.functions = {}
-        for name, (res, args) in abi.kernel_signatures(with_stream=False).items():
-            try:
-                fn = getattr(self.cdll, prefix + name)
-            except AttributeError:
-                continue
-            fn.restype, fn.argtypes = res, args
-            self.functions[name] = fn
-
-    def set_accumulate(self, wide):
-        self.cdll.oracle_set_accumulate(1 if wide else 0)
-
-
-_oracle = None
-_reference = False
-
-
-def oracle_library():
-    global _oracle
-    if _oracle is None:
-        path = os.path.join(ORACLE_DIR, "liboracle.so")
-        if not os.path.exists(path):
-            subprocess.run(["make", "-C", ORACLE_DIR, "liboracle.so"], check=True, capture_output=True)
-        _oracle = HostLibrary(path, "oracle_")
-    return _oracle
-
-
-def reference_library():
-    global _reference
-    if _reference is False:
-        path = os.path.join(ORACLE_DIR, "_ref", "libtannic_ref.so")
-        _reference = HostLibrary(path, "ref_") if os.path.exists(path) else None
-    return _reference
+from host_library import HostLibrary, oracle_library, reference_library  # noqa: E402,F401
 
 
 class use_functions:
@@ -71,54 +34,8 @@ class use_functions:
         ta.ops.set_host_functions(self.previous)
 
 
-# ---- seeded inputs: counter-based, identical on every host -----------------
-def _splitmix64(x):
-    x = (x + np.uint64(0x9E3779B97F4A7C15))
-    z = x
-    z = (z ^ (z >> np.uint64(30))) * np.uint64(0xBF58476D1CE4E5B9)
-    z = (z ^ (z >> np.uint64(27))) * np.uint64(0x94D049BB133111EB)
-    return z ^ (z >> np.uint64(31))
-
-
-def random_bits(seed, tensor_id, n):
-    with np.errstate(over="ignore"):
-        base = _splitmix64(np.uint64(seed) * np.uint64(0x100000001B3) + np.uint64(tensor_id))
-        return _splitmix64(base + np.arange(n, dtype=np.uint64))
-
-
-def uniform(seed, tensor_id, shape, low=-1.0, high=1.0):
-    n = int(np.prod(shape, dtype=np.int64))
-    u = (random_bits(seed, tensor_id, n) >> np.uint64(40)).astype(np.float64) * 2.0 ** -24
-    return (low + (high - low) * u).astype(np.float32).reshape(shape)
-
-
-def normal(seed, tensor_id, shape, sigma=1.0):
-    n = int(np.prod(shape, dtype=np.int64))
-    bits = random_bits(seed, tensor_id, 2 * n)
-    u1 = ((bits[:n] >> np.uint64(11)).astype(np.float64) + 1.0) * 2.0 ** -53
-    u2 = (bits[n:] >> np.uint64(11)).astype(np.float64) * 2.0 ** -53
-    z = np.sqrt(-2.0 * np.log(u1)) * np.cos(2.0 * np.pi * u2)
-    return (sigma * z).astype(np.float32).reshape(shape)
-
-
-def integers(seed, tensor_id, shape, low=-4, high=4):
-    return np.floor(uniform(seed, tensor_id, shape, low, high)).astype(np.int64)
-
-
-def values_for(dtype, seed, tensor_id, shape, low=-4.0, high=4.0):
-    """Seeded values representable in ``dtype`` (as a numeric numpy array)."""
-    if dtype.is_integral:
-        return integers(seed, tensor_id, shape, int(low), int(high)).astype(dtype.storage)
-    if dtype.is_complex:
-        re = uniform(seed, tensor_id, shape, low, high)
-        im = uniform(seed, tensor_id + 7919, shape, low, high)
-        return (re + 1j * im).astype(dtype.storage)
-    x = uniform(seed, tensor_id, shape, low, high)
-    if dtype is types.float16:
-        return x.astype(np.float16)
-    if dtype is types.bfloat16:
-        return types.bfloat16_bits_to_float32(types.float32_to_bfloat16_bits(x))
-    return x.astype(dtype.storage)
+# ---- seeded inputs (tannic_amd.synthetic) -----------------
+from tannic_amd.synthetic import random_bits, uniform, normal, integers, values_for  # noqa: E402,F401
 
 
 def host_tensor(values, dtype):
