@@ -92,11 +92,17 @@ def split_heads(t, heads):
     return t._view((b, seq, heads, d), (t.strides[0], t.strides[1], d, 1)).transpose(1, 2)
 
 
-def forward_fused(s, w, x, cos, sin, mask):
+def _keep(trace, **stages):
+    """Records intermediate tensors by name when a caller asked for them (tests check every stage by itself)."""
+    if trace is not None:
+        trace.update(stages)
+
+
+def forward_fused(s, w, x, cos, sin, mask, trace=None):
     """The same layer with the device library's one-pass operators (``ops.rms_norm``, ``ops.rope``, ``ops.softmax``,
     ``ops.swiglu``) in place of the chains; these have no counterpart in the reference's front end.  With the
     concatenated parameters of ``pack_weights`` the q/k/v and the gate/up projections are one product each and their
-    parts are column slices of its result."""
+    parts are column slices of its result.  ``trace``: a dictionary that receives the intermediate tensors."""
     _, seq, _ = x.shape
     nq, nkv = s.heads * s.head_dim, s.kv_heads * s.head_dim
     xn = ops.rms_norm(x, w["g1"], s.eps)
@@ -105,45 +111,59 @@ def forward_fused(s, w, x, cos, sin, mask):
         q, k, v = qkv[..., 0:nq], qkv[..., nq:nq + nkv], qkv[..., nq + nkv:nq + 2 * nkv]
     else:
         q, k, v = (ops.matmul(xn, w[name].transpose()) for name in ("wq", "wk", "wv"))
+    _keep(trace, xn=xn, q=q, k=k, v=v)
     q, k, v = split_heads(q, s.heads), split_heads(k, s.kv_heads), split_heads(v, s.kv_heads)
     q, k = ops.rope(q, cos, sin), ops.rope(k, cos, sin)
+    _keep(trace, q_rot=q, k_rot=k)
     group = s.heads // s.kv_heads
     k, v = ops.repeat(k, group, 1), ops.repeat(v, group, 1)
-    p = ops.softmax(ops.matmul(q, k.transpose(-1, -2)), mask, 1.0 / math.sqrt(s.head_dim))
-    o = ops.repack(ops.matmul(p, v).transpose(1, 2)).view(1, seq, s.heads * s.head_dim)
+    scores = ops.matmul(q, k.transpose(-1, -2))
+    p = ops.softmax(scores, mask, 1.0 / math.sqrt(s.head_dim))
+    pv = ops.matmul(p, v)
+    o = ops.repack(pv.transpose(1, 2)).view(1, seq, s.heads * s.head_dim)
     h = ops.add(x, ops.matmul(o, w["wo"].transpose()))
     hn = ops.rms_norm(h, w["g2"], s.eps)
     if "w13" in w:
         both = ops.matmul(hn, w["w13"].transpose())
-        act = ops.swiglu(both[..., 0:s.ffn], both[..., s.ffn:2 * s.ffn])
+        gate, up = both[..., 0:s.ffn], both[..., s.ffn:2 * s.ffn]
     else:
-        act = ops.swiglu(ops.matmul(hn, w["w1"].transpose()), ops.matmul(hn, w["w3"].transpose()))
-    return ops.add(h, ops.matmul(act, w["w2"].transpose()))
+        gate, up = ops.matmul(hn, w["w1"].transpose()), ops.matmul(hn, w["w3"].transpose())
+    act = ops.swiglu(gate, up)
+    y = ops.matmul(act, w["w2"].transpose())
+    out = ops.add(h, y)
+    _keep(trace, k_all=k, v_all=v, scores=scores, p=p, pv=pv, o=o, h=h, hn=hn, gate=gate, up=up, act=act, y=y, out=out)
+    return out
 
 
-def forward(s, w, x, cos, sin, mask, one):
-    """x: [1, seq, hidden].  Returns the layer's output, same shape and dtype."""
+def forward(s, w, x, cos, sin, mask, one, trace=None):
+    """x: [1, seq, hidden].  Returns the layer's output, same shape and dtype.  ``trace``: a dictionary that receives
+    the intermediate tensors."""
     _, seq, _ = x.shape
     xn = rms_norm(x, w["g1"], s.eps)
     q = ops.matmul(xn, w["wq"].transpose())
     k = ops.matmul(xn, w["wk"].transpose())
     v = ops.matmul(xn, w["wv"].transpose())
+    _keep(trace, xn=xn, q=q, k=k, v=v)
     q = q.view(1, seq, s.heads, s.head_dim).transpose(1, 2)
     k = k.view(1, seq, s.kv_heads, s.head_dim).transpose(1, 2)
     v = v.view(1, seq, s.kv_heads, s.head_dim).transpose(1, 2)
     q, k = rope(q, cos, sin), rope(k, cos, sin)
+    _keep(trace, q_rot=q, k_rot=k)
     group = s.heads // s.kv_heads
     k, v = ops.repeat(k, group, 1), ops.repeat(v, group, 1)
     scores = ops.scale(ops.matmul(q, k.transpose(-1, -2)), 1.0 / math.sqrt(s.head_dim))
     p = softmax_rows(ops.add(scores, mask))
-    o = ops.matmul(p, v)
-    o = ops.repack(o.transpose(1, 2)).view(1, seq, s.heads * s.head_dim)
+    pv = ops.matmul(p, v)
+    o = ops.repack(pv.transpose(1, 2)).view(1, seq, s.heads * s.head_dim)
     h = ops.add(x, ops.matmul(o, w["wo"].transpose()))
     hn = rms_norm(h, w["g2"], s.eps)
     gate = ops.matmul(hn, w["w1"].transpose())
     up = ops.matmul(hn, w["w3"].transpose())
-    y = ops.matmul(ops.mul(silu(gate, one), up), w["w2"].transpose())
-    return ops.add(h, y)
+    act = ops.mul(silu(gate, one), up)
+    y = ops.matmul(act, w["w2"].transpose())
+    out = ops.add(h, y)
+    _keep(trace, k_all=k, v_all=v, scores=scores, p=p, pv=pv, o=o, h=h, hn=hn, gate=gate, up=up, act=act, y=y, out=out)
+    return out
 
 
 def flop_count(s, seq):

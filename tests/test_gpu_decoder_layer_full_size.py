@@ -1,0 +1,229 @@
+"""The decoder layer at its real size: hidden 4096, 32 query / 8 key-value heads of 128, FFN 14336, 512 positions, bf16.
+
+At this size the matrix products take other kernels than in the small layer of test_gpu_decoder_layer.py (tiles of
+256 x 128 and 128 x 128 filled by direct global -> LDS loads, K shared between workgroups for the 4096-wide
+projections, batched products of 32 heads) and the row kernels other row lengths, so every STAGE of the layer is
+checked by itself, from the inputs the device itself fed to that stage (errors of earlier stages do not add up):
+
+  (1) the CPU checker on slices it can finish: rows of each projection, whole heads of the attention, the
+      elementwise chains in full where they are cheap (those are bit-exact or within the rounding of a sum's order);
+  (2) float64 numpy on more of each stage, with a bar of a few bf16 roundings of that stage's own chain;
+  (3) properties: probabilities of later positions are exactly zero and rows sum to one, changing a later position
+      leaves earlier outputs untouched bit for bit, the layer with concatenated q/k/v and gate/up parameters gives
+      the layer with separate ones.
+"""
+import gc
+import math
+
+import numpy as np
+import pytest
+
+import support
+import tannic_amd as ta
+from tannic_amd import decoder_layer as dl
+from tannic_amd import ops, types
+
+pytestmark = pytest.mark.gpu
+SEQ = 512
+ULP = 2.0 ** -7      # bf16 keeps 8 significant bits: neighbouring values are at most this far apart, relatively
+BLOCK = 1 << 22
+
+
+def bf16(values):
+    """Values rounded to bf16, as float32 numbers."""
+    return types.bfloat16_bits_to_float32(types.float32_to_bfloat16_bits(np.asarray(values, dtype=np.float32)))
+
+
+def drawn(kind, tensor_id, shape, scale):
+    n = int(np.prod(shape))
+    period = min(n, BLOCK)
+    base = support.normal(0, tensor_id, (period,), scale) if kind == "normal" else support.uniform(0, tensor_id, (period,), 0.5, 1.5)
+    return np.resize(bf16(base), n).reshape(shape)
+
+
+@pytest.fixture(scope="module")
+def layer(device, oracle):
+    """Parameters, input and the traced intermediate tensors of both forms of the layer (computed once)."""
+    s = dl.LayerShape()
+    values = {}
+    for i, (name, shape) in enumerate(dl.weight_shapes(s).items()):
+        values[name] = drawn("gain", 40 + i, shape, 1.0) if name.startswith("g") else drawn("normal", 40 + i, shape, 0.02)
+    x = drawn("normal", 39, (1, SEQ, s.hidden), 1.0)
+    w = {k: ta.tensor(v, ta.bfloat16, device) for k, v in values.items()}
+    dx = ta.tensor(x, ta.bfloat16, device)
+    cos, sin = dl.rotary_tables(s, SEQ, ta.bfloat16, device)
+    mask, one = dl.causal_mask(SEQ, ta.bfloat16, device), ta.tensor(np.ones(1), ta.bfloat16, device)
+    composed, fused = {}, {}
+    dl.forward(s, w, dx, cos, sin, mask, one, composed)
+    packed = dl.pack_weights(w)
+    dl.forward_fused(s, packed, dx, cos, sin, mask, fused)
+    yield {"s": s, "values": values, "x": x, "w": w, "packed": packed, "dx": dx, "cos": cos, "sin": sin, "mask": mask, "one": one,
+           "composed": composed, "fused": fused}
+    composed.clear()
+    fused.clear()
+    gc.collect()
+
+
+def numbers(t):
+    return t.numpy().astype(np.float64)
+
+
+def host(values):
+    return ta.tensor(values, ta.bfloat16, ta.Host())
+
+
+def rms64(v, gain, eps):
+    return v / np.sqrt((v * v).mean(-1, keepdims=True) + eps) * gain
+
+
+ROWS = [0, 255, 511]
+
+
+def check_projection(got, a, w, what, every=16):
+    """got = a . w^T (bf16, fp32 accumulation): the checker on three rows, float64 on every `every`-th row."""
+    want = ops.matmul(host(a[ROWS]), host(w).transpose()).numpy()
+    support.assert_close(got[ROWS], want, ULP, 1e-3, f"{what}: checker rows")
+    band = np.arange(0, a.shape[0], every)
+    exact = a[band].astype(np.float64) @ w.astype(np.float64).T
+    support.assert_close(got[band], exact, ULP, 1e-3, f"{what}: float64 rows")
+
+
+@pytest.mark.parametrize("form", ["composed", "fused"])
+def test_normalisation_and_projections(layer, form):
+    s, t, v = layer["s"], layer[form], layer["values"]
+    x = layer["x"][0].astype(np.float64)
+    xn = numbers(t["xn"])[0]
+    # the chain rounds five times (square, mean, rsqrt, two products), the one-pass operator once
+    support.assert_close(xn, rms64(x, v["g1"].astype(np.float64), s.eps), (4 if form == "composed" else 1.01) * ULP, 1e-6, f"{form} rms_norm")
+    if form == "composed":
+        want = dl.rms_norm(host(layer["x"][:, ROWS]), host(v["g1"]), s.eps).numpy()[0]
+        support.assert_close(xn[ROWS], want, ULP, 1e-6, "rms_norm chain against the checker (a sum's order apart)")
+    xn_bf = xn.astype(np.float32)
+    for name, weight in (("q", "wq"), ("k", "wk"), ("v", "wv")):
+        check_projection(numbers(t[name])[0], xn_bf, v[weight], f"{form} {name} projection")
+
+
+@pytest.mark.parametrize("form", ["composed", "fused"])
+def test_rotary_embedding_and_head_repetition(layer, form):
+    s, t = layer["s"], layer[form]
+    cos, sin = numbers(layer["cos"]), numbers(layer["sin"])
+    for name, heads in (("q", s.heads), ("k", s.kv_heads)):
+        flat = numbers(t[name])[0]                                                   # [seq, heads * d]
+        src = flat.reshape(SEQ, heads, s.head_dim).transpose(1, 0, 2)                # [heads, seq, d]
+        even, odd = src[..., 0::2], src[..., 1::2]
+        got = numbers(t[name + "_rot"])[0]
+        if form == "composed":
+            # every product and sum of the chain is rounded to bf16: restated here, bit for bit
+            re = bf16(bf16(even * cos) - bf16(odd * sin))
+            im = bf16(bf16(even * sin) + bf16(odd * cos))
+            np.testing.assert_array_equal(got[..., 0::2], re)
+            np.testing.assert_array_equal(got[..., 1::2], im)
+        else:
+            support.assert_close(got[..., 0::2], even * cos - odd * sin, 1.01 * ULP, 2.0 ** -9 * np.abs(src).max(), "rope, real parts")
+            support.assert_close(got[..., 1::2], even * sin + odd * cos, 1.01 * ULP, 2.0 ** -9 * np.abs(src).max(), "rope, imaginary parts")
+    group = s.heads // s.kv_heads
+    np.testing.assert_array_equal(numbers(t["k_all"])[0], np.repeat(numbers(t["k_rot"])[0], group, axis=0))
+    v_heads = numbers(t["v"])[0].reshape(SEQ, s.kv_heads, s.head_dim).transpose(1, 0, 2)
+    np.testing.assert_array_equal(numbers(t["v_all"])[0], np.repeat(v_heads, group, axis=0))
+
+
+@pytest.mark.parametrize("form", ["composed", "fused"])
+def test_attention(layer, form):
+    s, t = layer["s"], layer[form]
+    q, k, v = numbers(t["q_rot"])[0], numbers(t["k_all"])[0], numbers(t["v_all"])[0]     # [32, 512, 128]
+    scale = 1.0 / math.sqrt(s.head_dim)
+    scores = numbers(t["scores"])[0]
+    raw = q @ k.transpose(0, 2, 1)
+    if form == "composed":
+        # product rounded to bf16, then scaled by the bf16 value of 1/sqrt(128) and rounded again
+        support.assert_close(scores, raw * float(np.ravel(bf16(scale))[0]), 2 * ULP, 1e-3, "scores (all heads, float64)")
+        for head in (0, 31):
+            want = ops.scale(ops.matmul(host(q[head][None].astype(np.float32)), host(k[head][None].astype(np.float32)).transpose(-1, -2)), scale).numpy()[0]
+            support.assert_close(scores[head], want, ULP, 1e-3, f"scores of head {head} against the checker")
+    else:
+        support.assert_close(scores, raw, ULP, 1e-3, "scores before scaling (all heads, float64)")
+    p = numbers(t["p"])[0]
+    upper = np.triu(np.ones((SEQ, SEQ), dtype=bool), 1)
+    assert (p[:, upper] == 0).all(), "a position attends to a later one"
+    logits = np.where(upper, -np.inf, scores if form == "composed" else scores * scale)
+    e = np.exp(logits - logits.max(-1, keepdims=True))
+    exact = e / e.sum(-1, keepdims=True)
+    # chain: the difference to the row maximum, exp, sum, rsqrt and two products are each rounded to bf16 (the rounding of
+    # the difference is an absolute error of the exponent, so it grows with the distance to the maximum); one-pass: one rounding
+    distance = np.where(upper, 0.0, logits.max(-1, keepdims=True) - np.where(upper, 0.0, logits))
+    allowed = ((5 * ULP + distance * ULP) if form == "composed" else 1.01 * ULP) * exact + 1e-30
+    worst = np.abs(p - exact) - allowed
+    assert worst.max() <= 0, f"{form} softmax (float64): off by {np.abs(p - exact).max()} at {np.unravel_index(worst.argmax(), worst.shape)}"
+    assert np.abs(p.sum(-1) - 1.0).max() <= (8 if form == "composed" else 2) * ULP
+    pv = numbers(t["pv"])[0]
+    support.assert_close(pv, p @ v, ULP, 1e-3, "probabilities . values (all heads, float64)")
+    if form == "composed":
+        for head in (0, 31):
+            want = ops.matmul(host(p[head][None].astype(np.float32)), host(v[head][None].astype(np.float32))).numpy()[0]
+            support.assert_close(pv[head], want, ULP, 1e-3, f"head {head} against the checker")
+    np.testing.assert_array_equal(numbers(t["o"])[0], pv.transpose(1, 0, 2).reshape(SEQ, s.heads * s.head_dim))
+
+
+@pytest.mark.parametrize("form", ["composed", "fused"])
+def test_output_projection_and_feed_forward(layer, form):
+    s, t, v = layer["s"], layer[form], layer["values"]
+    x = layer["x"][0].astype(np.float64)
+    o = numbers(t["o"])[0].astype(np.float32)
+    h = numbers(t["h"])[0]
+    # h = x + o . wo^T: the product is rounded to bf16, then the sum
+    band = np.arange(0, SEQ, 16)
+    proj = bf16(o[band].astype(np.float64) @ v["wo"].astype(np.float64).T).astype(np.float64)
+    support.assert_close(h[band], x[band] + proj, ULP, ULP * np.abs(proj).max(), "residual after attention (float64)")
+    want = ops.add(host(layer["x"][:, ROWS]), ops.matmul(host(o[ROWS][None]), host(v["wo"]).transpose())).numpy()[0]
+    support.assert_close(h[ROWS], want, ULP, ULP * np.abs(proj).max(), "residual after attention against the checker")
+    hn = numbers(t["hn"])[0]
+    support.assert_close(hn, rms64(h, v["g2"].astype(np.float64), s.eps), (4 if form == "composed" else 1.01) * ULP, 1e-6, f"{form} second rms_norm")
+    hn_bf = hn.astype(np.float32)
+    gate, up = numbers(t["gate"])[0], numbers(t["up"])[0]
+    check_projection(gate, hn_bf, v["w1"], f"{form} gate projection", every=32)
+    check_projection(up, hn_bf, v["w3"], f"{form} up projection", every=32)
+    act = numbers(t["act"])[0]
+    exact = gate / (1.0 + np.exp(-gate)) * up
+    # chain: neg, exp, +1, rsqrt, three products, each rounded; one-pass: one rounding
+    support.assert_close(act, exact, (7 if form == "composed" else 1.01) * ULP, 1e-6, f"{form} SwiGLU (float64)")
+    if form == "composed":
+        g3, u3 = host(gate[ROWS][None].astype(np.float32)), host(up[ROWS][None].astype(np.float32))
+        want = ops.mul(dl.silu(g3, host(np.ones(1))), u3).numpy()[0]
+        support.assert_close(act[ROWS], want, 2 * ULP, 1e-6, "SwiGLU chain against the checker (exp and rsqrt within one rounding)")
+    y = numbers(t["y"])[0]
+    check_projection(y, act.astype(np.float32), v["w2"], f"{form} down projection", every=32)
+    np.testing.assert_array_equal(numbers(t["out"])[0], bf16(h + y))
+
+
+def test_both_forms_and_both_parameter_layouts_agree(layer):
+    """The one-pass operators round once where the chains round several times: the outputs differ by a few roundings of
+    the intermediate values, which the second normalisation and the products spread; the layer with concatenated
+    parameters multiplies the same numbers in the same order of k, so its projections are those of the separate ones."""
+    s = layer["s"]
+    composed, fused = numbers(layer["composed"]["out"]), numbers(layer["fused"]["out"])
+    assert np.isfinite(composed).all() and np.isfinite(fused).all()
+    spread = composed.std()
+    # (measured: 0.087 of the output's spread at most, 0.010 on average; every stage is checked by itself above)
+    assert np.abs(composed - fused).max() <= 0.15 * spread, (np.abs(composed - fused).max(), spread)
+    assert np.abs(composed - fused).mean() <= 0.02 * spread, (np.abs(composed - fused).mean(), spread)
+    separate = {}
+    dl.forward_fused(s, layer["w"], layer["dx"], layer["cos"], layer["sin"], layer["mask"], separate)
+    for name in ("q", "k", "v", "gate", "up"):
+        support.assert_close(numbers(separate[name]), numbers(layer["fused"][name]), ULP, 1e-3, f"{name}: concatenated against separate parameters")
+    support.assert_close(numbers(separate["out"]), fused, 4 * ULP, 0.02 * spread, "layer: concatenated against separate parameters")
+
+
+@pytest.mark.parametrize("form", ["composed", "fused"])
+def test_full_size_layer_is_causal(layer, device, form):
+    """Changing positions 300.. must leave outputs 0..299 untouched, bit for bit."""
+    s = layer["s"]
+    changed = layer["x"].copy()
+    changed[0, 300:] = bf16(changed[0, 300:] + 1.0)
+    dx = ta.tensor(changed, ta.bfloat16, device)
+    if form == "composed":
+        again = dl.forward(s, layer["w"], dx, layer["cos"], layer["sin"], layer["mask"], layer["one"]).numpy()
+    else:
+        again = dl.forward_fused(s, layer["packed"], dx, layer["cos"], layer["sin"], layer["mask"]).numpy()
+    before = layer[form]["out"].numpy()
+    np.testing.assert_array_equal(again[0, :300], before[0, :300])
+    assert np.abs(again[0, 300:].astype(np.float64) - before[0, 300:].astype(np.float64)).max() > 1e-2
