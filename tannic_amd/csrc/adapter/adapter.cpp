@@ -113,11 +113,20 @@ status concat(const tensor_t* a, const tensor_t* b, tensor_t* d, stream_t q, int
 status triu(const tensor_t* s, tensor_t* d, stream_t q, int k) { return static_cast<status>(tannic_hip_triu(in(s), out(d), st(q), k)); }
 status tril(const tensor_t* s, tensor_t* d, stream_t q, int k) { return static_cast<status>(tannic_hip_tril(in(s), out(d), st(q), k)); }
 
+#define TH_CMP(name) status name(const tensor_t* a, const tensor_t* b, tensor_t* d, stream_t q) { return code(tannic_hip_##name(in(a), in(b), out(d), st(q))); }
+TH_CMP(eq) TH_CMP(ne) TH_CMP(gt) TH_CMP(ge) TH_CMP(lt) TH_CMP(le)
+
 }  // namespace cuda
 
 namespace tannic_hip {
-#define TH_CMP(name) status name(const tensor_t* a, const tensor_t* b, tensor_t* d, stream_t q) { return code(tannic_hip_##name(in(a), in(b), out(d), st(q))); }
-TH_CMP(eq) TH_CMP(ne) TH_CMP(gt) TH_CMP(ge) TH_CMP(lt) TH_CMP(le)
 status max(const tensor_t* s, tensor_t* d, stream_t q, uint8_t axis) { return code(tannic_hip_max(in(s), out(d), st(q), axis)); }
 status min(const tensor_t* s, tensor_t* d, stream_t q, uint8_t axis) { return code(tannic_hip_min(in(s), out(d), st(q), axis)); }
+status div(const tensor_t* a, const tensor_t* b, tensor_t* d, stream_t q) { return code(tannic_hip_div(in(a), in(b), out(d), st(q))); }
+status swiglu(const tensor_t* a, const tensor_t* b, tensor_t* d, stream_t q) { return code(tannic_hip_swiglu(in(a), in(b), out(d), st(q))); }
+status cast(const tensor_t* s, tensor_t* d, stream_t q) { return code(tannic_hip_cast(in(s), out(d), st(q))); }
+status rms_norm(const tensor_t* x, const tensor_t* g, tensor_t* d, stream_t q, float eps) { return code(tannic_hip_rms_norm(in(x), in(g), out(d), st(q), eps)); }
+status softmax(const tensor_t* x, const tensor_t* mask, tensor_t* d, stream_t q, float scale) {
+    return code(tannic_hip_softmax(in(x), mask ? in(mask) : nullptr, out(d), st(q), scale));
+}
+status rope(const tensor_t* x, const tensor_t* c, const tensor_t* s, tensor_t* d, stream_t q) { return code(tannic_hip_rope(in(x), in(c), in(s), out(d), st(q))); }
 }  // namespace tannic_hip

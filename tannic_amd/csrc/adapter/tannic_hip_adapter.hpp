@@ -106,16 +106,29 @@ status tril(const tensor_t*, tensor_t*, stream_t, int k = 0);
 // cuda::eq..le itself, unconditionally (src/comparisons.cpp:18-29), so the
 // device twins cannot share those names.  A front end that wants them guards its
 // stubs with `#ifndef CUDA` and forwards to these.
-namespace tannic_hip {
-using tannic::status;
-using tannic::stream_t;
-using tannic::tensor_t;
+// Comparisons on the device.  The reference has no device kernels for them: src/comparisons.cpp:18-29 defines these six
+// as throwing stubs even in a device build, so a front end that links this backend needs those stubs put under
+// `#ifndef CUDA` (frontend.patch next to this header does that).
+namespace cuda {
 status eq(const tensor_t*, const tensor_t*, tensor_t*, stream_t);
 status ne(const tensor_t*, const tensor_t*, tensor_t*, stream_t);
 status gt(const tensor_t*, const tensor_t*, tensor_t*, stream_t);
 status ge(const tensor_t*, const tensor_t*, tensor_t*, stream_t);
 status lt(const tensor_t*, const tensor_t*, tensor_t*, stream_t);
 status le(const tensor_t*, const tensor_t*, tensor_t*, stream_t);
+}  // namespace cuda
+
+// Operators the reference's front end does not have (tannic_hip_functions.hpp builds expression nodes on them).
+namespace tannic_hip {
+using tannic::status;
+using tannic::stream_t;
+using tannic::tensor_t;
 status max(const tensor_t*, tensor_t*, stream_t, uint8_t axis);
 status min(const tensor_t*, tensor_t*, stream_t, uint8_t axis);
+status div(const tensor_t*, const tensor_t*, tensor_t*, stream_t);
+status swiglu(const tensor_t* gate, const tensor_t* up, tensor_t*, stream_t);
+status cast(const tensor_t*, tensor_t*, stream_t);
+status rms_norm(const tensor_t* x, const tensor_t* gain, tensor_t*, stream_t, float eps);
+status softmax(const tensor_t* x, const tensor_t* mask_or_null, tensor_t*, stream_t, float scale);
+status rope(const tensor_t* x, const tensor_t* cos, const tensor_t* sin, tensor_t*, stream_t);
 }  // namespace tannic_hip

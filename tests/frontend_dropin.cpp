@@ -4,6 +4,9 @@
 // once on Host (the reference's CPU kernels) and once on Device (this backend)
 // — and the two results are compared on the device with the front end's own
 // allclose (rtol = atol = 0 where the operation is exact on both sides).
+// The operators this backend adds (tannic_hip_functions.hpp: div, cast, max, min, softmax, rms_norm, swiglu, rope) have
+// no CPU twin: their device results are compared with plain loops written here.  Device comparisons and the copy of
+// a device tensor to the host go through the front end as patched by csrc/adapter/frontend.patch.
 //
 // This file is this repository's code; it is compiled against the reference's
 // headers and linked with the reference's front-end sources where they are
@@ -24,6 +27,9 @@
 #include "functions.hpp"
 #include "reductions.hpp"
 #include "transformations.hpp"
+#include "tannic_hip_functions.hpp"   // the operators this backend adds to the front end's surface
+
+#include <cmath>
 
 using namespace tannic;
 
@@ -60,6 +66,16 @@ static Tensor place(Tensor const& host, Environment env) {
     if (std::holds_alternative<Host>(env)) return host;
     return host.to(env);
 }
+
+// host float32 tensor filled by f(flat index)
+template <class F>
+static Tensor computed(Shape shape, F&& f) {
+    Tensor t(float32, shape);
+    t.initialize();
+    for (size_t i = 0; i < t.nelements(); ++i) reinterpret_cast<float*>(t.bytes())[i] = static_cast<float>(f(i));
+    return t;
+}
+static const float* values(Tensor const& host) { return reinterpret_cast<const float*>(host.bytes()); }
 
 int main() {
     if (Devices::count() < 1) {
@@ -121,7 +137,109 @@ int main() {
         {"conv1d k4 s2 p1", 1e-5, 1e-5, [&](Environment e) { return Tensor(convolve1D(place(Sig, e), place(W1, e), 2, 1)); }},
     };
 
+    // ---- operators without a CPU twin: the device against loops in double -----------------------------------------------
+    const Tensor G = seeded(float32, {32}, 22, 0.5, 1.5);
+    const Tensor Mask = computed({64, 32}, [](size_t i) { return (i % 32) > (i / 32) % 32 ? -INFINITY : 0.0; });
+    const Tensor Cs = computed({64, 16}, [](size_t i) { return std::cos(0.37 * (i / 16) / (1.0 + i % 16)); });
+    const Tensor Sn = computed({64, 16}, [](size_t i) { return std::sin(0.37 * (i / 16) / (1.0 + i % 16)); });
+    const float* x = values(X);
+    const float* pv = values(P);
+    const float* g = values(G);
+    struct DeviceOnly {
+        std::string name;
+        double rtol, atol;
+        std::function<Tensor()> device;      // evaluated on the device
+        std::function<Tensor()> expected;    // host tensor computed here
+    };
+    auto rows = [&](auto&& per_row) {   // X as 512 rows of 32
+        return computed({8, 64, 32}, [&, cache = std::vector<double>(32), row = size_t(-1)](size_t i) mutable {
+            if (i / 32 != row) { row = i / 32; per_row(x + row * 32, row, cache.data()); }
+            return cache[i % 32];
+        });
+    };
+    std::vector<DeviceOnly> added = {
+        {"div(X, P)", 1e-6, 0, [&] { return Tensor(div(X.to(Device()), P.to(Device()))); }, [&] { return computed({8, 64, 32}, [&](size_t i) { return x[i] / pv[i]; }); }},
+        {"div broadcast: X / Z", 1e-6, 0, [&] { return Tensor(div(X.to(Device()), Z.to(Device()))); },
+         [&] { return computed({8, 64, 32}, [&](size_t i) { return x[i] / values(Z)[(i / 32) % 64]; }); }},
+        {"cast int32 -> float32", 0, 0, [&] { return Tensor(cast(I.to(Device()), float32)); },
+         [&] { return computed({4, 9, 5}, [&](size_t i) { return reinterpret_cast<const int32_t*>(I.bytes())[i]; }); }},
+        {"cast float32 -> int32 -> float32 (truncation)", 0, 0, [&] { return Tensor(cast(cast(X.to(Device()), int32), float32)); },
+         [&] { return computed({8, 64, 32}, [&](size_t i) { return std::trunc(x[i]); }); }},
+        {"max over the last axis, kept", 0, 0, [&] { return Tensor(max(X.to(Device()), -1, true)); },
+         [&] { return computed({8, 64, 1}, [&](size_t r) { double m = x[r * 32]; for (int j = 1; j < 32; ++j) m = std::max<double>(m, x[r * 32 + j]); return m; }); }},
+        {"min over axis 1", 0, 0, [&] { return Tensor(min(X.to(Device()), 1)); },
+         [&] { return computed({8, 32}, [&](size_t o) { double m = INFINITY; for (int j = 0; j < 64; ++j) m = std::min<double>(m, x[(o / 32) * 2048 + j * 32 + o % 32]); return m; }); }},
+        {"X / max(|X|) composed of the new nodes", 1e-6, 0, [&] { Tensor d = X.to(Device()); return Tensor(div(d, max(abs(d), -1, true))); },
+         [&] { return rows([](const float* r, size_t, double* out) { double m = 0; for (int j = 0; j < 32; ++j) m = std::max<double>(m, std::fabs(r[j])); for (int j = 0; j < 32; ++j) out[j] = r[j] / m; }); }},
+        {"rms_norm(X, G, 1e-5)", 2e-6, 1e-7, [&] { return Tensor(rms_norm(X.to(Device()), G.to(Device()), 1e-5f)); },
+         [&] { return rows([&](const float* r, size_t, double* out) { double ms = 0; for (int j = 0; j < 32; ++j) ms += double(r[j]) * r[j]; ms = 1.0 / std::sqrt(ms / 32 + 1e-5f); for (int j = 0; j < 32; ++j) out[j] = r[j] * ms * g[j]; }); }},
+        {"softmax(0.5 * X)", 2e-6, 1e-9, [&] { return Tensor(softmax(X.to(Device()), 0.5f)); },
+         [&] { return rows([](const float* r, size_t, double* out) { double m = -INFINITY, sum = 0; for (int j = 0; j < 32; ++j) m = std::max<double>(m, 0.5 * r[j]); for (int j = 0; j < 32; ++j) sum += out[j] = std::exp(0.5 * r[j] - m); for (int j = 0; j < 32; ++j) out[j] /= sum; }); }},
+        {"softmax(X + causal mask)", 2e-6, 1e-9, [&] { return Tensor(softmax(X.to(Device()), Mask.to(Device()))); },
+         [&] { return rows([](const float* r, size_t row, double* out) { const int q = row % 64 % 32; double m = -INFINITY, sum = 0; for (int j = 0; j <= q; ++j) m = std::max<double>(m, r[j]); for (int j = 0; j < 32; ++j) sum += out[j] = j <= q ? std::exp(r[j] - m) : 0.0; for (int j = 0; j < 32; ++j) out[j] /= sum; }); }},
+        {"swiglu(X, P)", 2e-6, 1e-7, [&] { return Tensor(swiglu(X.to(Device()), P.to(Device()))); }, [&] { return computed({8, 64, 32}, [&](size_t i) { return x[i] / (1.0 + std::exp(-double(x[i]))) * pv[i]; }); }},
+        {"rope(X, cos, sin)", 2e-6, 1e-6, [&] { return Tensor(rope(X.to(Device()), Cs.to(Device()), Sn.to(Device()))); },
+         [&] { return computed({8, 64, 32}, [&](size_t i) { const size_t n = (i / 32) % 64, pair = (i % 32) / 2; const double c = values(Cs)[n * 16 + pair], sn = values(Sn)[n * 16 + pair];
+                                                         const double e = x[i - i % 2], o = x[i - i % 2 + 1]; return i % 2 == 0 ? e * c - o * sn : e * sn + o * c; }); }},
+    };
+
     int failures = 0;
+    for (auto& c : added) {
+        bool ok = false;
+        std::string note;
+        try {
+            Tensor device = c.device();
+            Tensor expected = c.expected();
+            if (device.shape() != expected.shape() || device.dtype() != expected.dtype()) note = "shape or dtype differs";
+            else if (!(ok = allclose(device, expected.to(Device()), c.rtol, c.atol))) note = "allclose failed";
+        } catch (std::exception const& ex) {
+            note = std::string("exception: ") + ex.what();
+        }
+        std::printf("%-50s %s %s\n", c.name.c_str(), ok ? "ok" : "FAILED", note.c_str());
+        std::fflush(stdout);
+        failures += ok ? 0 : 1;
+    }
+    // the new nodes exist on the device only
+    {
+        bool threw = false;
+        try { Tensor t = softmax(X); } catch (std::exception const&) { threw = true; }
+        std::printf("%-50s %s\n", "softmax of a host tensor throws", threw ? "ok" : "FAILED");
+        failures += threw ? 0 : 1;
+    }
+    // ---- comparisons on the device and the copy back to the host, through the (patched) front end ------------------------
+    {
+        const Tensor I2 = seeded(int32, {4, 9, 5}, 23, -50, 50);
+        const Tensor X2 = seeded(float32, {8, 64, 32}, 24, -4, 4);
+        struct Pair { const char* name; std::function<Tensor(Tensor const&, Tensor const&)> run; };
+        const std::vector<Pair> comparisons = {
+            {"==", [](Tensor const& a, Tensor const& b) { return Tensor(a == b); }}, {"!=", [](Tensor const& a, Tensor const& b) { return Tensor(a != b); }},
+            {">", [](Tensor const& a, Tensor const& b) { return Tensor(a > b); }},   {">=", [](Tensor const& a, Tensor const& b) { return Tensor(a >= b); }},
+            {"<", [](Tensor const& a, Tensor const& b) { return Tensor(a < b); }},   {"<=", [](Tensor const& a, Tensor const& b) { return Tensor(a <= b); }},
+        };
+        for (auto const& [left, right, what] : {std::tuple<Tensor const&, Tensor const&, const char*>{I, I2, "int32"}, {X, X2, "float32"}, {X, X, "float32 with itself"}}) {
+            for (auto const& c : comparisons) {
+                bool ok = false;
+                std::string note;
+                try {
+                    Tensor host = c.run(left, right);
+                    Tensor device = c.run(left.to(Device()), right.to(Device()));
+                    Tensor back = device.to(Host{});              // device -> host through Tensor::to
+                    ok = back.dtype() == boolean && back.shape() == host.shape() && std::memcmp(back.bytes(), host.bytes(), (host.nelements() + 7) / 8) == 0;
+                    if (!ok) note = "bit masks differ";
+                } catch (std::exception const& ex) {
+                    note = std::string("exception: ") + ex.what();
+                }
+                std::printf("%-50s %s %s\n", (std::string("device ") + c.name + " on " + what + ", copied back with to(Host)").c_str(), ok ? "ok" : "FAILED", note.c_str());
+                failures += ok ? 0 : 1;
+            }
+        }
+        // a float tensor's round trip host -> device -> host
+        Tensor back = X.to(Device()).to(Host{});
+        const bool same = std::memcmp(back.bytes(), X.bytes(), X.nelements() * sizeof(float)) == 0;
+        std::printf("%-50s %s\n", "host -> device -> host round trip", same ? "ok" : "FAILED");
+        failures += same ? 0 : 1;
+    }
+
     for (auto& c : cases) {
         bool ok = false;
         std::string note;
@@ -141,6 +259,6 @@ int main() {
         std::fflush(stdout);
         failures += ok ? 0 : 1;
     }
-    std::printf("%d of %zu cases failed\n", failures, cases.size());
+    std::printf("%d of %zu cases failed\n", failures, cases.size() + added.size() + 20);
     return failures ? 1 : 0;
 }
