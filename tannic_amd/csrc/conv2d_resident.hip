@@ -346,12 +346,14 @@ int run_resident(const ConvProblem& p, const void* x, const void* w, const void*
     q.div_colblocks = FastDiv(p.W / 8);
     q.div_chunks = FastDiv(p.C / kRC);
     q.div_row_blocks = FastDiv(q.row_blocks);
-    static int cus = 0;   // compute units of the device, asked once
+    static std::atomic<int> known_cus{0};   // compute units of the device, asked once
+    int cus = known_cus.load(std::memory_order_relaxed);
     if (cus == 0) {
         cus = 256;
         hipDeviceProp_t prop;
         int dev = 0;
         if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess && prop.multiProcessorCount > 0) cus = prop.multiProcessorCount;
+        known_cus.store(cus, std::memory_order_relaxed);
     }
     uint32_t workers = static_cast<uint32_t>(cus) / q.co_tiles;
     if (workers == 0) workers = 1;

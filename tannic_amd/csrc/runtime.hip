@@ -92,6 +92,8 @@ static std::vector<ScratchBlock> g_scratch_free, g_scratch_live;
 static size_t g_scratch_cached = 0;
 constexpr size_t kScratchCacheLimit = size_t(2) << 30;
 
+void release_idle_memory();   // defined below, next to the kept tensor blocks
+
 int scratch_acquire(void** ptr, size_t nbytes, hipStream_t stream) {
     int device = 0;
     TH_TRY(hipGetDevice(&device));
@@ -111,10 +113,21 @@ int scratch_acquire(void** ptr, size_t nbytes, hipStream_t stream) {
             return TANNIC_SUCCESS;
         }
     }
-    const size_t size = (nbytes + 0xFFFF) & ~size_t(0xFFFF);
-    TH_TRY(hipMalloc(ptr, size ? size : 0x10000));
+    const size_t size = ((nbytes + 0xFFFF) & ~size_t(0xFFFF)) ? ((nbytes + 0xFFFF) & ~size_t(0xFFFF)) : 0x10000;
+    hipError_t err = hipMalloc(ptr, size);
+    if (err == hipErrorOutOfMemory) {
+        // Idle memory the library itself holds may be all that is missing: the cached scratch blocks and the tensor
+        // blocks kept for reuse go back to the driver (once every stream has passed their last use), then one more try.
+        (void)hipGetLastError();
+        release_idle_memory();
+        err = hipMalloc(ptr, size);
+    }
+    if (err != hipSuccess) {
+        set_error("hipMalloc (kernel scratch)", __FILE__, __LINE__, err);
+        return TANNIC_ERROR;
+    }
     std::lock_guard<std::mutex> lock(g_scratch_mutex);
-    g_scratch_live.push_back(ScratchBlock{*ptr, size ? size : 0x10000, stream, device});
+    g_scratch_live.push_back(ScratchBlock{*ptr, size, stream, device});
     return TANNIC_SUCCESS;
 }
 
@@ -134,8 +147,10 @@ int scratch_release(void* ptr, hipStream_t stream) {
             return TANNIC_SUCCESS;
         }
     }
-    // over the cache limit (or unknown pointer): give it back once the stream has passed this point
-    TH_TRY(hipFreeAsync(ptr, stream));
+    // over the cache limit (or unknown pointer): the block came from hipMalloc, so it goes back with hipFree, once the
+    // stream has passed the kernels that used it
+    TH_TRY(hipStreamSynchronize(stream));
+    TH_TRY(hipFree(ptr));
     return TANNIC_SUCCESS;
 }
 
@@ -190,7 +205,41 @@ size_t block_size(size_t nbytes) {
     const size_t grain = nbytes < (size_t(1) << 20) ? 512 : (size_t(2) << 20);
     return (nbytes + grain - 1) / grain * grain;
 }
+
+// Gives every tensor block kept for reuse back to the pool (stream-ordered: each after its stream's last use of it).
+void release_kept_blocks() {
+    std::vector<FreeBlock> all;
+    {
+        std::lock_guard<std::mutex> lock(g_mem_mutex);
+        all.swap(g_mem_free);
+        g_mem_kept = 0;
+    }
+    for (const FreeBlock& f : all) (void)hipFreeAsync(f.ptr, f.info.stream);
+    (void)hipGetLastError();
+}
 }  // namespace
+
+}  // extern "C"
+
+// Everything idle the library holds goes back to the driver: the kept tensor blocks, the pool's cached memory and the
+// cached scratch blocks.  Called when an allocation outside the pool fails for lack of memory.
+void th::release_idle_memory() {
+    release_kept_blocks();
+    (void)hipDeviceSynchronize();
+    int device = 0;
+    hipMemPool_t pool;
+    if (hipGetDevice(&device) == hipSuccess && hipDeviceGetDefaultMemPool(&pool, device) == hipSuccess) (void)hipMemPoolTrimTo(pool, 0);
+    std::vector<ScratchBlock> idle;
+    {
+        std::lock_guard<std::mutex> lock(g_scratch_mutex);
+        idle.swap(g_scratch_free);
+        g_scratch_cached = 0;
+    }
+    for (const ScratchBlock& b : idle) (void)hipFree(b.ptr);
+    (void)hipGetLastError();
+}
+
+extern "C" {
 
 void* tannic_hip_allocate(const tannic_device_t* device, size_t nbytes) {
     if (!device || tannic_hip_set_device(device->id) != TANNIC_SUCCESS) return nullptr;
@@ -219,14 +268,7 @@ void* tannic_hip_allocate(const tannic_device_t* device, size_t nbytes) {
     hipError_t err = hipMallocAsync(&ptr, size, stream);
     if (err != hipSuccess) {
         // give the kept blocks back and try once more
-        std::vector<FreeBlock> all;
-        {
-            std::lock_guard<std::mutex> lock(g_mem_mutex);
-            all.swap(g_mem_free);
-            g_mem_kept = 0;
-        }
-        for (const FreeBlock& f : all) (void)hipFreeAsync(f.ptr, f.info.stream);
-        (void)hipGetLastError();
+        release_kept_blocks();
         err = hipMallocAsync(&ptr, size, stream);
     }
     if (err != hipSuccess) {

@@ -208,7 +208,8 @@ def test_both_forms_and_both_parameter_layouts_agree(layer):
     assert np.abs(composed - fused).mean() <= 0.02 * spread, (np.abs(composed - fused).mean(), spread)
     separate = {}
     dl.forward_fused(s, layer["w"], layer["dx"], layer["cos"], layer["sin"], layer["mask"], separate)
-    for name in ("q", "k", "v", "gate", "up"):
+    # q, k and v have the same input in both (the normalised x); what follows them has inputs a rounding apart
+    for name in ("q", "k", "v"):
         support.assert_close(numbers(separate[name]), numbers(layer["fused"][name]), ULP, 1e-3, f"{name}: concatenated against separate parameters")
     support.assert_close(numbers(separate["out"]), fused, 4 * ULP, 0.02 * spread, "layer: concatenated against separate parameters")
 
