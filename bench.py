@@ -37,7 +37,7 @@ import numpy as np  # noqa: E402
 
 PREHEAT_SECONDS = 0.25
 SECONDARY_PREHEAT_SECONDS = 0.08   # the secondary matrix workloads: as long as it takes the clock to settle
-MFMA_PEAK_TFLOPS = {"f16": 2500.0, "bf16": 2500.0, "f32": 157.3}
+MFMA_PEAK_TFLOPS = {"f16": 2500.0, "bf16": 2500.0, "f32": 157.3, "i8": 5000.0}   # i8: tera-operations per second
 HBM_PEAK_GBS = 8000.0
 
 
@@ -140,16 +140,17 @@ def gemm_entry(b, dtype, M, N, K, iters, layout="NT"):
     """layout: how the operands lie in memory. "NT": X[M,K] . W[N,K]^T (a linear layer); "NN": X[M,K] . W[K,N];
     "TN": X[K,M]^T . W[K,N]."""
     ta = b.ta
-    x = b.filled(dtype, (K, M) if layout[0] == "T" else (M, K), "normal", 0, 1, 1.0)
-    w = b.filled(dtype, (N, K) if layout[1] == "T" else (K, N), "normal", 0, 2, 0.02)
-    y = ta.Tensor(dtype, (M, N)).initialize(b.device)
+    sx, sw = (30.0, 30.0) if dtype.is_integral else (1.0, 0.02)    # integers: values across most of the int8 range
+    x = b.filled(dtype, (K, M) if layout[0] == "T" else (M, K), "normal", 0, 1, sx)
+    w = b.filled(dtype, (N, K) if layout[1] == "T" else (K, N), "normal", 0, 2, sw)
+    y = ta.Tensor(ta.int32 if dtype is ta.int8 else dtype, (M, N)).initialize(b.device)
     run = b.raw_call("gemm", [x.transpose() if layout[0] == "T" else x, w.transpose() if layout[1] == "T" else w], y)
     b.heat(run, SECONDARY_PREHEAT_SECONDS)
     ms = b.event_time(run, iters)
     flops = 2.0 * M * N * K
-    nbytes = (M * K + N * K + M * N) * dtype.itemsize
+    nbytes = (M * K + N * K) * dtype.itemsize + M * N * y.dtype.itemsize
     tflops, gbs = flops / ms / 1e9, nbytes / ms / 1e6
-    peak = MFMA_PEAK_TFLOPS["f32" if dtype is ta.float32 else "f16"]
+    peak = MFMA_PEAK_TFLOPS["f32" if dtype is ta.float32 else "i8" if dtype is ta.int8 else "f16"]
     hbm_bound = flops / nbytes < peak * 1e3 / HBM_PEAK_GBS   # below the ridge of the matrix peak over 8 TB/s
     name = {"NT": f"X[{M},{K}].W[{N},{K}]^T", "NN": f"X[{M},{K}].W[{K},{N}]", "TN": f"X[{K},{M}]^T.W[{K},{N}]"}[layout]
     return {"op": f"gemm {dtype} {name}", "us": round(ms * 1e3, 2), "tflops": round(tflops, 2), "gbs": round(gbs, 1),
@@ -413,6 +414,7 @@ def secondary(b, only):
         work.append(gemm_entry(b, ta.float16, 4096, 4096, 4096, 20, "NN"))
         work.append(gemm_entry(b, ta.float16, 4096, 4096, 4096, 20, "TN"))
         work.append(gemm_entry(b, ta.bfloat16, 4096, 4096, 4096, 20))
+        work.append(gemm_entry(b, ta.int8, 4096, 4096, 4096, 20))
         work.append(gemm_entry(b, ta.float32, 512, 512, 512, 20))
         work.append(gemm_entry(b, ta.float32, 4096, 4096, 4096, 5))
     if only in (None, "gemm-ceiling"):

@@ -1,8 +1,8 @@
 // gemm entry point: problem description, dtype table, generic kernel.
 //
 // Destination type per operand pair as in src/cpu/matmul.cpp:189-252.  The
-// 16-bit same-type pairs and fp32 go to the MFMA kernels (gemm_mfma.hip) when
-// their layout conditions hold; every other pair, and the leftovers, run the
+// 16-bit same-type pairs, int8 x int8 and fp32 go to the MFMA kernels (gemm_mfma.hip,
+// gemm_dtl.hip) when their layout conditions hold; every other pair, and the leftovers, run the
 // LDS-tiled scalar kernel below, which accepts any strides.
 //
 // Differences from the reference CPU path, all documented at the ABI:
@@ -210,6 +210,9 @@ int gemm_entry(const tannic_tensor_t* a, const tannic_tensor_t* b, tannic_tensor
                 if (status != TANNIC_SUCCESS) return;
                 if constexpr (std::is_same_v<A, B> && is_16bit<A>::value) {
                     status = gemm_mfma_16bit(p, a->dtype, a->address, b->address, dst->address, s, workspace);
+                    if (status != TANNIC_UNSUPPORTED_DTYPE) return;
+                } else if constexpr (std::is_same_v<A, int8_t> && std::is_same_v<B, int8_t>) {
+                    status = gemm_mfma_int8(p, a->address, b->address, dst->address, s);
                     if (status != TANNIC_UNSUPPORTED_DTYPE) return;
                 } else if constexpr (std::is_same_v<A, float> && std::is_same_v<B, float>) {
                     status = gemm_mfma_f32(p, static_cast<const float*>(a->address), static_cast<const float*>(b->address),

@@ -21,6 +21,8 @@
 // fragment reads (lane l: row l % 16, k chunk l / 16 of the slice) and 64 MFMAs.  The B fragment is the first operand,
 // so an accumulator holds C transposed: lane l has row l % 16 of the 16 x 16 block and its four values are columns
 // 4 * (l / 16) .. + 3.  Sums are formed in the same order of k as in gemm16_kernel: results are bit-identical.
+//
+// int8 x int8 -> int32 runs the same kernel on v_mfma_i32_16x16x64_i8: a 128-byte tile row is 128 elements, a k-slice 64.
 #include "gemm_tiles.hpp"
 
 namespace th {
@@ -28,9 +30,20 @@ namespace th {
 typedef __attribute__((address_space(3))) void* lds_void;
 
 typedef float float4v __attribute__((ext_vector_type(4)));
+typedef int int4v __attribute__((ext_vector_type(4)));
 
-template <class T> __device__ inline void mfma16x16_in_place(float4v& acc, const uint4v& first, const uint4v& second) {
-    if constexpr (std::is_same_v<T, f16>) {
+// int8 operands: v_mfma_i32_16x16x64_i8, the same 16-byte fragments (lane l: row l % 16, the 16 k of chunk l / 16 of a
+// 64-byte slice), int32 accumulators that wrap like the CPU path's; results are written from the registers.
+template <class T> struct DtlTypes { using Acc = float4v; using Out = T; };
+template <> struct DtlTypes<int8_t> { using Acc = int4v; using Out = int32_t; };
+
+template <class T> __device__ inline void mfma16x16_in_place(typename DtlTypes<T>::Acc& acc, const uint4v& first, const uint4v& second) {
+    if constexpr (std::is_same_v<T, int8_t>) {
+        int4v x, y;
+        __builtin_memcpy(&x, &first, 16);
+        __builtin_memcpy(&y, &second, 16);
+        acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(x, y, acc, 0, 0, 0);
+    } else if constexpr (std::is_same_v<T, f16>) {
         half8 x, y;
         __builtin_memcpy(&x, &first, 16);
         __builtin_memcpy(&y, &second, 16);
@@ -46,9 +59,9 @@ template <class T> __device__ inline void mfma16x16_in_place(float4v& acc, const
 // BM x BN: 256 x 256, 256 x 128 or 128 x 128 (2 x 2 wavefronts each).  The smaller tiles are for products with too few
 // large tiles to fill the chip; two workgroups of the smallest share a compute unit.
 template <class T, int BM, int BN, int STAGES, int BLOCKS_PER_CU>
-__global__ __launch_bounds__(256, BLOCKS_PER_CU) void gemm16_dtl_kernel(const T* A, const T* B, T* C, GemmProblem p, uint32_t tiles_m, uint32_t tiles_n) {
+__global__ __launch_bounds__(256, BLOCKS_PER_CU) void gemm16_dtl_kernel(const T* A, const T* B, typename DtlTypes<T>::Out* C, GemmProblem p, uint32_t tiles_m, uint32_t tiles_n) {
 #if defined(__HIP_DEVICE_COMPILE__)   // the host pass needs the launch stub only (and loses it over the body's device-only builtins)
-    constexpr int BK = 64, WAVES_N = 2;
+    constexpr int ES = sizeof(T), BK = 128 / ES, WAVES_N = 2;   // a tile row is 128 bytes: 64 elements of 16 bits, 128 of 8
     constexpr int WM = BM / 2, WN = BN / 2, TM = WM / 16, TN = WN / 16;
     constexpr uint32_t A_TILE = BM * BK, B_TILE = BN * BK, STAGE = A_TILE + B_TILE;   // elements
     constexpr int LOADS_A = BM / 32, LOADS_B = BN / 32, LOADS = LOADS_A + LOADS_B;     // 1 KB loads per wavefront and tile
@@ -70,7 +83,7 @@ __global__ __launch_bounds__(256, BLOCKS_PER_CU) void gemm16_dtl_kernel(const T*
     const T* a_base = A + oa + static_cast<int64_t>(m0) * p.a_rs;
     const T* b_base = B + ob + static_cast<int64_t>(n0) * p.b_cs;
     auto records = [](uint64_t rows_left, int64_t stride, uint32_t K) -> uint32_t {
-        const uint64_t bytes = ((rows_left - 1) * static_cast<uint64_t>(stride) + K) * 2;
+        const uint64_t bytes = ((rows_left - 1) * static_cast<uint64_t>(stride) + K) * ES;
         return bytes > 0xFFFFFFFFull ? 0xFFFFFFFFu : static_cast<uint32_t>(bytes);
     };
     const __amdgpu_buffer_rsrc_t rsrc_a = __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(a_base), 0, records(p.M - m0, p.a_rs, p.K), 0x00020000);
@@ -82,18 +95,19 @@ __global__ __launch_bounds__(256, BLOCKS_PER_CU) void gemm16_dtl_kernel(const T*
     for (int j = 0; j < LOADS; ++j) {
         const uint32_t row = (j < LOADS_A ? wave * LOADS_A + j : wave * LOADS_B + (j - LOADS_A)) * 8 + lane / 8;
         const uint32_t chunk = (lane % 8) ^ ((row >> 1) & 7u);
-        voff[j] = row * static_cast<uint32_t>(j < LOADS_A ? p.a_rs : p.b_cs) * 2 + chunk * 16;
+        voff[j] = row * static_cast<uint32_t>(j < LOADS_A ? p.a_rs : p.b_cs) * ES + chunk * 16;
     }
     auto issue_load = [&](int j, uint32_t stage, uint32_t k_bytes) {
-        const uint32_t at = stage * (STAGE * 2) + (j < LOADS_A ? (wave * LOADS_A + j) * 1024 : A_TILE * 2 + (wave * LOADS_B + (j - LOADS_A)) * 1024);
+        const uint32_t at = stage * (STAGE * ES) + (j < LOADS_A ? (wave * LOADS_A + j) * 1024 : A_TILE * ES + (wave * LOADS_B + (j - LOADS_A)) * 1024);
         __builtin_amdgcn_raw_ptr_buffer_load_lds(j < LOADS_A ? rsrc_a : rsrc_b, (lds_void)(lds_raw + at), 16, voff[j], k_bytes, 0, 0);
     };
 
-    float4v acc[TM][TN];
+    using Acc = typename DtlTypes<T>::Acc;
+    Acc acc[TM][TN];
 #pragma unroll
     for (int i = 0; i < TM; ++i)
 #pragma unroll
-        for (int j = 0; j < TN; ++j) acc[i][j] = float4v{0.0f, 0.0f, 0.0f, 0.0f};
+        for (int j = 0; j < TN; ++j) acc[i][j] = Acc{0, 0, 0, 0};
 
     // Tile loads complete in the order they were issued: waiting until at most AHEAD of them are outstanding leaves the
     // tiles that are not needed yet in flight.
@@ -113,7 +127,7 @@ __global__ __launch_bounds__(256, BLOCKS_PER_CU) void gemm16_dtl_kernel(const T*
     for (int t = 0; t < STAGES - 1; ++t) {
         if (static_cast<uint32_t>(t) < steps) {
 #pragma unroll
-            for (int j = 0; j < LOADS; ++j) issue_load(j, t, t * (BK * 2));
+            for (int j = 0; j < LOADS; ++j) issue_load(j, t, t * 128);
         }
     }
     wait_loads(steps < static_cast<uint32_t>(STAGES - 1));
@@ -153,7 +167,7 @@ __global__ __launch_bounds__(256, BLOCKS_PER_CU) void gemm16_dtl_kernel(const T*
             if constexpr (!(FIRST && group == 0)) mfma16x16_in_place<T>(acc[i][j], fb[now][j], fa[now][i]);
             if constexpr (q < TM + TN && !(FIRST && group == 0)) read_one(a_tile, b_tile, group == 0 ? 0 : 1, group == 0 ? 0 : 1, q);
             constexpr int slot = FIRST ? m - PER_KS : m;
-            if constexpr (FETCH && slot >= 0 && slot % LOAD_EVERY == LOAD_EVERY / 2 && slot / LOAD_EVERY < LOADS) issue_load(slot / LOAD_EVERY, fill, (s + STAGES - 1) * (BK * 2));
+            if constexpr (FETCH && slot >= 0 && slot % LOAD_EVERY == LOAD_EVERY / 2 && slot / LOAD_EVERY < LOADS) issue_load(slot / LOAD_EVERY, fill, (s + STAGES - 1) * 128);
             __builtin_amdgcn_sched_barrier(0);
         });
         wait_loads(!FETCH);    // tile s+1 is in LDS (steps that issue no loads wait for all that are left)
@@ -175,6 +189,20 @@ __global__ __launch_bounds__(256, BLOCKS_PER_CU) void gemm16_dtl_kernel(const T*
 
     // Each wavefront rounds its block into its own LDS area (no operand tile is read after the last barrier) and
     // writes it out as whole rows, 16 bytes per lane.
+    if constexpr (ES == 1) {
+        // int32 results: a lane's four consecutive columns are 16 bytes already
+        int32_t* c32 = C + oc;
+#pragma unroll
+        for (int i = 0; i < TM; ++i) {
+            const uint32_t row = m0 + wm + i * 16 + lane % 16;
+#pragma unroll
+            for (int j = 0; j < TN; ++j) {
+                const uint32_t col = n0 + wn + j * 16 + 4 * (lane / 16);
+                if (row < p.M && col < p.N) *reinterpret_cast<int4v*>(c32 + static_cast<int64_t>(row) * p.c_rs + col) = acc[i][j];
+            }
+        }
+        return;
+    } else {
     T* c = C + oc;
     constexpr int PITCH = WN + 8;
     T* stage = lds + wave * (WM * PITCH);
@@ -197,19 +225,20 @@ __global__ __launch_bounds__(256, BLOCKS_PER_CU) void gemm16_dtl_kernel(const T*
         const uint4v bits = *reinterpret_cast<const uint4v*>(stage + r * PITCH + (lane % LANES_PER_ROW) * 8);
         if (row < p.M && col < p.N) *reinterpret_cast<uint4v*>(c + static_cast<int64_t>(row) * p.c_rs + col) = bits;
     }
+    }
 #endif
 }
 
 template <class T, int BM, int BN, int STAGES>
 static int launch_dtl(const GemmProblem& p, const void* a, const void* b, void* c, hipStream_t stream) {
     const uint32_t tiles_m = (p.M + BM - 1) / BM, tiles_n = (p.N + BN - 1) / BN;
-    constexpr size_t tile_bytes = STAGES * (BM + BN) * 128, stage_bytes = 2 * 4 * (BM / 2) * (BN / 2 + 8);   // the operand stages; the output staging
+    constexpr size_t tile_bytes = STAGES * (BM + BN) * 128, stage_bytes = sizeof(T) == 2 ? 2 * 4 * (BM / 2) * (BN / 2 + 8) : 0;   // the operand stages; the output staging (16-bit results)
     constexpr size_t lds_bytes = tile_bytes > stage_bytes ? tile_bytes : stage_bytes;
     auto kernel = gemm16_dtl_kernel<T, BM, BN, STAGES, (lds_bytes <= 80 * 1024 ? 2 : 1)>;
     static std::atomic<uint64_t> configured{0};
     if (int rc = raise_lds_limit(reinterpret_cast<const void*>(kernel), lds_bytes, configured)) return rc;
     hipLaunchKernelGGL(kernel, dim3(tiles_m * tiles_n, p.batches), dim3(256), lds_bytes, stream, static_cast<const T*>(a), static_cast<const T*>(b),
-                       static_cast<T*>(c), p, tiles_m, tiles_n);
+                       static_cast<typename DtlTypes<T>::Out*>(c), p, tiles_m, tiles_n);
     return launch_status("gemm16_dtl_kernel");
 }
 
@@ -217,10 +246,11 @@ static int launch_dtl(const GemmProblem& p, const void* a, const void* b, void* 
 template <class T>
 int gemm16_dtl(const GemmProblem& p, int bm, int bn, const void* a, const void* b, void* c, hipStream_t stream) {
     if (p.a_cs != 1 || p.b_rs != 1) return TANNIC_UNSUPPORTED_DTYPE;                     // both operands K-contiguous
-    if (p.K == 0 || p.K % 64 != 0 || p.row_bias) return TANNIC_UNSUPPORTED_DTYPE;         // whole K steps only, no start values
-    if (p.N % 8 != 0 || p.c_rs % 8 != 0 || reinterpret_cast<uintptr_t>(c) % 16 != 0) return TANNIC_UNSUPPORTED_DTYPE;
+    constexpr int step = 128 / sizeof(T), quad = 16 / sizeof(typename DtlTypes<T>::Out);   // K elements per step; results per 16-byte store
+    if (p.K == 0 || p.K % step != 0 || p.row_bias) return TANNIC_UNSUPPORTED_DTYPE;       // whole K steps only, no start values
+    if (p.N % quad != 0 || p.c_rs % quad != 0 || reinterpret_cast<uintptr_t>(c) % 16 != 0) return TANNIC_UNSUPPORTED_DTYPE;
     for (int d = 0; d < p.batch_rank; ++d)
-        if (p.c_bs[d] % 8 != 0) return TANNIC_UNSUPPORTED_DTYPE;
+        if (p.c_bs[d] % quad != 0) return TANNIC_UNSUPPORTED_DTYPE;
     // a row's offset inside a tile is a 32-bit byte count; rows must not overlap (the range check relies on it)
     if (p.a_rs < static_cast<int64_t>(p.K) || p.b_cs < static_cast<int64_t>(p.K)) return TANNIC_UNSUPPORTED_DTYPE;
     if (p.a_rs >= (1 << 22) || p.b_cs >= (1 << 22)) return TANNIC_UNSUPPORTED_DTYPE;
@@ -233,5 +263,21 @@ int gemm16_dtl(const GemmProblem& p, int bm, int bn, const void* a, const void* 
 
 template int gemm16_dtl<f16>(const GemmProblem&, int, int, const void*, const void*, void*, hipStream_t);
 template int gemm16_dtl<bf16>(const GemmProblem&, int, int, const void*, const void*, void*, hipStream_t);
+template int gemm16_dtl<int8_t>(const GemmProblem&, int, int, const void*, const void*, void*, hipStream_t);
+
+// int8 x int8 -> int32 (src/cpu/matmul.cpp:191-209): exact, so the tiled kernel's results are the scalar kernel's bit for
+// bit.  Both operands K-contiguous and 16-byte friendly; the tile follows the number of tiles it leaves.
+int gemm_mfma_int8(const GemmProblem& p, const void* a, const void* b, void* c, hipStream_t stream) {
+    if (p.M == 0 || p.N == 0 || p.batches == 0) return TANNIC_SUCCESS;
+    if (p.a_cs != 1 || p.b_rs != 1 || p.K % 128 != 0 || p.batches > 65535) return TANNIC_UNSUPPORTED_DTYPE;
+    if (reinterpret_cast<uintptr_t>(a) % 16 || reinterpret_cast<uintptr_t>(b) % 16 || p.a_rs % 16 || p.b_cs % 16) return TANNIC_UNSUPPORTED_DTYPE;
+    for (int d = 0; d < p.batch_rank; ++d)
+        if (p.a_bs[d] % 16 || p.b_bs[d] % 16) return TANNIC_UNSUPPORTED_DTYPE;
+    auto tiles = [&](uint64_t bm, uint64_t bn) { return ((p.M + bm - 1) / bm) * ((p.N + bn - 1) / bn) * p.batches; };
+    if (p.M > 192 && tiles(256, 256) >= 200) return gemm16_dtl<int8_t>(p, 256, 256, a, b, c, stream);
+    if (p.M > 192 && tiles(256, 128) >= 128) return gemm16_dtl<int8_t>(p, 256, 128, a, b, c, stream);
+    if (p.M > 32) return gemm16_dtl<int8_t>(p, 128, 128, a, b, c, stream);
+    return TANNIC_UNSUPPORTED_DTYPE;
+}
 
 }  // namespace th

@@ -98,6 +98,24 @@ def test_integer_gemm_bit_exact(device, pair, layout):
     support.assert_bit_exact(got.storage(), want.storage(), f"gemm {pair} {layout}")
 
 
+@pytest.mark.parametrize("shape", [((300, 256), (520, 256)), ((16, 300, 128), (16, 520, 128)), ((50, 264, 128), (50, 264, 128)), ((2, 3, 70, 384), (136, 384)),
+                                   ((4096, 512), (1024, 512))], ids=lambda s: "x".join(map(str, s[0])) + "." + "x".join(map(str, s[1])) + "T")
+def test_int8_gemm_on_matrix_cores_is_bit_exact(device, shape):
+    """int8 x int8 -> int32 with both operands K-contiguous and K a multiple of 128: the tiled kernels on
+    v_mfma_i32_16x16x64_i8 in each tile size (128 x 128, 256 x 128, 256 x 256; ragged rows and columns, batches, a
+    broadcast second operand).  Integer sums are exact, so the checker's sequential loop and numpy agree bit for bit."""
+    sa, sb = shape
+    a = support.integers(SEED, 31, sa, -128, 128).astype(np.int8)
+    b = support.integers(SEED, 32, sb, -128, 128).astype(np.int8)
+    (ha, da), (hb, db) = support.both(a, ta.int8, device), support.both(b, ta.int8, device)
+    got = ops.matmul(da, db.transpose())
+    assert got.dtype is ta.int32
+    want = np.matmul(a.astype(np.int64), np.swapaxes(b.astype(np.int64), -1, -2)).astype(np.int32)
+    support.assert_bit_exact(got.storage(), want, f"int8 gemm {sa} x {sb}^T against numpy")
+    if int(np.prod(sa)) * sb[-2] < 40_000_000:
+        support.assert_bit_exact(got.storage(), ops.matmul(ha, hb.transpose()).storage(), f"int8 gemm {sa} x {sb}^T against the checker")
+
+
 @pytest.mark.parametrize("pair", [(ta.int32, ta.float32), (ta.float64, ta.float32), (ta.float16, ta.float32), (ta.float32, ta.bfloat16)],
                          ids=lambda p: f"{p[0]}-{p[1]}")
 def test_mixed_gemm(device, pair):
