@@ -46,22 +46,36 @@ struct Operand {
 // touches the loaded values (and waits for them) early.
 // Both loaders expose their work as single memory operations (fetch_one /
 // commit_one) so that the main loop can spread them between MFMAs.
-template <class T, int ROWS, int THREADS>
+// ALIGNED = false: the operand's address, leading dimension or K is not a multiple of 16 bytes, so a chunk is gathered
+// element by element (each element checked against K, rows past K's end of a chunk read as zero) - eight loads where
+// the aligned loader issues one, which still leaves the product on the matrix cores.
+template <class T, int ROWS, int THREADS, bool ALIGNED = true>
 struct KMajorLoader {
     static constexpr int ROWS_PER_PASS = THREADS / 8;
     static constexpr int LOADS = ROWS / ROWS_PER_PASS, STORES = ROWS / ROWS_PER_PASS;
     uint4v regs[LOADS];
     const T* base;      // operand base + this thread's k offset for the tile being fetched
     bool k_live;
+    uint32_t k_left;    // ALIGNED = false: how many of the chunk's elements lie inside K
     __device__ inline void begin_fetch(const Operand& op, uint32_t k0, uint32_t K) {
         const uint32_t k = k0 + (threadIdx.x % 8) * kChunkOf<T>;
         k_live = k < K;
+        k_left = k_live ? K - k : 0;
         base = static_cast<const T*>(op.base) + (k_live ? k : 0);
     }
     __device__ inline void fetch_one(int i, const Operand& op, uint32_t row0) {
         const uint32_t row = row0 + threadIdx.x / 8 + ROWS_PER_PASS * i;
         const uint32_t srow = row < op.rows ? row : op.rows - 1;
-        regs[i] = *reinterpret_cast<const uint4v*>(base + static_cast<int64_t>(srow) * op.row_stride);
+        if constexpr (ALIGNED) {
+            regs[i] = *reinterpret_cast<const uint4v*>(base + static_cast<int64_t>(srow) * op.row_stride);
+        } else {
+            using U = std::conditional_t<sizeof(T) == 2, uint16_t, uint32_t>;
+            const U* from = reinterpret_cast<const U*>(base + static_cast<int64_t>(srow) * op.row_stride);
+            U piece[kChunkOf<T>];
+#pragma unroll
+            for (int e = 0; e < kChunkOf<T>; ++e) piece[e] = static_cast<uint32_t>(e) < k_left ? from[e] : U(0);
+            __builtin_memcpy(&regs[i], piece, 16);
+        }
     }
     template <bool MASK>
     __device__ inline void commit_one(int i, T* tile) const {
@@ -170,8 +184,8 @@ template <class T, bool K_MAJOR> constexpr bool kAsIs = !K_MAJOR && sizeof(T) ==
 // elements of LDS that one buffer of an operand's tile takes
 template <class T, int ROWS, bool K_MAJOR> constexpr uint32_t kTileElements = kAsIs<T, K_MAJOR> ? kBKof<T> * (ROWS + 32) : ROWS * kBKof<T>;
 
-template <class T, int ROWS, int THREADS, bool K_MAJOR>
-using Loader = std::conditional_t<K_MAJOR, KMajorLoader<T, ROWS, THREADS>,
+template <class T, int ROWS, int THREADS, bool K_MAJOR, bool ALIGNED = true>
+using Loader = std::conditional_t<K_MAJOR, KMajorLoader<T, ROWS, THREADS, ALIGNED>,
                                   std::conditional_t<sizeof(T) == 2, AsIsLoader<T, ROWS, THREADS>, RowMajorLoader<T, ROWS, THREADS>>>;
 
 // WAVES_N: wavefronts along N (2 -> 256 threads, one wavefront per SIMD; 4 -> 512 threads, two per SIMD, so that
@@ -184,7 +198,7 @@ struct SplitK {
 
 // SPLIT: several blocks share an output tile, each taking a range of K and storing its fp32 accumulators; a second
 // kernel adds the shares in split order, rounds once and writes C.
-template <class T, int BM, int BN, int WAVES_N, bool A_KMAJOR, bool B_KMAJOR, bool SPLIT = false>
+template <class T, int BM, int BN, int WAVES_N, bool A_KMAJOR, bool B_KMAJOR, bool SPLIT = false, bool ALIGNED = true>
 __global__ __launch_bounds__(128 * WAVES_N) void gemm16_kernel(const T* A, const T* B, T* C, GemmProblem p, uint32_t tiles_m, uint32_t tiles_n, SplitK sk) {
     constexpr int THREADS = 128 * WAVES_N;
     constexpr int WM = BM / 2, WN = BN / WAVES_N;
@@ -225,8 +239,8 @@ __global__ __launch_bounds__(128 * WAVES_N) void gemm16_kernel(const T* A, const
             for (int v = 0; v < 16; ++v) acc[i][j][v] = start;
     }
 
-    using LA = Loader<T, BM, THREADS, A_KMAJOR>;
-    using LB = Loader<T, BN, THREADS, B_KMAJOR>;
+    using LA = Loader<T, BM, THREADS, A_KMAJOR, ALIGNED>;
+    using LB = Loader<T, BN, THREADS, B_KMAJOR, ALIGNED>;
     LA la;
     LB lb;
     const uint32_t steps = (K + kBK - 1) / kBK;
@@ -434,14 +448,14 @@ __global__ __launch_bounds__(128 * WAVES_N) void gemm16_kernel(const T* A, const
     }
 }
 
-template <class T, int BM, int BN, int WAVES_N, bool AK, bool BK_, bool SPLIT = false>
+template <class T, int BM, int BN, int WAVES_N, bool AK, bool BK_, bool SPLIT = false, bool ALIGNED = true>
 int launch16(const GemmProblem& p, const void* a, const void* b, void* c, hipStream_t stream, SplitK sk = SplitK{1, 0, nullptr}) {
     const uint32_t tiles_m = (p.M + BM - 1) / BM, tiles_n = (p.N + BN - 1) / BN;
     // operand tiles (two buffers each); the same memory later stages the output, BM*BN elements in padded rows
     constexpr size_t tile_bytes = sizeof(T) * 2 * (kTileElements<T, BM, AK> + kTileElements<T, BN, BK_>);
     constexpr size_t stage_bytes = sizeof(T) * 2 * WAVES_N * (BM / 2) * (BN / WAVES_N + 8);
     constexpr size_t lds_bytes = (sizeof(T) == 2 && stage_bytes > tile_bytes) ? stage_bytes : tile_bytes;   // fp32 results are not staged
-    auto kernel = gemm16_kernel<T, BM, BN, WAVES_N, AK, BK_, SPLIT>;
+    auto kernel = gemm16_kernel<T, BM, BN, WAVES_N, AK, BK_, SPLIT, ALIGNED>;
     static std::atomic<uint64_t> configured{0};
     if (int rc = raise_lds_limit(reinterpret_cast<const void*>(kernel), lds_bytes, configured)) return rc;
     hipLaunchKernelGGL(kernel, dim3(tiles_m * tiles_n * sk.splits, p.batches), dim3(128 * WAVES_N), lds_bytes, stream, static_cast<const T*>(a),
@@ -543,12 +557,17 @@ int run16(const GemmProblem& p, const void* a, const void* b, void* c, hipStream
     // 16-byte accesses: addresses, leading dimensions, batch strides and the
     // contiguous extent must be multiples of a chunk (8 elements of 16 bits, 4 of 32)
     auto mult8 = [](int64_t v) { return v % kChunkOf<T> == 0; };
-    if (reinterpret_cast<uintptr_t>(a) % 16 || reinterpret_cast<uintptr_t>(b) % 16) return TANNIC_UNSUPPORTED_DTYPE;
-    if (!mult8(ak ? p.a_rs : p.a_cs) || !mult8(bk ? p.b_cs : p.b_rs)) return TANNIC_UNSUPPORTED_DTYPE;
-    if (!mult8(ak ? p.K : p.M) || !mult8(bk ? p.K : p.N)) return TANNIC_UNSUPPORTED_DTYPE;
-    for (int d = 0; d < p.batch_rank; ++d)
-        if (!mult8(p.a_bs[d]) || !mult8(p.b_bs[d])) return TANNIC_UNSUPPORTED_DTYPE;
+    bool aligned = !(reinterpret_cast<uintptr_t>(a) % 16 || reinterpret_cast<uintptr_t>(b) % 16);
+    aligned = aligned && mult8(ak ? p.a_rs : p.a_cs) && mult8(bk ? p.b_cs : p.b_rs) && mult8(ak ? p.K : p.M) && mult8(bk ? p.K : p.N);
+    for (int d = 0; d < p.batch_rank; ++d) aligned = aligned && mult8(p.a_bs[d]) && mult8(p.b_bs[d]);
     if (p.batches > 65535) return TANNIC_UNSUPPORTED_DTYPE;
+    if (!aligned) {
+        // Both operands K-contiguous (a linear layer whose width or row pitch is odd): the tiles are gathered element by
+        // element and the product stays on the matrix cores.  Other layouts take the scalar kernel.
+        if (!(ak && bk) || p.row_bias) return TANNIC_UNSUPPORTED_DTYPE;
+        if (p.M > 64) return launch16<T, 128, 128, 2, true, true, false, false>(p, a, b, c, stream);
+        return launch16<T, 64, 128, 2, true, true, false, false>(p, a, b, c, stream);
+    }
     // Tile height by M (a tile taller than M multiplies padding), large tiles only when they still give every CU work.
     const uint64_t big = static_cast<uint64_t>((p.M + 255) / 256) * ((p.N + 255) / 256) * p.batches;
     if (p.M > 192 && big >= 200) {

@@ -47,6 +47,10 @@ LAYOUTS = {
     "tt_tiles_ragged": ((136, 264), (520, 136), [("transpose", (-1, -2))], [("transpose", (-1, -2))]),
     "tn_large_tiles_batched": ((50, 24, 264), (50, 24, 264), [("transpose", (-1, -2))], []),
     "nn_large_tiles_batched": ((50, 264, 72), (50, 72, 264), [], []),
+    # K-contiguous operands that 16-byte loads cannot take: odd K, odd row pitch, a view starting at an odd column
+    "nt_odd_k": ((130, 75), (190, 75), [], [("transpose", (-1, -2))]),
+    "nt_odd_pitch_and_start": ((130, 77), (190, 79), [("index", (slice(None), slice(1, 73)))], [("index", (slice(None), slice(3, 75))), ("transpose", (-1, -2))]),
+    "nt_odd_k_few_rows_batched": ((3, 40, 203), (3, 150, 203), [], [("transpose", (-1, -2))]),
     # both operands K-contiguous, whole K steps, 200 large tiles: the tiles filled by direct global -> LDS loads
     # (rows past the end of both operands; one, two and three K steps)
     "nt_direct_one_step": ((50, 264, 64), (50, 264, 64), [], [("transpose", (-1, -2))]),
