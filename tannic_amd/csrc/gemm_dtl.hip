@@ -58,8 +58,9 @@ template <class T> __device__ inline void mfma16x16_in_place(typename DtlTypes<T
 
 // BM x BN: 256 x 256, 256 x 128 or 128 x 128 (2 x 2 wavefronts each).  The smaller tiles are for products with too few
 // large tiles to fill the chip; two workgroups of the smallest share a compute unit.
-template <class T, int BM, int BN, int STAGES, int BLOCKS_PER_CU>
-__global__ __launch_bounds__(256, BLOCKS_PER_CU) void gemm16_dtl_kernel(const T* A, const T* B, typename DtlTypes<T>::Out* C, GemmProblem p, uint32_t tiles_m, uint32_t tiles_n) {
+// SPLIT: `sk.splits` workgroups share a tile, each taking sk.k_chunk of K and storing its fp32 accumulators.
+template <class T, int BM, int BN, int STAGES, int BLOCKS_PER_CU, bool SPLIT = false>
+__global__ __launch_bounds__(256, BLOCKS_PER_CU) void gemm16_dtl_kernel(const T* A, const T* B, typename DtlTypes<T>::Out* C, GemmProblem p, uint32_t tiles_m, uint32_t tiles_n, SplitK sk) {
 #if defined(__HIP_DEVICE_COMPILE__)   // the host pass needs the launch stub only (and loses it over the body's device-only builtins)
     constexpr int ES = sizeof(T), BK = 128 / ES, WAVES_N = 2;   // a tile row is 128 bytes: 64 elements of 16 bits, 128 of 8
     constexpr int WM = BM / 2, WN = BN / 2, TM = WM / 16, TN = WN / 16;
@@ -69,11 +70,15 @@ __global__ __launch_bounds__(256, BLOCKS_PER_CU) void gemm16_dtl_kernel(const T*
     T* lds = reinterpret_cast<T*>(lds_raw);           // stage s: A tile at s * STAGE, B tile right behind it
 
     uint32_t tm, tn;
-    tile_of(blockIdx.x, tiles_m, tiles_n, tm, tn);
+    const uint32_t split = SPLIT ? blockIdx.x % sk.splits : 0;
+    tile_of(SPLIT ? blockIdx.x / sk.splits : blockIdx.x, tiles_m, tiles_n, tm, tn);
     int64_t oa, ob, oc;
     batch_offsets(p, blockIdx.y, oa, ob, oc);
     const uint32_t m0 = tm * BM, n0 = tn * BN;
-    const uint32_t steps = p.K / BK;
+    // this workgroup's range of K: all of it, or its share (whole steps)
+    const uint32_t k_first = SPLIT ? split * sk.k_chunk : 0;
+    const uint32_t steps = (SPLIT ? (p.K - k_first < sk.k_chunk ? p.K - k_first : sk.k_chunk) : p.K) / BK;
+    const uint32_t k_first_bytes = k_first * ES;
 
     const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
     const int wm = (wave / WAVES_N) * WM, wn = (wave % WAVES_N) * WN;
@@ -127,7 +132,7 @@ __global__ __launch_bounds__(256, BLOCKS_PER_CU) void gemm16_dtl_kernel(const T*
     for (int t = 0; t < STAGES - 1; ++t) {
         if (static_cast<uint32_t>(t) < steps) {
 #pragma unroll
-            for (int j = 0; j < LOADS; ++j) issue_load(j, t, t * 128);
+            for (int j = 0; j < LOADS; ++j) issue_load(j, t, k_first_bytes + t * 128);
         }
     }
     wait_loads(steps < static_cast<uint32_t>(STAGES - 1));
@@ -167,7 +172,7 @@ __global__ __launch_bounds__(256, BLOCKS_PER_CU) void gemm16_dtl_kernel(const T*
             if constexpr (!(FIRST && group == 0)) mfma16x16_in_place<T>(acc[i][j], fb[now][j], fa[now][i]);
             if constexpr (q < TM + TN && !(FIRST && group == 0)) read_one(a_tile, b_tile, group == 0 ? 0 : 1, group == 0 ? 0 : 1, q);
             constexpr int slot = FIRST ? m - PER_KS : m;
-            if constexpr (FETCH && slot >= 0 && slot % LOAD_EVERY == LOAD_EVERY / 2 && slot / LOAD_EVERY < LOADS) issue_load(slot / LOAD_EVERY, fill, (s + STAGES - 1) * 128);
+            if constexpr (FETCH && slot >= 0 && slot % LOAD_EVERY == LOAD_EVERY / 2 && slot / LOAD_EVERY < LOADS) issue_load(slot / LOAD_EVERY, fill, k_first_bytes + (s + STAGES - 1) * 128);
             __builtin_amdgcn_sched_barrier(0);
         });
         wait_loads(!FETCH);    // tile s+1 is in LDS (steps that issue no loads wait for all that are left)
@@ -189,7 +194,20 @@ __global__ __launch_bounds__(256, BLOCKS_PER_CU) void gemm16_dtl_kernel(const T*
 
     // Each wavefront rounds its block into its own LDS area (no operand tile is read after the last barrier) and
     // writes it out as whole rows, 16 bytes per lane.
-    if constexpr (ES == 1) {
+    if constexpr (SPLIT) {
+        // fp32 partial sums, [split][batch][M][N]: a lane's four consecutive columns are 16 bytes
+        float* mine = sk.partials + (static_cast<size_t>(split) * p.batches + blockIdx.y) * p.M * p.N;
+#pragma unroll
+        for (int i = 0; i < TM; ++i) {
+            const uint32_t row = m0 + wm + i * 16 + lane % 16;
+#pragma unroll
+            for (int j = 0; j < TN; ++j) {
+                const uint32_t col = n0 + wn + j * 16 + 4 * (lane / 16);
+                if (row < p.M && col < p.N) *reinterpret_cast<Acc*>(mine + static_cast<size_t>(row) * p.N + col) = acc[i][j];
+            }
+        }
+        return;
+    } else if constexpr (ES == 1) {
         // int32 results: a lane's four consecutive columns are 16 bytes already
         int32_t* c32 = C + oc;
 #pragma unroll
@@ -229,18 +247,35 @@ __global__ __launch_bounds__(256, BLOCKS_PER_CU) void gemm16_dtl_kernel(const T*
 #endif
 }
 
-template <class T, int BM, int BN, int STAGES>
-static int launch_dtl(const GemmProblem& p, const void* a, const void* b, void* c, hipStream_t stream) {
+template <class T, int BM, int BN, int STAGES, bool SPLIT = false>
+static int launch_dtl(const GemmProblem& p, const void* a, const void* b, void* c, hipStream_t stream, SplitK sk = SplitK{1, 0, nullptr}) {
     const uint32_t tiles_m = (p.M + BM - 1) / BM, tiles_n = (p.N + BN - 1) / BN;
     constexpr size_t tile_bytes = STAGES * (BM + BN) * 128, stage_bytes = sizeof(T) == 2 ? 2 * 4 * (BM / 2) * (BN / 2 + 8) : 0;   // the operand stages; the output staging (16-bit results)
     constexpr size_t lds_bytes = tile_bytes > stage_bytes ? tile_bytes : stage_bytes;
-    auto kernel = gemm16_dtl_kernel<T, BM, BN, STAGES, (lds_bytes <= 80 * 1024 ? 2 : 1)>;
+    auto kernel = gemm16_dtl_kernel<T, BM, BN, STAGES, (lds_bytes <= 80 * 1024 ? 2 : 1), SPLIT>;
     static std::atomic<uint64_t> configured{0};
     if (int rc = raise_lds_limit(reinterpret_cast<const void*>(kernel), lds_bytes, configured)) return rc;
-    hipLaunchKernelGGL(kernel, dim3(tiles_m * tiles_n, p.batches), dim3(256), lds_bytes, stream, static_cast<const T*>(a), static_cast<const T*>(b),
-                       static_cast<typename DtlTypes<T>::Out*>(c), p, tiles_m, tiles_n);
+    hipLaunchKernelGGL(kernel, dim3(tiles_m * tiles_n * sk.splits, p.batches), dim3(256), lds_bytes, stream, static_cast<const T*>(a), static_cast<const T*>(b),
+                       static_cast<typename DtlTypes<T>::Out*>(c), p, tiles_m, tiles_n, sk);
     return launch_status("gemm16_dtl_kernel");
 }
+
+// Whether the operands are this kernel's: both K-contiguous, whole K steps, rows that do not overlap.
+template <class T>
+static bool operands_fit(const GemmProblem& p) {
+    constexpr int step = 128 / sizeof(T);
+    if (p.a_cs != 1 || p.b_rs != 1 || p.K == 0 || p.K % step != 0 || p.row_bias) return false;
+    if (p.a_rs < static_cast<int64_t>(p.K) || p.b_cs < static_cast<int64_t>(p.K)) return false;
+    return p.a_rs < (1 << 22) && p.b_cs < (1 << 22);
+}
+
+template <class T>
+int gemm16_dtl_split(const GemmProblem& p, uint32_t splits, uint32_t k_chunk, float* partials, const void* a, const void* b, hipStream_t stream) {
+    if (!operands_fit<T>(p) || p.N % 4 != 0 || k_chunk % 64 != 0) return TANNIC_UNSUPPORTED_DTYPE;
+    return launch_dtl<T, 128, 128, 4, true>(p, a, b, nullptr, stream, SplitK{splits, k_chunk, partials});
+}
+template int gemm16_dtl_split<f16>(const GemmProblem&, uint32_t, uint32_t, float*, const void*, const void*, hipStream_t);
+template int gemm16_dtl_split<bf16>(const GemmProblem&, uint32_t, uint32_t, float*, const void*, const void*, hipStream_t);
 
 // Returns TANNIC_UNSUPPORTED_DTYPE when the problem is not this kernel's: the caller then takes the register-staged one.
 template <class T>

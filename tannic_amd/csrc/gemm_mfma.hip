@@ -190,11 +190,6 @@ using Loader = std::conditional_t<K_MAJOR, KMajorLoader<T, ROWS, THREADS, ALIGNE
 
 // WAVES_N: wavefronts along N (2 -> 256 threads, one wavefront per SIMD; 4 -> 512 threads, two per SIMD, so that
 // one wavefront's waits are covered by the other's MFMAs); always two wavefronts along M.
-// Where a block of a split product leaves its share: fp32, [split][batch][M][N].
-struct SplitK {
-    uint32_t splits, k_chunk;    // blocks per tile; K elements per block, a multiple of kBK
-    float* partials;
-};
 
 // SPLIT: several blocks share an output tile, each taking a range of K and storing its fp32 accumulators; a second
 // kernel adds the shares in split order, rounds once and writes C.
@@ -529,8 +524,10 @@ int run16_split(const GemmProblem& p, bool ak, bool bk, uint32_t splits, const v
     } else if (scratch_acquire(reinterpret_cast<void**>(&sk.partials), bytes, stream) != TANNIC_SUCCESS) {
         return TANNIC_ERROR;
     }
-    int status;
-    if (ak && bk) status = launch16<T, BM, BN, 2, true, true, true>(p, a, b, c, stream, sk);
+    int status = TANNIC_UNSUPPORTED_DTYPE;
+    if constexpr (sizeof(T) == 2 && BM == 128) status = gemm16_dtl_split<T>(p, sk.splits, sk.k_chunk, sk.partials, a, b, stream);
+    if (status != TANNIC_UNSUPPORTED_DTYPE) {}
+    else if (ak && bk) status = launch16<T, BM, BN, 2, true, true, true>(p, a, b, c, stream, sk);
     else if (ak) status = launch16<T, BM, BN, 2, true, false, true>(p, a, b, c, stream, sk);
     else if (bk) status = launch16<T, BM, BN, 2, false, true, true>(p, a, b, c, stream, sk);
     else status = launch16<T, BM, BN, 2, false, false, true>(p, a, b, c, stream, sk);
@@ -590,12 +587,15 @@ int run16(const GemmProblem& p, const void* a, const void* b, void* c, hipStream
         if ((bm == 128 && !tall) || (bm == 256 && p.M <= 192)) continue;
         const uint64_t tiles = static_cast<uint64_t>((p.M + bm - 1) / bm) * ((p.N + 127) / 128) * p.batches;
         for (uint32_t splits : {1u, 2u, 4u, 8u, 16u}) {
-            if (splits > 1 && (bm == 256 || p.row_bias || splits > p.K / 256)) break;
+            if (splits > 1 && (bm == 256 || p.row_bias || splits > p.K / (sizeof(T) == 4 ? 64 : 256))) break;
             const double blocks = static_cast<double>(tiles) * splits;
             const double rounds = static_cast<double>((static_cast<uint64_t>(blocks) + 255) / 256);
             // a step costs more the more compute units pull operands through the L2s at the same time
             const double busy = blocks < 256.0 ? blocks / 256.0 : 1.0;
-            const double step_us = bm == 256 ? 1.0 : bm == 128 ? 0.375 + 0.175 * busy : 0.30 + 0.075 * busy;
+            double step_us = bm == 256 ? 1.0 : bm == 128 ? 0.375 + 0.175 * busy : 0.30 + 0.075 * busy;
+            // fp32: the matrix pipe, sixteen times slower than for the 16-bit types, sets the pace of a step
+            // (2 * bm * 128 * 64 flops at 157.3 TFLOP/s over 256 compute units)
+            if constexpr (sizeof(T) == 4) step_us = std::max(step_us, 2.0 * bm * 128 * 64 / (157.3e6 / 256));
             double cost = rounds * (steps_all / splits) * step_us + 5.0;
             if (splits > 1) cost += 4.0 + (splits + 0.5) * static_cast<double>(p.M) * p.N * p.batches * 4.0 / 5.0e6;
             if (cost < best_cost) { best_cost = cost; best_bm = bm; best_splits = splits; }

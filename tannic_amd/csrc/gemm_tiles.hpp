@@ -74,4 +74,11 @@ __device__ inline void static_for(F&& f) {
 // that 16 consecutive rows of one logical chunk land in 16 different slots.
 template <class T> __device__ inline uint32_t tile_offset(uint32_t row, uint32_t chunk) { return row * kBKof<T> + ((chunk ^ ((row >> 1) & 7u)) * kChunkOf<T>); }
 
+
+// Where a block of a split product leaves its share: fp32, [split][batch][M][N].
+struct SplitK {
+    uint32_t splits, k_chunk;    // blocks per tile; K elements per block, a multiple of kBK
+    float* partials;
+};
+
 }  // namespace th
