@@ -128,14 +128,18 @@ __global__ __launch_bounds__(kK1Threads) void conv2d_k1_kernel(const T* x, const
         // tile number k of this block into register set `set`
         auto fetch = [&](auto set_, uint32_t k) {
             constexpr int set = decltype(set_)::value;
-            // never skipped: the count of memory operations between a tile's loads and their use is the same on every
-            // path, which lets the wait before the use leave the younger loads and stores in flight
-            locate(first + (k < count ? k : count - 1) * q.workers);
+            // Never skipped: the count of memory operations between a tile's loads and their use is the same on every
+            // path, which lets the wait before the use leave the younger loads and stores in flight.  Past the block's
+            // last tile every lane loads the signal's first 16 bytes: one cache line an instruction, never used.
+            const bool real = k < count;
+            locate(first + (real ? k : 0) * q.workers);
+            const int64_t step = real ? cstep : 0;
+            if (!real) src = x;
 #pragma unroll
             for (int b = 0; b < BLOCKS; ++b) {
                 const uint32_t block = block_is_mine(b) ? kb + 16 * b : kb % (C / 8);
 #pragma unroll
-                for (int kk = 0; kk < 8; ++kk) raw[set][b][kk] = *reinterpret_cast<const uint4p*>(src + static_cast<int64_t>(block * 8 + kk) * cstep);
+                for (int kk = 0; kk < 8; ++kk) raw[set][b][kk] = *reinterpret_cast<const uint4p*>(src + static_cast<int64_t>(block * 8 + kk) * step);
             }
         };
         // The records of two pixels of a transposed micro-block (this thread's 8 channels each): two 16-byte LDS writes.
