@@ -42,7 +42,9 @@ UNITS = [
     ("gemm.hip", "gemm.o", []),
     ("gemm_mfma.hip", "gemm_mfma.o", []),
     ("gemm_skinny.hip", "gemm_skinny.o", []),
-    ("gemm_dtl.hip", "gemm_dtl.o", []),
+    ("gemm_dtl.hip", "gemm_dtl.o", ["-DTH_DTL_PART=0"]),
+    ("gemm_dtl.hip", "gemm_dtl_krows_f16.o", ["-DTH_DTL_PART=1"]),
+    ("gemm_dtl.hip", "gemm_dtl_krows_bf16.o", ["-DTH_DTL_PART=2"]),
     ("probes.hip", "probes.o", []),
     ("conv2d.hip", "conv2d.o", []),
     ("conv2d_mfma.hip", "conv2d_mfma.o", []),

@@ -23,6 +23,15 @@
 // 4 * (l / 16) .. + 3.  Sums are formed in the same order of k as in gemm16_kernel: results are bit-identical.
 //
 // int8 x int8 -> int32 runs the same kernel on v_mfma_i32_16x16x64_i8: a 128-byte tile row is 128 elements, a k-slice 64.
+//
+// An operand that is contiguous along its other index (A stored as [K][M], B as [K][N]: the X . W, X^T . W and X^T . W^T
+// products) keeps that order in LDS: a tile is 64 k-rows of BM (BN) elements, filled by the same loads, and a fragment
+// is two ds_read_b64_tr_b16, the transposing LDS read of gfx950: in every group of 16 lanes, lane j supplies the
+// address of four consecutive elements and receives element j % 4 of the lanes j / 4, j / 4 + 4, j / 4 + 8, j / 4 + 12.
+// With lane 16 g + m pointing at row 8 g + m / 4 (+ 4 for the second read), elements 4 * (m % 4) .. + 3 of the
+// fragment's 16 columns, lane 16 g + j ends up with column j, k = 8 g .. 8 g + 7: the MFMA's operand layout.  The
+// 32-byte units of a k-row are XOR-swizzled by (k % 4) + 4 * ((k / 8) % 2), on the global side as above, so that the 32
+// lanes of a read pass (rows 0..3 and 8..11, or 16..19 and 24..27, 32 bytes each) cover all banks.
 #include "gemm_tiles.hpp"
 
 namespace th {
@@ -59,7 +68,8 @@ template <class T> __device__ inline void mfma16x16_in_place(typename DtlTypes<T
 // BM x BN: 256 x 256, 256 x 128 or 128 x 128 (2 x 2 wavefronts each).  The smaller tiles are for products with too few
 // large tiles to fill the chip; two workgroups of the smallest share a compute unit.
 // SPLIT: `sk.splits` workgroups share a tile, each taking sk.k_chunk of K and storing its fp32 accumulators.
-template <class T, int BM, int BN, int STAGES, int BLOCKS_PER_CU, bool SPLIT = false>
+// A_T, B_T: the operand is contiguous along M (N) and its tile is kept as k-rows.
+template <class T, int BM, int BN, int STAGES, int BLOCKS_PER_CU, bool SPLIT = false, bool A_T = false, bool B_T = false>
 __global__ __launch_bounds__(256, BLOCKS_PER_CU) void gemm16_dtl_kernel(const T* A, const T* B, typename DtlTypes<T>::Out* C, GemmProblem p, uint32_t tiles_m, uint32_t tiles_n, SplitK sk) {
 #if defined(__HIP_DEVICE_COMPILE__)   // the host pass needs the launch stub only (and loses it over the body's device-only builtins)
     constexpr int ES = sizeof(T), BK = 128 / ES, WAVES_N = 2;   // a tile row is 128 bytes: 64 elements of 16 bits, 128 of 8
@@ -78,33 +88,45 @@ __global__ __launch_bounds__(256, BLOCKS_PER_CU) void gemm16_dtl_kernel(const T*
     // this workgroup's range of K: all of it, or its share (whole steps)
     const uint32_t k_first = SPLIT ? split * sk.k_chunk : 0;
     const uint32_t steps = (SPLIT ? (p.K - k_first < sk.k_chunk ? p.K - k_first : sk.k_chunk) : p.K) / BK;
-    const uint32_t k_first_bytes = k_first * ES;
 
     const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
     const int wm = (wave / WAVES_N) * WM, wn = (wave % WAVES_N) * WN;
     const uint32_t frag_row = lane % 16, frag_chunk = lane / 16;
 
     // Buffer resources starting at the tile's first row: offsets stay below 2^31 and rows past the end are out of range.
+    // (A k-row operand starts at the tile's first column; its extent is a whole number of tiles.)
     const T* a_base = A + oa + static_cast<int64_t>(m0) * p.a_rs;
     const T* b_base = B + ob + static_cast<int64_t>(n0) * p.b_cs;
     auto records = [](uint64_t rows_left, int64_t stride, uint32_t K) -> uint32_t {
         const uint64_t bytes = ((rows_left - 1) * static_cast<uint64_t>(stride) + K) * ES;
         return bytes > 0xFFFFFFFFull ? 0xFFFFFFFFu : static_cast<uint32_t>(bytes);
     };
-    const __amdgpu_buffer_rsrc_t rsrc_a = __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(a_base), 0, records(p.M - m0, p.a_rs, p.K), 0x00020000);
-    const __amdgpu_buffer_rsrc_t rsrc_b = __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(b_base), 0, records(p.N - n0, p.b_cs, p.K), 0x00020000);
-    // Load j of a wavefront fills eight rows of a tile (j < LOADS_A: rows 8 * (LOADS_A * wave + j) .. + 7 of A's, then B's
-    // likewise); the lane's byte offset from the tile's first row:
+    const __amdgpu_buffer_rsrc_t rsrc_a = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<T*>(a_base), 0, A_T ? records(p.K, p.a_cs, BM) : records(p.M - m0, p.a_rs, p.K), 0x00020000);
+    const __amdgpu_buffer_rsrc_t rsrc_b = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<T*>(b_base), 0, B_T ? records(p.K, p.b_rs, BN) : records(p.N - n0, p.b_cs, p.K), 0x00020000);
+    // Load j of a wavefront fills 1 KB of a tile (j < LOADS_A: bytes 1024 * (LOADS_A * wave + j) .. of A's, then B's
+    // likewise): eight rows of 128 bytes, or 1024 / (2 BM) k-rows; the lane's byte offset from the tile's first element:
     uint32_t voff[LOADS];
 #pragma unroll
     for (int j = 0; j < LOADS; ++j) {
-        const uint32_t row = (j < LOADS_A ? wave * LOADS_A + j : wave * LOADS_B + (j - LOADS_A)) * 8 + lane / 8;
-        const uint32_t chunk = (lane % 8) ^ ((row >> 1) & 7u);
-        voff[j] = row * static_cast<uint32_t>(j < LOADS_A ? p.a_rs : p.b_cs) * ES + chunk * 16;
+        const bool of_a = j < LOADS_A;
+        const uint32_t slot = (of_a ? wave * LOADS_A + j : wave * LOADS_B + (j - LOADS_A)) * 64 + lane;   // 16-byte slot of the tile
+        if ((of_a && A_T) || (!of_a && B_T)) {
+            const uint32_t per_row = (of_a ? BM : BN) / 8, k = slot / per_row, in_row = slot % per_row;
+            const uint32_t unit = (in_row / 2) ^ ((k % 4) + 4 * ((k / 8) % 2));
+            voff[j] = k * static_cast<uint32_t>(of_a ? p.a_cs : p.b_rs) * ES + (unit * 2 + in_row % 2) * 16;
+        } else {
+            const uint32_t row = slot / 8;
+            const uint32_t chunk = (lane % 8) ^ ((row >> 1) & 7u);
+            voff[j] = row * static_cast<uint32_t>(of_a ? p.a_rs : p.b_cs) * ES + chunk * 16;
+        }
     }
-    auto issue_load = [&](int j, uint32_t stage, uint32_t k_bytes) {
+    // the tile that starts at element k of K
+    const uint32_t a_kstep = A_T ? static_cast<uint32_t>(p.a_cs) * ES : ES, b_kstep = B_T ? static_cast<uint32_t>(p.b_rs) * ES : ES;
+    auto issue_load = [&](int j, uint32_t stage, uint32_t k) {
         const uint32_t at = stage * (STAGE * ES) + (j < LOADS_A ? (wave * LOADS_A + j) * 1024 : A_TILE * ES + (wave * LOADS_B + (j - LOADS_A)) * 1024);
-        __builtin_amdgcn_raw_ptr_buffer_load_lds(j < LOADS_A ? rsrc_a : rsrc_b, (lds_void)(lds_raw + at), 16, voff[j], k_bytes, 0, 0);
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(j < LOADS_A ? rsrc_a : rsrc_b, (lds_void)(lds_raw + at), 16, voff[j], k * (j < LOADS_A ? a_kstep : b_kstep), 0, 0);
     };
 
     using Acc = typename DtlTypes<T>::Acc;
@@ -132,7 +154,7 @@ __global__ __launch_bounds__(256, BLOCKS_PER_CU) void gemm16_dtl_kernel(const T*
     for (int t = 0; t < STAGES - 1; ++t) {
         if (static_cast<uint32_t>(t) < steps) {
 #pragma unroll
-            for (int j = 0; j < LOADS; ++j) issue_load(j, t, k_first_bytes + t * 128);
+            for (int j = 0; j < LOADS; ++j) issue_load(j, t, k_first + t * BK);
         }
     }
     wait_loads(steps < static_cast<uint32_t>(STAGES - 1));
@@ -141,17 +163,45 @@ __global__ __launch_bounds__(256, BLOCKS_PER_CU) void gemm16_dtl_kernel(const T*
     constexpr int PER_KS = TM * TN;   // MFMAs per k-slice
     constexpr int LOAD_EVERY = PER_KS / LOADS > 0 ? PER_KS / LOADS : 1;   // the loads of a step go out during its first half
     uint4v fa[2][TM], fb[2][TN];
-    auto read_fragments = [&](const T* a_tile, const T* b_tile, int ks, int into) {
+    // fragment of the 16 rows (columns) from `first` on, k-slice ks of a tile
+    const uint32_t tr_unit = (frag_row / 4) + 4 * (frag_chunk % 2), tr_row = 8 * frag_chunk + frag_row / 4, tr_quad = (frag_row % 4) * 4;
+    // The transposing reads are written as assembly: as a builtin, every such read that follows a global -> LDS load in
+    // program order is made to wait for that load (the two might touch the same LDS bytes, for all the compiler knows),
+    // which puts the memory latency into every step.  The price: the compiler does not count them in lgkmcnt, so the
+    // MFMAs of a half are preceded by an explicit wait for the reads issued during the half before.
+    const uint32_t lds_address = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((lds_void)(lds_raw)));   // of the dynamic area
+    auto fragment = [&](const T* tile, auto transposed_tag, auto width_tag, uint32_t first, auto ks_tag) -> uint4v {
+        constexpr int ks = decltype(ks_tag)::value;
+        if constexpr (decltype(transposed_tag)::value) {
+            constexpr uint32_t WIDTH = decltype(width_tag)::value;
+            typedef unsigned int uint2v __attribute__((ext_vector_type(2)));
+            const uint32_t at = lds_address + static_cast<uint32_t>(tile - lds) * ES + (tr_row * WIDTH + ((first / 16) ^ tr_unit) * 16 + tr_quad) * ES;
+            uint2v low, high;
+            asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(low) : "v"(at), "n"(ks * 32 * WIDTH * ES));
+            asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(high) : "v"(at), "n"((ks * 32 + 4) * WIDTH * ES));
+            return uint4v{low[0], low[1], high[0], high[1]};
+        } else {
+            return *reinterpret_cast<const uint4v*>(tile + tile_offset<T>(first + frag_row, ks * 4 + frag_chunk));
+        }
+    };
+    auto wait_fragments = [] {
+        if constexpr (A_T || B_T) asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    };
+    using ATag = std::integral_constant<bool, A_T>;
+    using BTag = std::integral_constant<bool, B_T>;
+    using AWidth = std::integral_constant<uint32_t, BM>;
+    using BWidth = std::integral_constant<uint32_t, BN>;
+    auto read_fragments = [&](const T* a_tile, const T* b_tile, auto ks_tag, int into) {
 #pragma unroll
-        for (int x = 0; x < TM; ++x) fa[into][x] = *reinterpret_cast<const uint4v*>(a_tile + tile_offset<T>(wm + x * 16 + frag_row, ks * 4 + frag_chunk));
+        for (int x = 0; x < TM; ++x) fa[into][x] = fragment(a_tile, ATag{}, AWidth{}, wm + x * 16, ks_tag);
 #pragma unroll
-        for (int y = 0; y < TN; ++y) fb[into][y] = *reinterpret_cast<const uint4v*>(b_tile + tile_offset<T>(wn + y * 16 + frag_row, ks * 4 + frag_chunk));
+        for (int y = 0; y < TN; ++y) fb[into][y] = fragment(b_tile, BTag{}, BWidth{}, wn + y * 16, ks_tag);
     };
     // fragment read r of a k-slice: the first A fragment and the B fragments first, in the order the MFMAs want them
-    auto read_one = [&](const T* a_tile, const T* b_tile, int ks, int into, int r) {
-        if (r == 0) fa[into][0] = *reinterpret_cast<const uint4v*>(a_tile + tile_offset<T>(wm + frag_row, ks * 4 + frag_chunk));
-        else if (r <= TN) fb[into][r - 1] = *reinterpret_cast<const uint4v*>(b_tile + tile_offset<T>(wn + (r - 1) * 16 + frag_row, ks * 4 + frag_chunk));
-        else fa[into][r - TN] = *reinterpret_cast<const uint4v*>(a_tile + tile_offset<T>(wm + (r - TN) * 16 + frag_row, ks * 4 + frag_chunk));
+    auto read_one = [&](const T* a_tile, const T* b_tile, auto ks_tag, int into, int r) {
+        if (r == 0) fa[into][0] = fragment(a_tile, ATag{}, AWidth{}, wm, ks_tag);
+        else if (r <= TN) fb[into][r - 1] = fragment(b_tile, BTag{}, BWidth{}, wn + (r - 1) * 16, ks_tag);
+        else fa[into][r - TN] = fragment(a_tile, ATag{}, AWidth{}, wm + (r - TN) * 16, ks_tag);
     };
     // A step issues the MFMAs of the second k-slice of the previous tile (its fragments are in registers since before
     // the barrier) and those of the first slice of this tile.  Behind the first MFMAs of each half go the fragment
@@ -162,17 +212,18 @@ __global__ __launch_bounds__(256, BLOCKS_PER_CU) void gemm16_dtl_kernel(const T*
         const T* a_tile = lds + cur * STAGE;
         const T* b_tile = a_tile + A_TILE;
         // the first step has no MFMAs in its first half: its fragment reads go out at once
-        if constexpr (FIRST) read_fragments(a_tile, b_tile, 0, 0);
+        if constexpr (FIRST) read_fragments(a_tile, b_tile, std::integral_constant<int, 0>{}, 0);
         __builtin_amdgcn_sched_barrier(0);
         static_for<2 * PER_KS>([&](auto m_tag) {
             constexpr int m = decltype(m_tag)::value;
             constexpr int group = m / PER_KS;           // 0: slice 1 of the previous tile (set 1); 1: slice 0 of this tile (set 0)
             constexpr int q = m % PER_KS, i = q / TN, j = q % TN;
             constexpr int now = group == 0 ? 1 : 0;
+            if constexpr (q == 0) wait_fragments();
             if constexpr (!(FIRST && group == 0)) mfma16x16_in_place<T>(acc[i][j], fb[now][j], fa[now][i]);
-            if constexpr (q < TM + TN && !(FIRST && group == 0)) read_one(a_tile, b_tile, group == 0 ? 0 : 1, group == 0 ? 0 : 1, q);
+            if constexpr (q < TM + TN && !(FIRST && group == 0)) read_one(a_tile, b_tile, std::integral_constant<int, group == 0 ? 0 : 1>{}, group == 0 ? 0 : 1, q);
             constexpr int slot = FIRST ? m - PER_KS : m;
-            if constexpr (FETCH && slot >= 0 && slot % LOAD_EVERY == LOAD_EVERY / 2 && slot / LOAD_EVERY < LOADS) issue_load(slot / LOAD_EVERY, fill, k_first_bytes + (s + STAGES - 1) * 128);
+            if constexpr (FETCH && slot >= 0 && slot % LOAD_EVERY == LOAD_EVERY / 2 && slot / LOAD_EVERY < LOADS) issue_load(slot / LOAD_EVERY, fill, k_first + (s + STAGES - 1) * BK);
             __builtin_amdgcn_sched_barrier(0);
         });
         wait_loads(!FETCH);    // tile s+1 is in LDS (steps that issue no loads wait for all that are left)
@@ -187,6 +238,7 @@ __global__ __launch_bounds__(256, BLOCKS_PER_CU) void gemm16_dtl_kernel(const T*
     for (s = 1, cur = next(cur), fill = next(fill); s + STAGES - 1 < steps; ++s, cur = next(cur), fill = next(fill)) step(s, cur, fill, No{}, Yes{});
     for (; s < steps; ++s, cur = next(cur), fill = next(fill)) step(s, cur, fill, No{}, No{});
     // the second slice of the last tile
+    wait_fragments();
 #pragma unroll
     for (int i = 0; i < TM; ++i)
 #pragma unroll
@@ -247,12 +299,12 @@ __global__ __launch_bounds__(256, BLOCKS_PER_CU) void gemm16_dtl_kernel(const T*
 #endif
 }
 
-template <class T, int BM, int BN, int STAGES, bool SPLIT = false>
+template <class T, int BM, int BN, int STAGES, bool SPLIT = false, bool A_T = false, bool B_T = false>
 static int launch_dtl(const GemmProblem& p, const void* a, const void* b, void* c, hipStream_t stream, SplitK sk = SplitK{1, 0, nullptr}) {
     const uint32_t tiles_m = (p.M + BM - 1) / BM, tiles_n = (p.N + BN - 1) / BN;
     constexpr size_t tile_bytes = STAGES * (BM + BN) * 128, stage_bytes = sizeof(T) == 2 ? 2 * 4 * (BM / 2) * (BN / 2 + 8) : 0;   // the operand stages; the output staging (16-bit results)
     constexpr size_t lds_bytes = tile_bytes > stage_bytes ? tile_bytes : stage_bytes;
-    auto kernel = gemm16_dtl_kernel<T, BM, BN, STAGES, (lds_bytes <= 80 * 1024 ? 2 : 1), SPLIT>;
+    auto kernel = gemm16_dtl_kernel<T, BM, BN, STAGES, (lds_bytes <= 80 * 1024 ? 2 : 1), SPLIT, A_T, B_T>;
     static std::atomic<uint64_t> configured{0};
     if (int rc = raise_lds_limit(reinterpret_cast<const void*>(kernel), lds_bytes, configured)) return rc;
     hipLaunchKernelGGL(kernel, dim3(tiles_m * tiles_n * sk.splits, p.batches), dim3(256), lds_bytes, stream, static_cast<const T*>(a), static_cast<const T*>(b),
@@ -260,19 +312,69 @@ static int launch_dtl(const GemmProblem& p, const void* a, const void* b, void* 
     return launch_status("gemm16_dtl_kernel");
 }
 
-// Whether the operands are this kernel's: both K-contiguous, whole K steps, rows that do not overlap.
+// This file is compiled in parts (TH_DTL_PART): 0 holds the entry points and the kernels for operands contiguous along
+// K, 1 and 2 the kernels with k-row operands for float16 and bfloat16.
+#ifndef TH_DTL_PART
+#define TH_DTL_PART 0
+#endif
+
+// the kernels with k-row operands: a_t / b_t say which operand is one; splits == 0: whole K per workgroup
 template <class T>
-static bool operands_fit(const GemmProblem& p) {
+int gemm16_dtl_krows(const GemmProblem& p, int bm, int bn, bool a_t, bool b_t, SplitK sk, const void* a, const void* b, void* c, hipStream_t stream);
+
+#if TH_DTL_PART != 0
+template <class T, int BM, int BN, int STAGES, bool SPLIT>
+static int launch_dtl_krows(const GemmProblem& p, bool a_t, bool b_t, SplitK sk, const void* a, const void* b, void* c, hipStream_t stream) {
+    if (a_t && b_t) return launch_dtl<T, BM, BN, STAGES, SPLIT, true, true>(p, a, b, c, stream, sk);
+    if (a_t) return launch_dtl<T, BM, BN, STAGES, SPLIT, true, false>(p, a, b, c, stream, sk);
+    return launch_dtl<T, BM, BN, STAGES, SPLIT, false, true>(p, a, b, c, stream, sk);
+}
+
+template <class T>
+int gemm16_dtl_krows(const GemmProblem& p, int bm, int bn, bool a_t, bool b_t, SplitK sk, const void* a, const void* b, void* c, hipStream_t stream) {
+    if (sk.splits) return bm == 128 && bn == 128 ? launch_dtl_krows<T, 128, 128, 4, true>(p, a_t, b_t, sk, a, b, c, stream) : TANNIC_UNSUPPORTED_DTYPE;
+    sk.splits = 1;
+    if (bm == 256 && bn == 256) return launch_dtl_krows<T, 256, 256, 2, false>(p, a_t, b_t, sk, a, b, c, stream);
+    if (bm == 256 && bn == 128) return launch_dtl_krows<T, 256, 128, 3, false>(p, a_t, b_t, sk, a, b, c, stream);
+    if (bm == 128 && bn == 128) return launch_dtl_krows<T, 128, 128, 4, false>(p, a_t, b_t, sk, a, b, c, stream);
+    return TANNIC_UNSUPPORTED_DTYPE;
+}
+#if TH_DTL_PART == 1
+template int gemm16_dtl_krows<f16>(const GemmProblem&, int, int, bool, bool, SplitK, const void*, const void*, void*, hipStream_t);
+#else
+template int gemm16_dtl_krows<bf16>(const GemmProblem&, int, int, bool, bool, SplitK, const void*, const void*, void*, hipStream_t);
+#endif
+
+#else   // TH_DTL_PART == 0
+
+// Whether the operands are this kernel's (tile bm x bn): each contiguous along K, or (16-bit types) along its other
+// index; whole K steps; rows that do not overlap; offsets that fit 32 bits.
+template <class T>
+static bool operands_fit(const GemmProblem& p, int bm, int bn, bool& a_t, bool& b_t) {
+    a_t = p.a_cs != 1;
+    b_t = p.b_rs != 1;
+    if ((a_t || b_t) && sizeof(T) != 2) return false;
+    if ((a_t && p.a_rs != 1) || (b_t && p.b_cs != 1)) return false;
     constexpr int step = 128 / sizeof(T);
-    if (p.a_cs != 1 || p.b_rs != 1 || p.K == 0 || p.K % step != 0 || p.row_bias) return false;
-    if (p.a_rs < static_cast<int64_t>(p.K) || p.b_cs < static_cast<int64_t>(p.K)) return false;
-    return p.a_rs < (1 << 22) && p.b_cs < (1 << 22);
+    if (p.K == 0 || p.K % step != 0 || p.row_bias) return false;       // whole K steps only, no start values
+    // a row's offset inside a tile is a 32-bit byte count; rows must not overlap (the range check relies on it)
+    if (!a_t && (p.a_rs < static_cast<int64_t>(p.K) || p.a_rs >= (1 << 22))) return false;
+    if (!b_t && (p.b_cs < static_cast<int64_t>(p.K) || p.b_cs >= (1 << 22))) return false;
+    // k-row operands: whole tiles along the contiguous index (a tile's loads do not look at it), 32-bit byte offsets along K
+    if (a_t && (p.M % bm != 0 || p.a_cs < static_cast<int64_t>(p.M) || static_cast<uint64_t>(p.K) * p.a_cs * sizeof(T) >= (1ull << 32))) return false;
+    if (b_t && (p.N % bn != 0 || p.b_rs < static_cast<int64_t>(p.N) || static_cast<uint64_t>(p.K) * p.b_rs * sizeof(T) >= (1ull << 32))) return false;
+    return true;
 }
 
 template <class T>
 int gemm16_dtl_split(const GemmProblem& p, uint32_t splits, uint32_t k_chunk, float* partials, const void* a, const void* b, hipStream_t stream) {
-    if (!operands_fit<T>(p) || p.N % 4 != 0 || k_chunk % 64 != 0) return TANNIC_UNSUPPORTED_DTYPE;
-    return launch_dtl<T, 128, 128, 4, true>(p, a, b, nullptr, stream, SplitK{splits, k_chunk, partials});
+    bool a_t, b_t;
+    if (!operands_fit<T>(p, 128, 128, a_t, b_t) || p.N % 4 != 0 || k_chunk % 64 != 0) return TANNIC_UNSUPPORTED_DTYPE;
+    const SplitK sk{splits, k_chunk, partials};
+    if constexpr (sizeof(T) == 2) {
+        if (a_t || b_t) return gemm16_dtl_krows<T>(p, 128, 128, a_t, b_t, sk, a, b, nullptr, stream);
+    }
+    return launch_dtl<T, 128, 128, 4, true>(p, a, b, nullptr, stream, sk);
 }
 template int gemm16_dtl_split<f16>(const GemmProblem&, uint32_t, uint32_t, float*, const void*, const void*, hipStream_t);
 template int gemm16_dtl_split<bf16>(const GemmProblem&, uint32_t, uint32_t, float*, const void*, const void*, hipStream_t);
@@ -280,15 +382,15 @@ template int gemm16_dtl_split<bf16>(const GemmProblem&, uint32_t, uint32_t, floa
 // Returns TANNIC_UNSUPPORTED_DTYPE when the problem is not this kernel's: the caller then takes the register-staged one.
 template <class T>
 int gemm16_dtl(const GemmProblem& p, int bm, int bn, const void* a, const void* b, void* c, hipStream_t stream) {
-    if (p.a_cs != 1 || p.b_rs != 1) return TANNIC_UNSUPPORTED_DTYPE;                     // both operands K-contiguous
-    constexpr int step = 128 / sizeof(T), quad = 16 / sizeof(typename DtlTypes<T>::Out);   // K elements per step; results per 16-byte store
-    if (p.K == 0 || p.K % step != 0 || p.row_bias) return TANNIC_UNSUPPORTED_DTYPE;       // whole K steps only, no start values
+    bool a_t, b_t;
+    if (!operands_fit<T>(p, bm, bn, a_t, b_t)) return TANNIC_UNSUPPORTED_DTYPE;
+    constexpr int quad = 16 / sizeof(typename DtlTypes<T>::Out);   // results per 16-byte store
     if (p.N % quad != 0 || p.c_rs % quad != 0 || reinterpret_cast<uintptr_t>(c) % 16 != 0) return TANNIC_UNSUPPORTED_DTYPE;
     for (int d = 0; d < p.batch_rank; ++d)
         if (p.c_bs[d] % quad != 0) return TANNIC_UNSUPPORTED_DTYPE;
-    // a row's offset inside a tile is a 32-bit byte count; rows must not overlap (the range check relies on it)
-    if (p.a_rs < static_cast<int64_t>(p.K) || p.b_cs < static_cast<int64_t>(p.K)) return TANNIC_UNSUPPORTED_DTYPE;
-    if (p.a_rs >= (1 << 22) || p.b_cs >= (1 << 22)) return TANNIC_UNSUPPORTED_DTYPE;
+    if constexpr (sizeof(T) == 2) {
+        if (a_t || b_t) return gemm16_dtl_krows<T>(p, bm, bn, a_t, b_t, SplitK{0, 0, nullptr}, a, b, c, stream);
+    }
     // as many stages as LDS holds (160 KB): the smaller the tile, the shorter its step and the more steps a load needs to arrive
     if (bm == 256 && bn == 256) return launch_dtl<T, 256, 256, 2>(p, a, b, c, stream);
     if (bm == 256 && bn == 128) return launch_dtl<T, 256, 128, 3>(p, a, b, c, stream);
@@ -314,5 +416,7 @@ int gemm_mfma_int8(const GemmProblem& p, const void* a, const void* b, void* c, 
     if (p.M > 32) return gemm16_dtl<int8_t>(p, 128, 128, a, b, c, stream);
     return TANNIC_UNSUPPORTED_DTYPE;
 }
+
+#endif   // TH_DTL_PART == 0
 
 }  // namespace th

@@ -148,6 +148,30 @@ def test_operand_with_fewer_batch_dims_steps_by_its_own_batch_stride(device):
         support.assert_close(got, np.matmul(rb.swapaxes(-1, -2), ra.swapaxes(-1, -2)), rtol, atol, f"rank 4 x rank 3 {dtype}")
 
 
+@pytest.mark.parametrize("shape", [(1024, 2048, 512), (2048, 4096, 256), (512, 4096, 1024), (4096, 4096, 128), (25, 512, 1024, 64)], ids=str)
+@pytest.mark.parametrize("dtype", [ta.float16, ta.bfloat16], ids=str)
+def test_operands_contiguous_along_m_or_n_on_direct_tiles(device, dtype, shape):
+    """X . W, X^T . W and X^T . W^T with whole tiles along M and N, at sizes that choose each tile of the direct-to-LDS
+    kernel (128 x 128, 256 x 128, K shared between workgroups, 256 x 256, batches): operand tiles kept as k-rows and
+    read with the transposing LDS read.  Sums run over k in the same order as for X . W^T, so the four layouts agree
+    bit for bit; X . W^T itself is checked against float64 on sampled rows."""
+    *batch, m, n, k = shape
+    x = support.values_for(dtype, SEED, 5, (*batch, m, k), -1, 1)
+    w = support.values_for(dtype, SEED, 6, (*batch, k, n), -1, 1)
+    hx, dx = support.both(x, dtype, device)
+    _, dxt = support.both(np.ascontiguousarray(np.swapaxes(x, -1, -2)), dtype, device)
+    hw, dw = support.both(w, dtype, device)
+    _, dwt = support.both(np.ascontiguousarray(np.swapaxes(w, -1, -2)), dtype, device)
+    nt = ops.matmul(dx, dwt.transpose(-1, -2)).numpy()
+    rows = np.random.default_rng(SEED).choice(m, 32, replace=False)
+    exact = np.matmul(hx.numpy().astype(np.float64)[..., rows, :], hw.numpy().astype(np.float64))
+    rtol = 2e-3 if dtype is ta.float16 else 2.0 ** -7
+    support.assert_close(nt[..., rows, :], exact, rtol, 1e-3 * np.sqrt(k), f"nt {dtype} {shape}")
+    for name, a, b in (("nn", dx, dw), ("tn", dxt.transpose(-1, -2), dw), ("tt", dxt.transpose(-1, -2), dwt.transpose(-1, -2))):
+        got = ops.matmul(a, b).numpy()
+        support.assert_bit_exact(got, nt, f"{name} against nt, {dtype} {shape}")
+
+
 def test_integer_valued_fp16_gemm_is_exact(device):
     """Small integers: every product and partial sum is exact in fp32, so any order of summation agrees."""
     a = support.integers(SEED, 3, (192, 320), -4, 4)
