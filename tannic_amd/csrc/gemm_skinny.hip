@@ -10,7 +10,7 @@
 // wavefront are in flight.  The eight partial 16x16 tiles meet in LDS, the
 // first wavefront adds them, rounds once and stores four consecutive columns
 // per lane.
-#include "gemm_common.hpp"
+#include "gemm_tiles.hpp"
 
 namespace th {
 
@@ -123,6 +123,142 @@ __global__ __launch_bounds__(64 * kSkinnyWaves) void gemm_skinny_kernel(const T*
     }
 }
 
+// The same product with whole K windows of 64 (K a multiple of 64): the operands come in by direct global -> LDS loads.
+//
+// The kernel above asks for 16 bytes per lane with sixteen rows per instruction: 64 separate requests, and every
+// 128-byte line of W is asked for eight times.  Each request is a tag lookup in the vector cache, and at one lookup a
+// clock those lookups, not HBM, set the time.  Here a load instruction covers eight whole rows of a window (eight
+// lanes per 128-byte line: eight requests), and LDS does the regrouping into MFMA fragments: a wavefront owns a ring
+// of STAGES windows (per window 2 KB for each 16-row block of W and of x, rows XOR-swizzled like the tiles of the
+// large kernels, on the global side), keeps STAGES - 1 windows on their way and waits, by vmcnt, for the oldest only.
+// No barrier until the four wavefronts, which split K, add up their tiles.
+typedef __attribute__((address_space(3))) void* skinny_lds_void;
+constexpr int kStreamWaves = 4;
+constexpr int kStreamBytesPerWave = 32 * 1024;
+
+template <class T, int MB, int NB>
+__global__ __launch_bounds__(64 * kStreamWaves) void gemm_skinny_stream_kernel(const T* x, const T* w, T* c, GemmProblem p, uint32_t windows_per_wave) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    constexpr int BLOCKS = MB + NB;                       // 16-row blocks per window: W's, then x's
+    constexpr int STAGE_BYTES = BLOCKS * 2048, STAGES = kStreamBytesPerWave / STAGE_BYTES, LOADS = 2 * BLOCKS;
+    static_assert(STAGES >= 3, "a ring of at least three windows");
+    extern __shared__ __align__(16) unsigned char skinny_lds[];
+    int64_t ox, ow, oc;
+    batch_offsets(p, blockIdx.y, ox, ow, oc);
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x / 64), lane = threadIdx.x % 64;
+    const uint32_t r = lane % 16, kc = lane / 16;
+    const uint32_t n0 = blockIdx.x * 16 * NB;
+    unsigned char* ring = skinny_lds + wave * kStreamBytesPerWave;
+
+    // buffer resources from the block's first row of W and from x: rows past the end read zeros
+    auto records = [](uint64_t rows, int64_t pitch, uint32_t K) -> uint32_t {
+        const uint64_t bytes = ((rows - 1) * static_cast<uint64_t>(pitch) + K) * sizeof(T);
+        return bytes > 0xFFFFFFFFull ? 0xFFFFFFFFu : static_cast<uint32_t>(bytes);
+    };
+    const __amdgpu_buffer_rsrc_t rsrc_w = __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(w + ow + static_cast<int64_t>(n0) * p.b_cs), 0, records(p.N - n0, p.b_cs, p.K), 0x00020000);
+    const __amdgpu_buffer_rsrc_t rsrc_x = __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(x + ox), 0, records(p.M, p.a_rs, p.K), 0x00020000);
+    // load j of a window: rows 8 (j % 2) .. + 7 of block j / 2; the lane's row and its (swizzled) 16-byte chunk
+    uint32_t voff[LOADS];
+#pragma unroll
+    for (int j = 0; j < LOADS; ++j) {
+        const uint32_t row = (j % 2) * 8 + lane / 8, chunk = (lane % 8) ^ ((row >> 1) & 7u);
+        const bool of_w = j / 2 < NB;
+        const uint32_t block_row = (of_w ? j / 2 : j / 2 - NB) * 16 + row;
+        voff[j] = block_row * static_cast<uint32_t>(of_w ? p.b_cs : p.a_rs) * sizeof(T) + chunk * 16;
+    }
+    auto issue = [&](uint32_t window, uint32_t stage) {
+        const uint32_t k_bytes = window * 128;
+#pragma unroll
+        for (int j = 0; j < LOADS; ++j)
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(j / 2 < NB ? rsrc_w : rsrc_x, (skinny_lds_void)(ring + stage * STAGE_BYTES + j * 1024), 16, voff[j], k_bytes, 0, 0);
+    };
+    const uint32_t all = p.K / 64;
+    const uint32_t first = wave * windows_per_wave;
+    const uint32_t count = first >= all ? 0 : (all - first < windows_per_wave ? all - first : windows_per_wave);
+
+    float4y acc[MB][NB];
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb) acc[mb][nb] = float4y{0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+    for (int t = 0; t < STAGES - 1; ++t)
+        if (static_cast<uint32_t>(t) < count) issue(first + t, t);
+    uint32_t stage = 0, fill = STAGES - 1;
+    for (uint32_t i = 0; i < count; ++i) {
+        if (i + STAGES - 1 < count) {
+            issue(first + i + STAGES - 1, fill);
+            asm volatile("s_waitcnt vmcnt(%0)" ::"n"((STAGES - 1) * LOADS) : "memory");    // loads complete in order: window i is in
+        } else {
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        }
+        const T* at = reinterpret_cast<const T*>(ring + stage * STAGE_BYTES);
+        uint4y fw[2][NB], fx[2][MB];
+#pragma unroll
+        for (int half = 0; half < 2; ++half) {
+#pragma unroll
+            for (int nb = 0; nb < NB; ++nb) fw[half][nb] = *reinterpret_cast<const uint4y*>(at + nb * 1024 + tile_offset<T>(r, half * 4 + kc));
+#pragma unroll
+            for (int mb = 0; mb < MB; ++mb) fx[half][mb] = *reinterpret_cast<const uint4y*>(at + (NB + mb) * 1024 + tile_offset<T>(r, half * 4 + kc));
+        }
+#pragma unroll
+        for (int half = 0; half < 2; ++half)
+#pragma unroll
+            for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+                for (int nb = 0; nb < NB; ++nb) acc[mb][nb] = skinny_mfma<T>(fw[half][nb], fx[half][mb], acc[mb][nb]);
+        stage = stage + 1 == STAGES ? 0 : stage + 1;
+        fill = fill + 1 == STAGES ? 0 : fill + 1;
+    }
+    // the wavefronts' tiles meet in LDS (every wavefront's ring has been read: its own MFMAs needed the data)
+    __syncthreads();
+    float4y* partial = reinterpret_cast<float4y*>(skinny_lds);     // [wave][tile][lane]
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb) partial[(wave * MB * NB + mb * NB + nb) * 64 + lane] = acc[mb][nb];
+    __syncthreads();
+    // accumulator: lane -> row of x (m) lane % 16; value v -> column n0 + 4 * (lane / 16) + v; wavefront t adds up tile t, t + 4, ..
+    T* cb = c + oc;
+    const bool vector_ok = p.c_rs % 4 == 0 && p.N % 4 == 0 && reinterpret_cast<uintptr_t>(cb) % 8 == 0;
+    for (int t = wave; t < MB * NB; t += kStreamWaves) {
+        const int mb = t / NB, nb = t % NB;
+        float4y sum = partial[t * 64 + lane];
+#pragma unroll
+        for (int v = 1; v < kStreamWaves; ++v) sum += partial[(v * MB * NB + t) * 64 + lane];
+        const uint32_t m = mb * 16 + r, col = n0 + nb * 16 + 4 * kc;
+        if (m >= p.M) continue;
+        T out[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) out[e] = narrow_result<T>(sum[e]);
+        T* dst = cb + static_cast<int64_t>(m) * p.c_rs + col;
+        if (vector_ok) {
+            if (col < p.N) {
+                uint2 bits;
+                __builtin_memcpy(&bits, out, 8);
+                *reinterpret_cast<uint2*>(dst) = bits;
+            }
+        } else {
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+                if (col + e < p.N) dst[e] = out[e];
+        }
+    }
+#endif
+}
+
+template <class T, int MB, int NB>
+static int launch_stream(const GemmProblem& p, const void* a, const void* b, void* c, hipStream_t stream) {
+    auto kernel = gemm_skinny_stream_kernel<T, MB, NB>;
+    constexpr size_t lds = kStreamWaves * kStreamBytesPerWave;
+    static std::atomic<uint64_t> configured{0};
+    if (int rc = raise_lds_limit(reinterpret_cast<const void*>(kernel), lds, configured)) return rc;
+    const uint32_t windows = p.K / 64, per_wave = (windows + kStreamWaves - 1) / kStreamWaves;
+    hipLaunchKernelGGL(kernel, dim3((p.N + 16 * NB - 1) / (16 * NB), p.batches), dim3(64 * kStreamWaves), lds, stream, static_cast<const T*>(a), static_cast<const T*>(b),
+                       static_cast<T*>(c), p, per_wave);
+    return launch_status("gemm_skinny_stream_kernel");
+}
+
 template <class T>
 int run_skinny(const GemmProblem& p, const void* a, const void* b, void* c, hipStream_t stream) {
     if (p.M == 0 || p.M > 32 || p.N == 0 || p.K == 0 || p.batches == 0 || p.batches > 65535 || p.row_bias) return TANNIC_UNSUPPORTED_DTYPE;
@@ -133,6 +269,13 @@ int run_skinny(const GemmProblem& p, const void* a, const void* b, void* c, hipS
     if (reinterpret_cast<uintptr_t>(a) % 16 || reinterpret_cast<uintptr_t>(b) % 16) return TANNIC_UNSUPPORTED_DTYPE;
     for (int d = 0; d < p.batch_rank; ++d)
         if (!mult8(p.a_bs[d]) || !mult8(p.b_bs[d])) return TANNIC_UNSUPPORTED_DTYPE;
+    // whole windows of 64 and rows that do not overlap: the streaming kernel (offsets inside a block are 32-bit byte counts)
+    if (p.K % 64 == 0 && p.a_rs >= static_cast<int64_t>(p.K) && p.b_cs >= static_cast<int64_t>(p.K) && p.a_rs < (1 << 22) && p.b_cs < (1 << 22)) {
+        // two column blocks per wavefront (half as many workgroups, x read half as often) while every compute unit still gets one
+        const bool two = static_cast<uint64_t>((p.N + 31) / 32) * p.batches >= 400;
+        if (p.M <= 16) return two ? launch_stream<T, 1, 2>(p, a, b, c, stream) : launch_stream<T, 1, 1>(p, a, b, c, stream);
+        return two ? launch_stream<T, 2, 2>(p, a, b, c, stream) : launch_stream<T, 2, 1>(p, a, b, c, stream);
+    }
     // K is split evenly over the wavefronts, in whole steps of 32
     const uint32_t steps = (p.K + 31) / 32, per_wave = (steps + kSkinnyWaves - 1) / kSkinnyWaves;
     const uint32_t k_per_wave = per_wave * 32;
