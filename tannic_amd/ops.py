@@ -36,6 +36,8 @@ class TannicError(RuntimeError):
 def _resolve(*tensors):
     """``resolve_two_environment`` / ``resolve_three_environment`` (``src/bindings.cpp:118-188``)."""
     envs = [t.environment for t in tensors]
+    if len(envs) == 2 and envs[0] is envs[1]:
+        return envs[0]
     devices = [e for e in envs if isinstance(e, Device)]
     if not devices:
         return Host()
@@ -46,18 +48,15 @@ def _resolve(*tensors):
 
 def _call(name, env, sources, dst, extra=(), scalar=None):
     """One backend call in the order the ABI expects: sources, [scalar], dst, [stream], extra."""
-    descs = [s.descriptor() for s in sources]
-    out = dst.descriptor()
-    args = [C.byref(d) for d in descs]
+    args = [s.reference() for s in sources]
     if scalar is not None:
         args.append(C.byref(scalar))
-    args.append(C.byref(out))
+    args.append(dst.reference())
     if isinstance(env, Device):
         lib = library()
-        dvc = env.structure()
-        stream = lib.pop_stream(C.byref(dvc))
+        stream = lib.pop_stream(env.reference)
         status = lib.kernels[name](*args, stream, *extra)
-        lib.put_stream(C.byref(dvc), stream)
+        lib.put_stream(env.reference, stream)
         detail = lib.error_message() if status == abi.ERROR else ""
     else:
         if _host_functions is None:
@@ -71,7 +70,7 @@ def _call(name, env, sources, dst, extra=(), scalar=None):
 
 
 def _new(dtype, shape, env):
-    return Tensor(dtype, shape).initialize(env)
+    return Tensor.fresh(dtype, shape, env)
 
 
 # ---- dtype / shape rules ------------------------------------------------
@@ -82,6 +81,8 @@ def promote(first, second):
 
 def broadcast(first, second):
     """``operation::broadcast`` (``include/tannic/operations.hpp:137-152``)."""
+    if first == second:
+        return tuple(first)
     rank = builtins.max(len(first), len(second))
     out = []
     for d in range(rank):
@@ -375,7 +376,7 @@ def repeat(x, repeats, axis=0):
     shape = list(x.shape)
     shape[axis] *= repeats
     env = _resolve(x)
-    dst = Tensor(x.dtype, tuple(shape)).initialize(env)
+    dst = _new(x.dtype, shape, env)
     _call("repeat", env, [x], dst, (C.c_int(axis), C.c_int(repeats)))
     return dst
 
@@ -395,7 +396,7 @@ def concatenate(first, second, axis=0):
         elif first.shape[d] != second.shape[d]:
             raise TannicError("All dimensions except concat axis must match")
     env = _resolve(first, second)
-    dst = Tensor(first.dtype, tuple(shape)).initialize(env)
+    dst = _new(first.dtype, shape, env)
     _call("concat", env, [first, second], dst, (C.c_int(axis),))
     return dst
 
@@ -407,13 +408,13 @@ def outer(first, second):
         raise TannicError("Outer product of tensors with rank more than 1 not supported")
     dtype = first.dtype if first.dtype.code > second.dtype.code else second.dtype
     env = _resolve(first, second)
-    dst = Tensor(dtype, (first.shape[0], second.shape[0])).initialize(env)
+    dst = _new(dtype, (first.shape[0], second.shape[0]), env)
     return _call("outer", env, [first, second], dst)
 
 
 def _triangular(name, x, k):
     env = _resolve(x)
-    dst = Tensor(x.dtype, x.shape).initialize(env)
+    dst = _new(x.dtype, x.shape, env)
     _call(name, env, [x], dst, (C.c_int(k),))
     return dst
 

@@ -9,6 +9,7 @@ layout SINGLETON / CONTIGUOUS / STRIDED.
 """
 import ctypes as C
 import math
+import struct
 
 import numpy as np
 
@@ -43,6 +44,7 @@ class Device:
             raise IndexError("Invalid device ID")
         self.id = id
         self._structure = abi.device_t(id)
+        self.reference = C.byref(self._structure)    # what every backend call on this device passes
 
     def structure(self):
         return self._structure
@@ -65,8 +67,7 @@ class Buffer:
         self.nbytes = nbytes
         self.environment = environment
         if isinstance(environment, Device):
-            dvc = environment.structure()
-            self.address = library().allocate(C.byref(dvc), max(nbytes, 1))
+            self.address = library().allocate(environment.reference, max(nbytes, 1))
             if not self.address:
                 raise BackendError("device allocation failed: " + library().error_message())
             self.array = None
@@ -77,11 +78,16 @@ class Buffer:
     def __del__(self):
         if isinstance(self.environment, Device) and getattr(self, "address", None):
             try:
-                dvc = self.environment.structure()
-                library().deallocate(C.byref(dvc), self.address)
+                library().deallocate(self.environment.reference, self.address)
             except Exception:
                 pass
             self.address = None
+
+
+# tensor_t: address, rank, shape[8], strides[8], dtype, environment (kind, device id or host traits), size, layout
+_TENSOR_T = struct.Struct("<QB7x8Q8qiii4xQi4x")
+_PAD = [(0,) * (abi.DIMENSIONS - r) for r in range(abi.DIMENSIONS + 1)]
+assert _TENSOR_T.size == C.sizeof(abi.tensor_t)
 
 
 def contiguous_strides(shape):
@@ -118,7 +124,23 @@ class Tensor:
 
     def is_contiguous(self):
         # include/tannic/tensor.hpp:60-69: every stride must equal the running product
-        return self.strides == contiguous_strides(self.shape)
+        known = self.__dict__.get("_contiguous")
+        if known is None:
+            known = self._contiguous = self.strides == contiguous_strides(self.shape)
+        return known
+
+    @classmethod
+    def fresh(cls, dtype, shape, environment):
+        """A new contiguous tensor with its own buffer: what an operator allocates for its result."""
+        t = cls.__new__(cls)
+        t.dtype = dtype
+        t.shape = shape = tuple(shape)
+        t.strides = contiguous_strides(shape)
+        t.offset = 0
+        t.nelements = math.prod(shape)
+        t._contiguous = True
+        t.buffer = Buffer(types.nbytesof(dtype, t.nelements), environment)
+        return t
 
     def is_singleton(self):
         return self.nelements == 1
@@ -223,23 +245,24 @@ class Tensor:
         cached = self.__dict__.get("_descriptor")
         if cached is not None:
             return cached
-        t = abi.tensor_t()
-        t.address = self.address
-        t.rank = self.rank
-        for i in range(self.rank):
-            t.shape.sizes[i] = self.shape[i]
-            t.strides.sizes[i] = self.strides[i]
-        t.dtype = self.dtype.code
-        env = self.environment
-        t.environment.kind = env.kind
-        if isinstance(env, Device):
-            t.environment.resource.device.id = env.id
-        else:
-            t.environment.resource.host.traits = abi.PAGEABLE
-        t.size = self.nelements
-        t.layout = abi.SINGLETON if self.is_singleton() else abi.CONTIGUOUS if self.is_contiguous() else abi.STRIDED
+        # one packed image of ``tensor_t`` (offsets checked against the structure when ``abi`` is imported)
+        rank, env = len(self.shape), self.buffer.environment
+        pad = _PAD[rank]
+        layout = abi.SINGLETON if self.nelements == 1 else abi.CONTIGUOUS if self.is_contiguous() else abi.STRIDED
+        resource = env.id if env.kind == abi.DEVICE else abi.PAGEABLE
+        t = abi.tensor_t.from_buffer_copy(_TENSOR_T.pack(self.buffer.address + self.offset, rank, *self.shape, *pad, *self.strides, *pad, self.dtype.code,
+                                                         env.kind, resource, self.nelements, layout))
         self._descriptor = t
+        self._reference = C.byref(t)
         return t
+
+    def reference(self):
+        """``byref(descriptor())``, kept with it: the argument a backend call takes."""
+        r = self.__dict__.get("_reference")
+        if r is None:
+            self.descriptor()
+            r = self._reference
+        return r
 
     # ---- views (include/tannic/views.hpp) --------------------------------
     def _view(self, shape, strides, offset=None):
