@@ -52,11 +52,14 @@ def _call(name, env, sources, dst, extra=(), scalar=None):
     if scalar is not None:
         args.append(C.byref(scalar))
     args.append(dst.reference())
-    if isinstance(env, Device):
+    if env.kind == abi.DEVICE:
         lib = library()
-        stream = lib.pop_stream(env.reference)
+        reference = env.reference
+        stream = lib.pop_stream(reference)
         status = lib.kernels[name](*args, stream, *extra)
-        lib.put_stream(env.reference, stream)
+        lib.put_stream(reference, stream)
+        if status == abi.SUCCESS:
+            return dst
         detail = lib.error_message() if status == abi.ERROR else ""
     else:
         if _host_functions is None:

@@ -66,7 +66,8 @@ class Buffer:
     def __init__(self, nbytes, environment):
         self.nbytes = nbytes
         self.environment = environment
-        if isinstance(environment, Device):
+        self.array, self.address = None, 0     # (what __del__ looks at, should the allocation raise)
+        if environment.kind == abi.DEVICE:
             self.address = library().allocate(environment.reference, max(nbytes, 1))
             if not self.address:
                 raise BackendError("device allocation failed: " + library().error_message())
@@ -76,7 +77,7 @@ class Buffer:
             self.address = self.array.ctypes.data
 
     def __del__(self):
-        if isinstance(self.environment, Device) and getattr(self, "address", None):
+        if self.array is None and self.address:
             try:
                 library().deallocate(self.environment.reference, self.address)
             except Exception:
@@ -90,12 +91,24 @@ _PAD = [(0,) * (abi.DIMENSIONS - r) for r in range(abi.DIMENSIONS + 1)]
 assert _TENSOR_T.size == C.sizeof(abi.tensor_t)
 
 
+_STRIDES = {}     # shape -> (contiguous strides, number of elements); shapes recur, the table stays small
+
+
+def _shape_facts(shape):
+    facts = _STRIDES.get(shape)
+    if facts is None:
+        strides, expected = [0] * len(shape), 1
+        for i in range(len(shape) - 1, -1, -1):
+            strides[i] = expected
+            expected *= shape[i]
+        if len(_STRIDES) > 4096:
+            _STRIDES.clear()
+        facts = _STRIDES[shape] = (tuple(strides), math.prod(shape))
+    return facts
+
+
 def contiguous_strides(shape):
-    strides, expected = [0] * len(shape), 1
-    for i in range(len(shape) - 1, -1, -1):
-        strides[i] = expected
-        expected *= shape[i]
-    return tuple(strides)
+    return _shape_facts(tuple(shape))[0]
 
 
 class Tensor:
@@ -135,9 +148,8 @@ class Tensor:
         t = cls.__new__(cls)
         t.dtype = dtype
         t.shape = shape = tuple(shape)
-        t.strides = contiguous_strides(shape)
+        t.strides, t.nelements = _shape_facts(shape)
         t.offset = 0
-        t.nelements = math.prod(shape)
         t._contiguous = True
         t.buffer = Buffer(types.nbytesof(dtype, t.nelements), environment)
         return t
@@ -266,7 +278,12 @@ class Tensor:
 
     # ---- views (include/tannic/views.hpp) --------------------------------
     def _view(self, shape, strides, offset=None):
-        v = Tensor(self.dtype, shape, strides, self.offset if offset is None else offset)
+        v = Tensor.__new__(Tensor)
+        v.dtype = self.dtype
+        v.shape = shape = tuple(shape)
+        v.strides = tuple(strides)
+        v.offset = self.offset if offset is None else offset
+        v.nelements = math.prod(shape)
         v.buffer = self.buffer
         return v
 
