@@ -592,7 +592,10 @@ int run16(const GemmProblem& p, const void* a, const void* b, void* c, hipStream
             const double rounds = static_cast<double>((static_cast<uint64_t>(blocks) + 255) / 256);
             // a step costs more the more compute units pull operands through the L2s at the same time
             const double busy = blocks < 256.0 ? blocks / 256.0 : 1.0;
-            double step_us = bm == 256 ? 1.0 : bm == 128 ? 0.375 + 0.175 * busy : 0.30 + 0.075 * busy;
+            // (A 64-row tile that walks all of K is register-staged with two stages: between other kernels, with its operands
+            // in no cache, its steps take a fifth longer than in a loop over the same product — 40 against 29 us for
+            // 512 x 4096 x 4096 inside a decoder layer — which those of the direct-to-LDS tiles do not: 33 us with K shared.)
+            double step_us = bm == 256 ? 1.0 : bm == 128 ? 0.375 + 0.175 * busy : splits == 1 ? 0.36 + 0.09 * busy : 0.30 + 0.075 * busy;
             // fp32: the matrix pipe, sixteen times slower than for the 16-bit types, sets the pace of a step
             // (2 * bm * 128 * 64 flops at 157.3 TFLOP/s over 256 compute units)
             if constexpr (sizeof(T) == 4) step_us = std::max(step_us, 2.0 * bm * 128 * 64 / (157.3e6 / 256));
