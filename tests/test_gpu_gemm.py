@@ -40,6 +40,14 @@ LAYOUTS = {
     # few rows: ragged K steps and columns, two row blocks, batches; a long K shared between blocks
     "skinny_17_rows_ragged": ((17, 72), (40, 72), [], [("transpose", (-1, -2))]),
     "skinny_batched": ((3, 5, 64), (3, 24, 64), [], [("transpose", (-1, -2))]),
+    # few rows with whole 64-wide K windows (operands streamed through LDS): one and two row blocks, ragged columns, one
+    # and two column blocks per wavefront, fewer windows than wavefronts, batches, rows longer than K (a view)
+    "stream_1_row": ((1, 1024), (200, 1024), [], [("transpose", (-1, -2))]),
+    "stream_16_rows_ragged_columns": ((16, 640), (90, 640), [], [("transpose", (-1, -2))]),
+    "stream_20_rows_one_window": ((20, 64), (48, 64), [], [("transpose", (-1, -2))]),
+    "stream_32_rows_many_columns": ((32, 128), (12840, 128), [], [("transpose", (-1, -2))]),
+    "stream_5_rows_many_columns": ((5, 192), (12816, 192), [], [("transpose", (-1, -2))]),
+    "stream_batched_views": ((3, 9, 320), (3, 70, 320), [("index", (Ellipsis, slice(0, 256)))], [("index", (Ellipsis, slice(64, 320))), ("transpose", (-1, -2))]),
     "split_k_nt": ((128, 1096), (136, 1096), [], [("transpose", (-1, -2))]),
     "split_k_nn": ((72, 2048), (2048, 64), [], []),
     # operands contiguous along M / N with ragged tiles and a K tail, in every tile size (the largest needs 200 tiles)
