@@ -162,6 +162,11 @@ __global__ __launch_bounds__(256, BLOCKS_PER_CU) void gemm16_dtl_kernel(const T*
 
     constexpr int PER_KS = TM * TN;   // MFMAs per k-slice
     constexpr int LOAD_EVERY = PER_KS / LOADS > 0 ? PER_KS / LOADS : 1;   // the loads of a step go out during its first half
+    // The fragment reads of a half are spread evenly over it.  A 16-byte read of a wavefront keeps the LDS busy for 8 clocks
+    // and the four wavefronts of a workgroup run in step: sixteen reads each behind sixteen consecutive MFMAs ask for
+    // 512 clocks of LDS time during 256 clocks of matrix work, and the wavefront that cannot hand its read over does not
+    // issue its next MFMA either (measured: 1240 clocks for a half of 64 MFMAs, 1024 of them matrix work).
+    constexpr int READ_EVERY = PER_KS / (TM + TN) > 0 ? PER_KS / (TM + TN) : 1;
     uint4v fa[2][TM], fb[2][TN];
     // fragment of the 16 rows (columns) from `first` on, k-slice ks of a tile
     const uint32_t tr_unit = (frag_row / 4) + 4 * (frag_chunk % 2), tr_row = 8 * frag_chunk + frag_row / 4, tr_quad = (frag_row % 4) * 4;
@@ -204,7 +209,7 @@ __global__ __launch_bounds__(256, BLOCKS_PER_CU) void gemm16_dtl_kernel(const T*
         else fa[into][r - TN] = fragment(a_tile, ATag{}, AWidth{}, wm + (r - TN) * 16, ks_tag);
     };
     // A step issues the MFMAs of the second k-slice of the previous tile (its fragments are in registers since before
-    // the barrier) and those of the first slice of this tile.  Behind the first MFMAs of each half go the fragment
+    // the barrier) and those of the first slice of this tile.  Spread over the MFMAs of each half go the fragment
     // reads of the slice the NEXT half multiplies (their registers were last read by the half before this one), and,
     // spread over the first half, the loads of the next tile.
     auto step = [&](uint32_t s, uint32_t cur, uint32_t fill, auto first_tag, auto fetch_tag) {   // cur: stage of tile s; fill: stage tile s-1 has left
@@ -221,7 +226,7 @@ __global__ __launch_bounds__(256, BLOCKS_PER_CU) void gemm16_dtl_kernel(const T*
             constexpr int now = group == 0 ? 1 : 0;
             if constexpr (q == 0) wait_fragments();
             if constexpr (!(FIRST && group == 0)) mfma16x16_in_place<T>(acc[i][j], fb[now][j], fa[now][i]);
-            if constexpr (q < TM + TN && !(FIRST && group == 0)) read_one(a_tile, b_tile, std::integral_constant<int, group == 0 ? 0 : 1>{}, group == 0 ? 0 : 1, q);
+            if constexpr (q % READ_EVERY == 0 && q / READ_EVERY < TM + TN && !(FIRST && group == 0)) read_one(a_tile, b_tile, std::integral_constant<int, group == 0 ? 0 : 1>{}, group == 0 ? 0 : 1, q / READ_EVERY);
             constexpr int slot = FIRST ? m - PER_KS : m;
             if constexpr (FETCH && slot >= 0 && slot % LOAD_EVERY == LOAD_EVERY / 2 && slot / LOAD_EVERY < LOADS) issue_load(slot / LOAD_EVERY, fill, k_first + (s + STAGES - 1) * BK);
             __builtin_amdgcn_sched_barrier(0);
