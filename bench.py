@@ -175,7 +175,7 @@ def gemm_ceiling_entries(b, iters=5):
                 v[8 * 256 * 8:] = b.values(dtype, (8 * 256 * 8,), "normal", 0, 2, 0.02)
             operands = ta.Tensor(dtype, (16 * 256 * 8,)).initialize(b.device)
             operands.write(v)
-            for shape, name in ((0, "v_mfma_f32_32x32x16"), (1, "v_mfma_f32_16x16x32")):
+            for shape, name in ((0, "v_mfma_f32_32x32x16"), (1, "v_mfma_f32_16x16x32"), (2, "v_mfma_f32_16x16x32 in pairs on one accumulator")):
                 def run():
                     rc = b.lib.probe_mfma(shape, dtype.code, operands.address, sink.address, blocks, iterations, b.stream)
                     if rc != 0:

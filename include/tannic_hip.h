@@ -198,7 +198,8 @@ float tannic_hip_event_elapsed_ms(void* start, void* stop);
 /* Rate probe of the matrix pipe, for benchmark harnesses (no reference twin): `blocks` workgroups of four wavefronts
  * issue nothing but MFMAs, `iterations` x 2^21 multiply-adds per wavefront, on operand values the caller supplies
  * (`operands`: 64 KiB of device memory, 16 x 256 vectors of 16 bytes, read once; `sink`: 1 KiB per block, written
- * once).  shape 0: v_mfma_f32_32x32x16, shape 1: v_mfma_f32_16x16x32; dtype TANNIC_FLOAT16 or TANNIC_BFLOAT16.
+ * once).  shape 0: v_mfma_f32_32x32x16, shape 1: v_mfma_f32_16x16x32, shape 2: v_mfma_f32_16x16x32 with every two
+ * consecutive MFMAs on the same accumulator; dtype TANNIC_FLOAT16 or TANNIC_BFLOAT16.
  * What it sustains on given values is the ceiling of a product of such values on this device. */
 int tannic_hip_probe_mfma(int shape, int dtype, const void* operands, void* sink, uint32_t blocks, uint32_t iterations, tannic_stream_t stream);
 

@@ -19,10 +19,12 @@ template <class T, int SHAPE, class Acc> __device__ inline void mfma_in_place(Ac
     if constexpr (SHAPE == 1 && std::is_same_v<T, bf16>) asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(acc) : "v"(a), "v"(b));
 }
 
-// SHAPE 0: v_mfma_f32_32x32x16, 16 accumulators of 16 registers; SHAPE 1: v_mfma_f32_16x16x32, 32 accumulators of 4.
+// SHAPE 0: v_mfma_f32_32x32x16, 16 accumulators of 16 registers; SHAPE 1: v_mfma_f32_16x16x32, 32 accumulators of 4;
+// CHAIN: how many consecutive MFMAs update the same accumulator (a dependent MFMA takes its addend from the one before
+// it, not from the register file: no slower, and cheaper in power).
 // One iteration is 2^21 multiply-adds per wavefront either way (64 resp. 128 MFMAs); operands rotate through eight
 // registers per side so that consecutive MFMAs see different values, as they do in a product.
-template <class T, int SHAPE>
+template <class T, int SHAPE, int CHAIN = 1>
 __global__ __launch_bounds__(256) void probe_mfma_kernel(const uint4v* operands, float* sink, uint32_t iterations) {
     uint4v a[8], b[8];
 #pragma unroll
@@ -54,7 +56,7 @@ __global__ __launch_bounds__(256) void probe_mfma_kernel(const uint4v* operands,
             for (int v = 0; v < 4; ++v) acc[i][v] = 0.0f;
         for (uint32_t it = 0; it < iterations; ++it) {
 #pragma unroll
-            for (int m = 0; m < 128; ++m) mfma_in_place<T, 1>(acc[m % 32], b[(m + m / 32) % 8], a[(m / 8) % 8]);
+            for (int m = 0; m < 128; ++m) mfma_in_place<T, 1>(acc[(m / CHAIN) % 32], b[(m + m / 32) % 8], a[(m / 8) % 8]);
         }
         asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
 #pragma unroll
@@ -70,8 +72,8 @@ __global__ __launch_bounds__(256) void probe_mfma_kernel(const uint4v* operands,
 using namespace th;
 
 extern "C" int tannic_hip_probe_mfma(int shape, int dtype, const void* operands, void* sink, uint32_t blocks, uint32_t iterations, tannic_stream_t stream) {
-    if (!operands || !sink || blocks == 0 || (shape != 0 && shape != 1)) {
-        set_error_text("probe_mfma: operands (64 KiB), sink (1 KiB per block) and a block count are required; shape is 0 or 1");
+    if (!operands || !sink || blocks == 0 || shape < 0 || shape > 2) {
+        set_error_text("probe_mfma: operands (64 KiB), sink (1 KiB per block) and a block count are required; shape is 0, 1 or 2");
         return TANNIC_ERROR;
     }
     hipStream_t s = as_stream(stream);
@@ -79,10 +81,12 @@ extern "C" int tannic_hip_probe_mfma(int shape, int dtype, const void* operands,
     float* out = static_cast<float*>(sink);
     if (dtype == TANNIC_FLOAT16) {
         if (shape == 0) hipLaunchKernelGGL((probe_mfma_kernel<f16, 0>), dim3(blocks), dim3(256), 0, s, ops, out, iterations);
-        else hipLaunchKernelGGL((probe_mfma_kernel<f16, 1>), dim3(blocks), dim3(256), 0, s, ops, out, iterations);
+        else if (shape == 1) hipLaunchKernelGGL((probe_mfma_kernel<f16, 1>), dim3(blocks), dim3(256), 0, s, ops, out, iterations);
+        else hipLaunchKernelGGL((probe_mfma_kernel<f16, 1, 2>), dim3(blocks), dim3(256), 0, s, ops, out, iterations);
     } else if (dtype == TANNIC_BFLOAT16) {
         if (shape == 0) hipLaunchKernelGGL((probe_mfma_kernel<bf16, 0>), dim3(blocks), dim3(256), 0, s, ops, out, iterations);
-        else hipLaunchKernelGGL((probe_mfma_kernel<bf16, 1>), dim3(blocks), dim3(256), 0, s, ops, out, iterations);
+        else if (shape == 1) hipLaunchKernelGGL((probe_mfma_kernel<bf16, 1>), dim3(blocks), dim3(256), 0, s, ops, out, iterations);
+        else hipLaunchKernelGGL((probe_mfma_kernel<bf16, 1, 2>), dim3(blocks), dim3(256), 0, s, ops, out, iterations);
     } else {
         return TANNIC_UNSUPPORTED_DTYPE;
     }
