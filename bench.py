@@ -269,6 +269,15 @@ def decoder_layer_entry(b, iters, composed=True, one_pass=True):
                         "tflops": round(flops / us / 1e6, 2), "mfma_frac": round(flops / us / 1e6 / MFMA_PEAK_TFLOPS["bf16"], 4),
                         "bound": "mixed: matrix products plus about 45 launch-bound elementwise, reduction and copy kernels", "stream_us": round(busy, 1),
                         "stream_tflops": round(flops / busy / 1e6, 2)})
+        # the same backend calls recorded once and replayed as one HIP graph: what the device needs when the host does not hold it up
+        with ta.Graph(b.device) as graph:
+            recorded = dl.forward(s, w, x, cos, sin, mask, one)
+        us, busy = timed(graph.launch)
+        del recorded
+        graph.close()
+        entries.append({"op": "the composed layer, its backend calls recorded once and replayed as a HIP graph", "us": round(us, 1),
+                        "tflops": round(flops / us / 1e6, 2), "mfma_frac": round(flops / us / 1e6 / MFMA_PEAK_TFLOPS["bf16"], 4),
+                        "bound": "the same kernels, issued by one graph launch", "stream_us": round(busy, 1), "stream_tflops": round(flops / busy / 1e6, 2)})
     if one_pass:
         packed = dl.pack_weights(w)
         us, busy = timed(lambda: dl.forward_fused(s, packed, x, cos, sin, mask))

@@ -188,6 +188,25 @@ void tannic_hip_put_stream(const tannic_device_t* device, tannic_stream_t stream
 int tannic_hip_stream_synchronize(tannic_stream_t stream);
 int tannic_hip_device_synchronize(void);
 
+/* A sequence of backend calls recorded once and replayed as one HIP graph: for loops whose cost is issuing the
+ * calls, not running them (a decoder layer is some sixty short kernels).  No counterpart in the reference, whose
+ * front end evaluates every expression where it is written.
+ *   graph_begin   starts recording on the stream the device's backend calls use; every call until graph_end is
+ *                 recorded instead of run.  One recording may be open at a time.  Calls that wait for the stream
+ *                 (copies to pageable host memory, allclose) cannot be recorded: they fail and graph_end reports it.
+ *   graph_end     closes the recording and prepares it for launching.
+ *   graph_launch  queues one replay on that stream, ordered with the eager calls around it.
+ *   graph_destroy waits for the stream and releases the recording.
+ * Memory: tensors allocated while recording are written by every replay, at the same addresses.  Their blocks, and the
+ * kernels' scratch, belong to the recording until graph_destroy (released earlier, they are reused only inside that
+ * recording), so a replay never writes memory that a tensor outside the recording has been given.  Tensors that
+ * existed before graph_begin and are read or written by the recorded calls (inputs, weights) must stay allocated for
+ * as long as the recording is launched; new input is copied into them before graph_launch. */
+void* tannic_hip_graph_begin(const tannic_device_t* device);
+int tannic_hip_graph_end(void* recording);
+int tannic_hip_graph_launch(void* recording);
+void tannic_hip_graph_destroy(void* recording);
+
 /* Timing events on a stream, for benchmark harnesses (no reference twin). */
 void* tannic_hip_event_create(void);
 void tannic_hip_event_destroy(void* event);

@@ -12,3 +12,4 @@ from .backend import BackendError, library, LIBRARY_PATH
 from .tensor import Tensor, Host, Device, tensor
 from . import ops
 from .ops import TannicError
+from .graph import Graph

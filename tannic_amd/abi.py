@@ -145,6 +145,10 @@ def runtime_signatures():
         "put_stream": (None, [DP, stream_t]),
         "stream_synchronize": (C.c_int, [stream_t]),
         "device_synchronize": (C.c_int, []),
+        "graph_begin": (C.c_void_p, [DP]),
+        "graph_end": (C.c_int, [C.c_void_p]),
+        "graph_launch": (C.c_int, [C.c_void_p]),
+        "graph_destroy": (None, [C.c_void_p]),
         "event_create": (C.c_void_p, []),
         "event_destroy": (None, [C.c_void_p]),
         "event_record": (C.c_int, [C.c_void_p, stream_t]),

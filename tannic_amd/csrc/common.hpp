@@ -212,4 +212,8 @@ struct FastDiv {
 int scratch_acquire(void** ptr, size_t nbytes, hipStream_t stream);
 int scratch_release(void* ptr, hipStream_t stream);
 
+// True while `stream` is being recorded into a graph: calls that wait for the stream refuse (and say why) instead of
+// breaking the recording.  Sets the error text when it returns true.
+bool refuses_while_recording(hipStream_t stream, const char* call);
+
 }  // namespace th

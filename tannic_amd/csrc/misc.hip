@@ -324,6 +324,7 @@ __global__ __launch_bounds__(kBlock) void allclose_kernel(const T* a, const T* b
 
 template <class T>
 int run_allclose(const tannic_tensor_t* a, const tannic_tensor_t* b, hipStream_t stream, double rtol, double atol) {
+    if (refuses_while_recording(stream, "allclose")) return -1;
     if (!same_extents(a, b)) {
         set_error_text("allclose: operand shapes differ");
         return -1;

@@ -1,6 +1,7 @@
 // Devices, memory, streams, host<->device copies.
 // Replaces the reference's src/cuda/mem.cu, src/cuda/streams.cu and
 // src/cuda/exc.cuh; cited per function in include/tannic_hip.h.
+#include <algorithm>
 #include <cstdlib>
 #include <mutex>
 #include <string>
@@ -86,13 +87,38 @@ struct ScratchBlock {
     size_t size;
     hipStream_t stream;
     int device;
+    int pins = 0;      // recorded graphs whose kernels hold this address: never freed while one of them lives
 };
+
+// A recorded sequence of backend calls (a HIP graph) and the memory its kernels address.  Tensor blocks allocated while
+// recording belong to the recording until it is destroyed: released, they wait in `idle` for the recording's own later
+// requests and never reach the blocks kept for everybody, so no tensor outside the graph can share an address with one
+// of its temporaries.
+struct Recording {
+    uint64_t id = 0;
+    int device = 0;
+    hipStream_t stream = nullptr;
+    hipGraph_t graph = nullptr;
+    hipGraphExec_t exec = nullptr;
+    bool capturing = false;
+    std::vector<void*> scratch;
+};
+static Recording* g_capturing = nullptr;   // at most one at a time, guarded by g_scratch_mutex and g_mem_mutex alike (set with both held)
 static std::mutex g_scratch_mutex;
 static std::vector<ScratchBlock> g_scratch_free, g_scratch_live;
 static size_t g_scratch_cached = 0;
 constexpr size_t kScratchCacheLimit = size_t(2) << 30;
 
 void release_idle_memory();   // defined below, next to the kept tensor blocks
+
+// With g_scratch_mutex held: a block handed out while `stream` is being recorded is addressed by the graph's kernels.
+static void pin_for_recording(ScratchBlock& b, hipStream_t stream) {
+    if (!g_capturing || !g_capturing->capturing || g_capturing->stream != stream) return;
+    for (void* seen : g_capturing->scratch)
+        if (seen == b.ptr) return;
+    g_capturing->scratch.push_back(b.ptr);
+    b.pins += 1;
+}
 
 int scratch_acquire(void** ptr, size_t nbytes, hipStream_t stream) {
     int device = 0;
@@ -108,6 +134,7 @@ int scratch_acquire(void** ptr, size_t nbytes, hipStream_t stream) {
             ScratchBlock b = g_scratch_free[best];
             g_scratch_free.erase(g_scratch_free.begin() + best);
             g_scratch_cached -= b.size;
+            pin_for_recording(b, stream);
             g_scratch_live.push_back(b);
             *ptr = b.ptr;
             return TANNIC_SUCCESS;
@@ -127,7 +154,9 @@ int scratch_acquire(void** ptr, size_t nbytes, hipStream_t stream) {
         return TANNIC_ERROR;
     }
     std::lock_guard<std::mutex> lock(g_scratch_mutex);
-    g_scratch_live.push_back(ScratchBlock{*ptr, size, stream, device});
+    ScratchBlock fresh{*ptr, size, stream, device};
+    pin_for_recording(fresh, stream);
+    g_scratch_live.push_back(fresh);
     return TANNIC_SUCCESS;
 }
 
@@ -141,7 +170,7 @@ int scratch_release(void* ptr, hipStream_t stream) {
                 g_scratch_live.erase(g_scratch_live.begin() + i);
                 break;
             }
-        if (block.ptr && g_scratch_cached + block.size <= kScratchCacheLimit) {
+        if (block.ptr && (block.pins > 0 || g_scratch_cached + block.size <= kScratchCacheLimit)) {
             g_scratch_free.push_back(block);
             g_scratch_cached += block.size;
             return TANNIC_SUCCESS;
@@ -152,6 +181,16 @@ int scratch_release(void* ptr, hipStream_t stream) {
     TH_TRY(hipStreamSynchronize(stream));
     TH_TRY(hipFree(ptr));
     return TANNIC_SUCCESS;
+}
+
+bool refuses_while_recording(hipStream_t stream, const char* call) {
+    {
+        std::lock_guard<std::mutex> lock(g_scratch_mutex);
+        if (!g_capturing || !g_capturing->capturing || (stream && g_capturing->stream != stream)) return false;
+    }
+    std::string text = std::string(call) + ": waits for the stream, which is being recorded into a graph; end the recording first";
+    set_error_text(text.c_str());
+    return true;
 }
 
 }  // namespace th
@@ -189,6 +228,8 @@ struct MemBlock {
     size_t size;
     hipStream_t stream;
     int device;
+    uint64_t recording = 0;   // the recorded graph that owns the block (0: nobody)
+    bool plain = false;       // from hipMalloc (allocated while a stream was being recorded), not from the stream-ordered pool
 };
 struct FreeBlock {
     void* ptr;
@@ -198,6 +239,22 @@ std::mutex g_mem_mutex;
 std::unordered_map<void*, MemBlock> g_mem_live;
 std::vector<FreeBlock> g_mem_free;     // oldest first
 size_t g_mem_kept = 0;
+std::unordered_map<uint64_t, std::vector<FreeBlock>> g_recording_idle;   // per living recording: its released blocks
+uint64_t g_recording_ids = 0;
+
+// Returns a block to the driver: stream-ordered for the pool's blocks; a hipMalloc block once its stream has passed it.
+void free_block(const FreeBlock& f) {
+    hipError_t err;
+    if (f.info.plain) {
+        err = hipStreamSynchronize(f.info.stream);
+        if (err == hipSuccess) err = hipFree(f.ptr);
+    } else {
+        err = hipFreeAsync(f.ptr, f.info.stream);
+    }
+    if (err != hipSuccess) set_error(f.info.plain ? "hipFree" : "hipFreeAsync", __FILE__, __LINE__, err);
+}
+
+bool fits(const MemBlock& b, size_t size) { return b.size >= size && b.size <= size + size / 4; }
 constexpr size_t kMemKeepLimit = size_t(48) << 30;
 
 size_t block_size(size_t nbytes) {
@@ -214,7 +271,7 @@ void release_kept_blocks() {
         all.swap(g_mem_free);
         g_mem_kept = 0;
     }
-    for (const FreeBlock& f : all) (void)hipFreeAsync(f.ptr, f.info.stream);
+    for (const FreeBlock& f : all) free_block(f);
     (void)hipGetLastError();
 }
 }  // namespace
@@ -232,8 +289,12 @@ void th::release_idle_memory() {
     std::vector<ScratchBlock> idle;
     {
         std::lock_guard<std::mutex> lock(g_scratch_mutex);
-        idle.swap(g_scratch_free);
+        for (const ScratchBlock& b : g_scratch_free) {
+            if (b.pins == 0) idle.push_back(b);
+        }
+        g_scratch_free.erase(std::remove_if(g_scratch_free.begin(), g_scratch_free.end(), [](const ScratchBlock& b) { return b.pins == 0; }), g_scratch_free.end());
         g_scratch_cached = 0;
+        for (const ScratchBlock& b : g_scratch_free) g_scratch_cached += b.size;
     }
     for (const ScratchBlock& b : idle) (void)hipFree(b.ptr);
     (void)hipGetLastError();
@@ -248,35 +309,53 @@ void* tannic_hip_allocate(const tannic_device_t* device, size_t nbytes) {
     hipStream_t stream = streams.pop(device->id);
     streams.put(device->id, stream);
     const size_t size = block_size(nbytes);
+    uint64_t recording = 0;
     {
         std::lock_guard<std::mutex> lock(g_mem_mutex);
+        if (g_capturing && g_capturing->capturing && g_capturing->stream == stream && g_capturing->device == device->id) {
+            // the recording's own released blocks first: their addresses are already private to it
+            recording = g_capturing->id;
+            std::vector<FreeBlock>& idle = g_recording_idle[recording];
+            size_t best = idle.size();
+            for (size_t i = 0; i < idle.size(); ++i)
+                if (fits(idle[i].info, size) && (best == idle.size() || idle[i].info.size < idle[best].info.size)) best = i;
+            if (best != idle.size()) {
+                const FreeBlock f = idle[best];
+                idle.erase(idle.begin() + best);
+                g_mem_live[f.ptr] = f.info;
+                return f.ptr;
+            }
+        }
         size_t best = g_mem_free.size();
         for (size_t i = 0; i < g_mem_free.size(); ++i) {
             const MemBlock& b = g_mem_free[i].info;
-            if (b.device != device->id || b.stream != stream || b.size < size || b.size > size + size / 4) continue;
+            if (b.device != device->id || b.stream != stream || !fits(b, size)) continue;
             if (best == g_mem_free.size() || b.size < g_mem_free[best].info.size) best = i;
         }
         if (best != g_mem_free.size()) {
-            const FreeBlock f = g_mem_free[best];
+            FreeBlock f = g_mem_free[best];
             g_mem_free.erase(g_mem_free.begin() + best);
             g_mem_kept -= f.info.size;
+            f.info.recording = recording;
             g_mem_live[f.ptr] = f.info;
             return f.ptr;
         }
     }
     void* ptr = nullptr;
-    hipError_t err = hipMallocAsync(&ptr, size, stream);
-    if (err != hipSuccess) {
+    // A stream-ordered allocation on a stream that is being recorded would become a node of the graph: take the block
+    // from hipMalloc instead (the recording owns it from here on).
+    hipError_t err = recording ? hipMalloc(&ptr, size) : hipMallocAsync(&ptr, size, stream);
+    if (err != hipSuccess && !recording) {
         // give the kept blocks back and try once more
         release_kept_blocks();
         err = hipMallocAsync(&ptr, size, stream);
     }
     if (err != hipSuccess) {
-        set_error("hipMallocAsync", __FILE__, __LINE__, err);
+        set_error(recording ? "hipMalloc (while recording)" : "hipMallocAsync", __FILE__, __LINE__, err);
         return nullptr;
     }
     std::lock_guard<std::mutex> lock(g_mem_mutex);
-    g_mem_live[ptr] = MemBlock{size, stream, device->id};
+    g_mem_live[ptr] = MemBlock{size, stream, device->id, recording, recording != 0};
     return ptr;
 }
 
@@ -288,12 +367,21 @@ void* tannic_hip_deallocate(const tannic_device_t* device, void* address) {
     streams.put(device->id, stream);
     std::vector<FreeBlock> evict;
     bool kept = false;
+    FreeBlock released{address, MemBlock{0, stream, device->id}};
     {
         std::lock_guard<std::mutex> lock(g_mem_mutex);
         auto it = g_mem_live.find(address);
         if (it != g_mem_live.end()) {
-            const MemBlock info = it->second;
+            MemBlock info = it->second;
             g_mem_live.erase(it);
+            auto owner = info.recording ? g_recording_idle.find(info.recording) : g_recording_idle.end();
+            if (owner != g_recording_idle.end()) {
+                // the graph's kernels address this block for as long as the recording lives
+                owner->second.push_back(FreeBlock{address, info});
+                return nullptr;
+            }
+            info.recording = 0;
+            released.info = info;
             // only a block released on the stream it lives on can be reused without waiting
             if (info.stream == stream && info.device == device->id && info.size <= kMemKeepLimit) {
                 g_mem_free.push_back(FreeBlock{address, info});
@@ -307,13 +395,14 @@ void* tannic_hip_deallocate(const tannic_device_t* device, void* address) {
             }
         }
     }
-    for (const FreeBlock& f : evict) {
-        hipError_t err = hipFreeAsync(f.ptr, f.info.stream);
-        if (err != hipSuccess) set_error("hipFreeAsync", __FILE__, __LINE__, err);
-    }
+    for (const FreeBlock& f : evict) free_block(f);
     if (!kept) {
-        hipError_t err = hipFreeAsync(address, stream);
-        if (err != hipSuccess) set_error("hipFreeAsync", __FILE__, __LINE__, err);
+        if (released.info.plain) {
+            free_block(released);
+        } else {
+            hipError_t err = hipFreeAsync(address, stream);
+            if (err != hipSuccess) set_error("hipFreeAsync", __FILE__, __LINE__, err);
+        }
     }
     return nullptr;
 }
@@ -325,6 +414,10 @@ int tannic_hip_copy_from_host(const tannic_device_t* device, const void* host, v
     TH_TRY(hipSetDevice(device->id));
     Streams& streams = Streams::instance();
     hipStream_t stream = streams.pop(device->id);
+    if (refuses_while_recording(stream, "copy_from_host")) {
+        streams.put(device->id, stream);
+        return TANNIC_ERROR;
+    }
     hipError_t err = hipMemcpyAsync(dev, host, nbytes, hipMemcpyHostToDevice, stream);
     // callers pass temporaries (one element of an initializer list): the source
     // must be consumed before returning
@@ -341,6 +434,10 @@ int tannic_hip_copy_device_to_host(const tannic_device_t* device, const void* de
     TH_TRY(hipSetDevice(device->id));
     Streams& streams = Streams::instance();
     hipStream_t stream = streams.pop(device->id);
+    if (refuses_while_recording(stream, "copy_device_to_host")) {
+        streams.put(device->id, stream);
+        return TANNIC_ERROR;
+    }
     hipError_t err = hipMemcpyAsync(host, dev, nbytes, hipMemcpyDeviceToHost, stream);
     if (err == hipSuccess) err = hipStreamSynchronize(stream);
     streams.put(device->id, stream);
@@ -368,6 +465,7 @@ int tannic_hip_copy(const tannic_tensor_t* src, tannic_tensor_t* dst, size_t nby
     hipStream_t stream = as_stream(s);
     const bool src_dev = src->environment.kind == TANNIC_DEVICE;
     const bool dst_dev = dst->environment.kind == TANNIC_DEVICE;
+    if (src_dev != dst_dev && refuses_while_recording(stream, "copy between host and device")) return TANNIC_ERROR;
     if (!src_dev && dst_dev) {
         TH_TRY(hipMemcpyAsync(dst->address, src->address, nbytes, hipMemcpyHostToDevice, stream));
         // pageable sources behave like the reference's blocking cudaMemcpy
@@ -394,13 +492,124 @@ void tannic_hip_put_stream(const tannic_device_t* device, tannic_stream_t stream
 }
 
 int tannic_hip_stream_synchronize(tannic_stream_t stream) {
+    if (refuses_while_recording(as_stream(stream), "stream_synchronize")) return TANNIC_ERROR;
     TH_TRY(hipStreamSynchronize(as_stream(stream)));
     return TANNIC_SUCCESS;
 }
 
 int tannic_hip_device_synchronize(void) {
+    if (refuses_while_recording(nullptr, "device_synchronize")) return TANNIC_ERROR;
     TH_TRY(hipDeviceSynchronize());
     return TANNIC_SUCCESS;
+}
+
+void* tannic_hip_graph_begin(const tannic_device_t* device) {
+    if (!device || tannic_hip_set_device(device->id) != TANNIC_SUCCESS) return nullptr;
+    Streams& streams = Streams::instance();
+    hipStream_t stream = streams.pop(device->id);
+    streams.put(device->id, stream);      // the next backend call pops this same stream
+    std::scoped_lock lock(g_scratch_mutex, g_mem_mutex);
+    if (g_capturing) {
+        set_error_text("graph_begin: another recording is open; end it first");
+        return nullptr;
+    }
+    hipError_t err = hipStreamBeginCapture(stream, hipStreamCaptureModeRelaxed);
+    if (err != hipSuccess) {
+        set_error("hipStreamBeginCapture", __FILE__, __LINE__, err);
+        return nullptr;
+    }
+    Recording* r = new Recording;
+    r->id = ++g_recording_ids;
+    r->device = device->id;
+    r->stream = stream;
+    r->capturing = true;
+    g_recording_idle[r->id];
+    g_capturing = r;
+    return r;
+}
+
+int tannic_hip_graph_end(void* recording) {
+    Recording* r = static_cast<Recording*>(recording);
+    if (!r || !r->capturing) {
+        set_error_text("graph_end: not an open recording");
+        return TANNIC_ERROR;
+    }
+    {
+        std::scoped_lock lock(g_scratch_mutex, g_mem_mutex);
+        r->capturing = false;
+        if (g_capturing == r) g_capturing = nullptr;
+    }
+    TH_TRY(hipSetDevice(r->device));
+    hipError_t err = hipStreamEndCapture(r->stream, &r->graph);
+    if (err != hipSuccess || !r->graph) {
+        // a call that cannot be recorded (a wait for the stream, a copy to pageable host memory) has ended the capture
+        set_error("hipStreamEndCapture", __FILE__, __LINE__, err);
+        r->graph = nullptr;
+        (void)hipGetLastError();
+        return TANNIC_ERROR;
+    }
+    err = hipGraphInstantiate(&r->exec, r->graph, nullptr, nullptr, 0);
+    if (err != hipSuccess) {
+        set_error("hipGraphInstantiate", __FILE__, __LINE__, err);
+        r->exec = nullptr;
+        return TANNIC_ERROR;
+    }
+    return TANNIC_SUCCESS;
+}
+
+int tannic_hip_graph_launch(void* recording) {
+    Recording* r = static_cast<Recording*>(recording);
+    if (!r || !r->exec) {
+        set_error_text("graph_launch: the recording was not ended successfully");
+        return TANNIC_ERROR;
+    }
+    TH_TRY(hipSetDevice(r->device));
+    TH_TRY(hipGraphLaunch(r->exec, r->stream));
+    return TANNIC_SUCCESS;
+}
+
+void tannic_hip_graph_destroy(void* recording) {
+    Recording* r = static_cast<Recording*>(recording);
+    if (!r) return;
+    (void)hipSetDevice(r->device);
+    if (r->capturing) {
+        // abandoned while open: close the capture and drop what it holds
+        {
+            std::scoped_lock lock(g_scratch_mutex, g_mem_mutex);
+            r->capturing = false;
+            if (g_capturing == r) g_capturing = nullptr;
+        }
+        hipGraph_t partial = nullptr;
+        (void)hipStreamEndCapture(r->stream, &partial);
+        if (partial) (void)hipGraphDestroy(partial);
+        (void)hipGetLastError();
+    }
+    (void)hipStreamSynchronize(r->stream);     // no replay is still running when the memory changes hands
+    if (r->exec) (void)hipGraphExecDestroy(r->exec);
+    if (r->graph) (void)hipGraphDestroy(r->graph);
+    std::vector<FreeBlock> idle;
+    {
+        std::scoped_lock lock(g_scratch_mutex, g_mem_mutex);
+        for (void* ptr : r->scratch) {
+            for (ScratchBlock& b : g_scratch_free)
+                if (b.ptr == ptr && b.pins > 0) b.pins -= 1;
+            for (ScratchBlock& b : g_scratch_live)
+                if (b.ptr == ptr && b.pins > 0) b.pins -= 1;
+        }
+        auto it = g_recording_idle.find(r->id);
+        if (it != g_recording_idle.end()) {
+            idle.swap(it->second);
+            g_recording_idle.erase(it);    // blocks of this recording that are still live are ordinary blocks from now on
+        }
+        // its released blocks join the blocks kept for everybody
+        for (FreeBlock& f : idle) {
+            f.info.recording = 0;
+            g_mem_free.push_back(f);
+            g_mem_kept += f.info.size;
+        }
+    }
+    (void)hipGetLastError();
+    delete r;
 }
 
 void* tannic_hip_event_create(void) {

@@ -1,0 +1,123 @@
+"""Backend calls recorded into a HIP graph and replayed (``tannic_hip_graph_*``, ``tannic_amd.Graph``).
+
+A replay must give what the eager calls give, every time: the graph is launched several times with the program's own
+eager work and waits between the launches, and each replay is compared bit for bit with the eager result."""
+import numpy as np
+import pytest
+
+import support
+import tannic_amd as ta
+from tannic_amd import decoder_layer as dl, ops
+
+pytestmark = pytest.mark.gpu
+
+
+def small_layer(dtype, env, seed):
+    s = dl.LayerShape(hidden=256, heads=4, kv_heads=2, head_dim=64, ffn=512)
+    seq = 48
+    w = {}
+    for i, (name, shape) in enumerate(dl.weight_shapes(s).items()):
+        values = np.ones(shape) if name.startswith("g") else support.normal(seed, 10 + i, shape, 0.05)
+        w[name] = ta.tensor(values, dtype, env)
+    x = ta.tensor(support.normal(seed, 1, (1, seq, s.hidden), 1.0), dtype, env)
+    cos, sin = dl.rotary_tables(s, seq, dtype, env)
+    return s, w, x, cos, sin, dl.causal_mask(seq, dtype, env), ta.tensor(np.ones(1), dtype, env)
+
+
+def eager_noise(env, rounds=3):
+    """Eager work of the sizes the layer uses: takes and returns blocks the way an unrelated caller would."""
+    kept = []
+    for r in range(rounds):
+        a = ta.tensor(support.normal(50 + r, 0, (1, 48, 256), 1.0), ta.bfloat16, env)
+        b = ops.add(a, a)
+        c = ops.matmul(b, ta.tensor(support.normal(60 + r, 0, (256, 512), 0.1), ta.bfloat16, env))
+        kept.append((ops.mul(c, c), None))
+    return kept
+
+
+@pytest.mark.parametrize("dtype", [ta.bfloat16, ta.float32], ids=["bfloat16", "float32"])
+def test_replays_of_a_layer_equal_the_eager_layer(device, dtype):
+    s, w, x, cos, sin, mask, one = small_layer(dtype, device, 5)
+    want = dl.forward(s, w, x, cos, sin, mask, one).storage()
+    with ta.Graph(device) as g:
+        y = dl.forward(s, w, x, cos, sin, mask, one)
+    for replay in range(4):
+        g.launch()
+        np.testing.assert_array_equal(y.storage(), want, err_msg=f"replay {replay}")
+        eager_noise(device)
+        # the eager layer between replays gives the same too (it shares the stream and the kept blocks with the graph)
+        np.testing.assert_array_equal(dl.forward(s, w, x, cos, sin, mask, one).storage(), want)
+    g.close()
+    np.testing.assert_array_equal(y.storage(), want)      # a live tensor outlives the recording that made it
+
+
+def test_replay_reads_the_inputs_as_they_are_at_launch(device):
+    s, w, x, cos, sin, mask, one = small_layer(ta.bfloat16, device, 6)
+    with ta.Graph(device) as g:
+        y = dl.forward(s, w, x, cos, sin, mask, one)
+    g.launch()
+    first = y.storage()
+    other = ta.tensor(support.normal(7, 1, x.shape, 1.0), ta.bfloat16, device)
+    want = dl.forward(s, w, other, cos, sin, mask, one).storage()
+    ops.copy_into(x, other)
+    g.launch()
+    second = y.storage()
+    np.testing.assert_array_equal(second, want)
+    assert (first != second).any()
+
+
+def test_a_recording_keeps_its_memory_to_itself(device):
+    """Tensors allocated after the recording, of the sizes of its temporaries, are not written by a replay."""
+    s, w, x, cos, sin, mask, one = small_layer(ta.bfloat16, device, 8)
+    with ta.Graph(device) as g:
+        y = dl.forward(s, w, x, cos, sin, mask, one)
+    g.launch()
+    want = y.storage()
+    sizes = [(1, 48, 256), (1, 48, 512), (1, 4, 48, 48), (1, 4, 48, 64), (1, 2, 48, 64), (48, 64)]
+    bystanders = []
+    for i, shape in enumerate(sizes * 6):
+        values = support.normal(9, i, shape, 1.0)
+        t = ta.tensor(values, ta.bfloat16, device)
+        bystanders.append((t, t.storage()))
+    g.launch()
+    g.launch()
+    np.testing.assert_array_equal(y.storage(), want)
+    for t, before in bystanders:
+        np.testing.assert_array_equal(t.storage(), before)
+
+
+def test_products_that_share_k_replay_with_their_partial_sums(device):
+    """A product whose workgroups share K keeps partial sums in library scratch; eager products use scratch between replays."""
+    a = ta.tensor(support.normal(11, 0, (128, 4096), 1.0), ta.float16, device)
+    b = ta.tensor(support.normal(11, 1, (4096, 4096), 0.02), ta.float16, device)
+    c = ta.tensor(support.normal(11, 2, (96, 2048), 1.0), ta.float16, device)
+    d = ta.tensor(support.normal(11, 3, (1024, 2048), 0.02), ta.float16, device)
+    want = ops.matmul(a, b.transpose()).storage()
+    with ta.Graph(device) as g:
+        y = ops.matmul(a, b.transpose())
+        z = ops.add(y, y)
+    for replay in range(3):
+        g.launch()
+        np.testing.assert_array_equal(y.storage(), want, err_msg=f"replay {replay}")
+        ops.matmul(c, d.transpose())
+        ops.matmul(a, b.transpose())
+    assert z.shape == y.shape
+
+
+def test_calls_that_wait_are_refused_while_recording(device):
+    x = ta.tensor(np.arange(8.0), ta.float32, device)
+    with pytest.raises(ta.BackendError, match="being recorded"):
+        with ta.Graph(device):
+            y = ops.add(x, x)
+            y.numpy()
+    # the failed recording is gone; the device works as before
+    np.testing.assert_array_equal(ops.add(x, x).numpy(), 2 * np.arange(8.0))
+    with ta.Graph(device) as g:
+        y = ops.add(x, x)
+    g.launch()
+    np.testing.assert_array_equal(y.numpy(), 2 * np.arange(8.0))
+    with pytest.raises(ta.BackendError):
+        with ta.Graph(device):
+            with ta.Graph(device):
+                pass
+    np.testing.assert_array_equal(ops.add(x, x).numpy(), 2 * np.arange(8.0))
