@@ -254,16 +254,20 @@ int launch_elementwise(F f, Plan p, hipStream_t stream) {
     p.total_vectors = rows * p.row_vectors;
     if (p.total_vectors == 0) return TANNIC_SUCCESS;
     const bool repeats = p.rank > 1 || p.stride[0][last] == 0 || (F::sources == 2 && p.stride[1][last] == 0);
-    const uint32_t per_block = kBlock * (repeats ? 2 : 1);
+    // Two vectors per thread pay only when the blocks are many generations deep (1 GiB with a broadcast operand: 6 %
+    // faster); at the sizes of a layer's activations (16 MB: one or two generations) one vector per thread and twice
+    // the blocks let stores of early blocks overlap loads of late ones (15 of a decoder layer's 600 us).
+    const bool two = repeats && p.total_vectors >= (1u << 23);
+    const uint32_t per_block = kBlock * (two ? 2 : 1);
     const uint32_t grid = (p.total_vectors + per_block - 1) / per_block;
     if constexpr (VEC > 1) {
         if (vec) {
-            if (repeats) hipLaunchKernelGGL((elementwise_kernel<F, VEC, 2>), dim3(grid), dim3(kBlock), 0, stream, f, p);
+            if (two) hipLaunchKernelGGL((elementwise_kernel<F, VEC, 2>), dim3(grid), dim3(kBlock), 0, stream, f, p);
             else hipLaunchKernelGGL((elementwise_kernel<F, VEC, 1>), dim3(grid), dim3(kBlock), 0, stream, f, p);
             return launch_status("elementwise_kernel");
         }
     }
-    if (repeats) hipLaunchKernelGGL((elementwise_kernel<F, 1, 2>), dim3(grid), dim3(kBlock), 0, stream, f, p);
+    if (two) hipLaunchKernelGGL((elementwise_kernel<F, 1, 2>), dim3(grid), dim3(kBlock), 0, stream, f, p);
     else hipLaunchKernelGGL((elementwise_kernel<F, 1, 1>), dim3(grid), dim3(kBlock), 0, stream, f, p);
     return launch_status("elementwise_kernel");
 }

@@ -54,10 +54,7 @@ def _call(name, env, sources, dst, extra=(), scalar=None):
     args.append(dst.reference())
     if env.kind == abi.DEVICE:
         lib = library()
-        reference = env.reference
-        stream = lib.pop_stream(reference)
-        status = lib.kernels[name](*args, stream, *extra)
-        lib.put_stream(reference, stream)
+        status = lib.kernels[name](*args, env.stream(), *extra)
         if status == abi.SUCCESS:
             return dst
         detail = lib.error_message() if status == abi.ERROR else ""

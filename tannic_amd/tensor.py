@@ -32,6 +32,9 @@ class Host:
         return "Host()"
 
 
+_STREAMS = {}      # device id -> its stream (see Device.stream)
+
+
 class Device:
     """One GPU.  Mirrors ``Device::Device`` (``src/resources.cpp:44-49``): ids outside
     ``[0, getDeviceCount())`` raise ``IndexError`` (``std::out_of_range`` there)."""
@@ -48,6 +51,18 @@ class Device:
 
     def structure(self):
         return self._structure
+
+    def stream(self):
+        """The stream this device's backend calls run on.  The reference pops a stream from a per-device LIFO pool
+        before every call and puts it back after (``src/bindings.cpp:22-42``, ``src/cuda/streams.cu:23-38``), which hands
+        a host thread the same stream every time; this mirror asks the pool once per device and keeps the answer."""
+        stream = _STREAMS.get(self.id)
+        if stream is None:
+            lib = library()
+            stream = lib.pop_stream(self.reference)
+            lib.put_stream(self.reference, stream)
+            _STREAMS[self.id] = stream
+        return stream
 
     def __eq__(self, other):
         return isinstance(other, Device) and other.id == self.id
