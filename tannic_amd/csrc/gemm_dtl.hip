@@ -65,7 +65,8 @@ template <class T> __device__ inline void mfma16x16_in_place(typename DtlTypes<T
     }
 }
 
-// BM x BN: 256 x 256, 256 x 128 or 128 x 128 (2 x 2 wavefronts each).  The smaller tiles are for products with too few
+// BM x BN: 256 x 256, 256 x 224, 256 x 192, 256 x 128 or 128 x 128 (2 x 2 wavefronts each; BN any multiple of 32 for
+// operands contiguous along K, a power of two for k-rows).  The smaller tiles are for products with too few
 // large tiles to fill the chip; two workgroups of the smallest share a compute unit.
 // SPLIT: `sk.splits` workgroups share a tile, each taking sk.k_chunk of K and storing its fp32 accumulators.
 // A_T, B_T: the operand is contiguous along M (N) and its tile is kept as k-rows.
@@ -292,13 +293,16 @@ __global__ __launch_bounds__(256, BLOCKS_PER_CU) void gemm16_dtl_kernel(const T*
             __builtin_memcpy(&bits, out, 8);
             *reinterpret_cast<uint2*>(stage + (i * 16 + lane % 16) * PITCH + j * 16 + 4 * (lane / 16)) = bits;
         }
-    constexpr int LANES_PER_ROW = WN / 8, ROWS_PER_PASS = 64 / LANES_PER_ROW;
-    const uint32_t col = n0 + wn + (lane % LANES_PER_ROW) * 8;
+    // a row of the wavefront's block is WN / 8 stores of 16 bytes: that many lanes per row, or the next power of two with the
+    // lanes beyond the row idle (tile widths that are not a power of two)
+    constexpr int PIECES = WN / 8, LANES_PER_ROW = PIECES <= 4 ? 4 : PIECES <= 8 ? 8 : 16, ROWS_PER_PASS = 64 / LANES_PER_ROW;
+    static_assert(PIECES <= 16, "a wavefront's block is at most 128 columns wide");
+    const uint32_t piece = lane % LANES_PER_ROW, col = n0 + wn + piece * 8;
 #pragma unroll
     for (int r0 = 0; r0 < WM; r0 += ROWS_PER_PASS) {
         const uint32_t r = r0 + lane / LANES_PER_ROW, row = m0 + wm + r;
-        const uint4v bits = *reinterpret_cast<const uint4v*>(stage + r * PITCH + (lane % LANES_PER_ROW) * 8);
-        if (row < p.M && col < p.N) *reinterpret_cast<uint4v*>(c + static_cast<int64_t>(row) * p.c_rs + col) = bits;
+        if (piece < PIECES && row < p.M && col < p.N)
+            *reinterpret_cast<uint4v*>(c + static_cast<int64_t>(row) * p.c_rs + col) = *reinterpret_cast<const uint4v*>(stage + r * PITCH + piece * 8);
     }
     }
 #endif
@@ -398,6 +402,11 @@ int gemm16_dtl(const GemmProblem& p, int bm, int bn, const void* a, const void* 
     }
     // as many stages as LDS holds (160 KB): the smaller the tile, the shorter its step and the more steps a load needs to arrive
     if (bm == 256 && bn == 256) return launch_dtl<T, 256, 256, 2>(p, a, b, c, stream);
+    if constexpr (sizeof(T) == 2) {
+        // widths between the powers of two, for extents that leave the last round of 256-wide tiles mostly empty
+        if (bm == 256 && bn == 224) return launch_dtl<T, 256, 224, 2>(p, a, b, c, stream);
+        if (bm == 256 && bn == 192) return launch_dtl<T, 256, 192, 2>(p, a, b, c, stream);
+    }
     if (bm == 256 && bn == 128) return launch_dtl<T, 256, 128, 3>(p, a, b, c, stream);
     if (bm == 128 && bn == 128) return launch_dtl<T, 128, 128, 4>(p, a, b, c, stream);
     return TANNIC_UNSUPPORTED_DTYPE;

@@ -541,6 +541,10 @@ int run16_split(const GemmProblem& p, bool ak, bool bk, uint32_t splits, const v
     return status;
 }
 
+// What a 256-row tile narrower than 256 columns loses per column it is narrower (operand bytes per multiply-add), as a
+// fraction of its time.
+constexpr double kNarrowTilePenalty = 0.001;
+
 template <class T>
 int run16(const GemmProblem& p, const void* a, const void* b, void* c, hipStream_t stream, const GemmWorkspace* workspace) {
     if (p.M == 0 || p.N == 0 || p.batches == 0) return TANNIC_SUCCESS;
@@ -565,9 +569,28 @@ int run16(const GemmProblem& p, const void* a, const void* b, void* c, hipStream
         if (p.M > 64) return launch16<T, 128, 128, 2, true, true, false, false>(p, a, b, c, stream);
         return launch16<T, 64, 128, 2, true, true, false, false>(p, a, b, c, stream);
     }
-    // Tile height by M (a tile taller than M multiplies padding), large tiles only when they still give every CU work.
-    const uint64_t big = static_cast<uint64_t>((p.M + 255) / 256) * ((p.N + 255) / 256) * p.batches;
-    if (p.M > 192 && big >= 200) {
+    // Tile height by M (a tile taller than M multiplies padding).  Large tiles when they give (nearly) every compute unit one.  Tile width: 256 unless a narrower one needs less time
+    // for its rounds over the 256 compute units (2048 x 14336: 448 tiles 256 wide are two rounds, the second three
+    // quarters full; 512 tiles 224 wide are two full rounds of tiles that take 7/8 of the time; 2048 x 6144 is 192 tiles
+    // 256 wide, and exactly 256 tiles 192 wide).  A narrower tile reads more operand bytes per multiply-add: it has to win
+    // by more than that.
+    const uint64_t tiles_m = (p.M + 255) / 256;
+    int width = 0;
+    double least = 1e30;
+    for (int w : {256, 224, 192}) {
+        if (w != 256 && (sizeof(T) != 2 || !(ak && bk))) continue;   // fp32 tiles and k-row tiles are powers of two wide
+        const uint64_t tiles = tiles_m * ((p.N + w - 1) / w) * p.batches;
+        if (tiles < 200) continue;
+        const double cost = static_cast<double>((tiles + 255) / 256) * w * (1.0 + (256 - w) * kNarrowTilePenalty);
+        if (cost < least) { least = cost; width = w; }
+    }
+    if constexpr (sizeof(T) == 2) {
+        if (p.M > 192 && width && width != 256) {
+            const int rc = gemm16_dtl<T>(p, 256, width, a, b, c, stream);
+            if (rc != TANNIC_UNSUPPORTED_DTYPE) return rc;
+        }
+    }
+    if (p.M > 192 && tiles_m * ((p.N + 255) / 256) * p.batches >= 200) {
         if constexpr (sizeof(T) == 2) {
             const int rc = gemm16_dtl<T>(p, 256, 256, a, b, c, stream);
             if (rc != TANNIC_UNSUPPORTED_DTYPE) return rc;

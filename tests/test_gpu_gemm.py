@@ -180,6 +180,27 @@ def test_operands_contiguous_along_m_or_n_on_direct_tiles(device, dtype, shape):
         support.assert_bit_exact(got, nt, f"{name} against nt, {dtype} {shape}")
 
 
+@pytest.mark.parametrize("shape", [(2048, 14336, 256), (2048, 12288, 192), (2000, 14000, 128), (2048, 12200, 64)], ids=str)
+@pytest.mark.parametrize("dtype", [ta.float16, ta.bfloat16], ids=str)
+def test_tile_widths_between_the_powers_of_two(device, dtype, shape):
+    """Extents for which 256 x 224 and 256 x 192 tiles need fewer rounds than 256 x 256 ones, with whole and with ragged
+    last tiles along both M and N: X . W^T against float64 on sampled rows (all columns, so every tile column is seen),
+    and, where N is a whole number of 256-wide tiles, bit for bit against X . W, which runs 256-wide k-row tiles."""
+    m, n, k = shape
+    x = support.values_for(dtype, SEED, 7, (m, k), -1, 1)
+    w = support.values_for(dtype, SEED, 8, (k, n), -1, 1)
+    hx, dx = support.both(x, dtype, device)
+    hw, dw = support.both(w, dtype, device)
+    _, dwt = support.both(np.ascontiguousarray(w.T), dtype, device)
+    nt = ops.matmul(dx, dwt.transpose()).numpy()
+    rows = np.concatenate([np.random.default_rng(SEED).choice(m, 30, replace=False), [0, m - 1]])
+    exact = np.matmul(hx.numpy().astype(np.float64)[rows, :], hw.numpy().astype(np.float64))
+    rtol = 2e-3 if dtype is ta.float16 else 2.0 ** -7
+    support.assert_close(nt[rows, :], exact, rtol, 1e-3 * np.sqrt(k), f"nt {dtype} {shape}")
+    if n % 256 == 0 and m % 256 == 0:
+        support.assert_bit_exact(ops.matmul(dx, dw).numpy(), nt, f"nn against nt, {dtype} {shape}")
+
+
 def test_integer_valued_fp16_gemm_is_exact(device):
     """Small integers: every product and partial sum is exact in fp32, so any order of summation agrees."""
     a = support.integers(SEED, 3, (192, 320), -4, 4)
