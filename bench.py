@@ -420,6 +420,7 @@ def secondary(b, only):
     if only in (None, "gemm"):
         for (m, n) in [(2048, 4096), (2048, 14336), (128, 4096), (128, 14336), (16, 4096), (16, 14336), (1, 4096), (1, 14336)]:
             work.append(gemm_entry(b, ta.float16, m, n, 4096, 20))
+        work.append(gemm_entry(b, ta.float16, 2048, 6144, 4096, 20))     # 192 tiles 256 wide, 256 tiles 192 wide
         work.append(gemm_entry(b, ta.float16, 4096, 4096, 4096, 20, "NN"))
         work.append(gemm_entry(b, ta.float16, 4096, 4096, 4096, 20, "TN"))
         work.append(gemm_entry(b, ta.bfloat16, 4096, 4096, 4096, 20))
