@@ -35,9 +35,11 @@ class TannicError(RuntimeError):
 
 def _resolve(*tensors):
     """``resolve_two_environment`` / ``resolve_three_environment`` (``src/bindings.cpp:118-188``)."""
+    if len(tensors) == 2:
+        first, second = tensors[0].buffer, tensors[1].buffer
+        if first is not None and second is not None and first.environment is second.environment:
+            return first.environment
     envs = [t.environment for t in tensors]
-    if len(envs) == 2 and envs[0] is envs[1]:
-        return envs[0]
     devices = [e for e in envs if isinstance(e, Device)]
     if not devices:
         return Host()
@@ -83,6 +85,9 @@ def broadcast(first, second):
     """``operation::broadcast`` (``include/tannic/operations.hpp:137-152``)."""
     if first == second:
         return tuple(first)
+    known = _BROADCASTS.get((first, second))
+    if known is not None:
+        return known
     rank = builtins.max(len(first), len(second))
     out = []
     for d in range(rank):
@@ -91,7 +96,13 @@ def broadcast(first, second):
         if not (a == b or a == 1 or b == 1):
             raise TannicError("Shapes are not broadcast-compatible.")
         out.append(builtins.max(a, b))
-    return tuple(out)
+    if len(_BROADCASTS) > 4096:
+        _BROADCASTS.clear()
+    known = _BROADCASTS[(tuple(first), tuple(second))] = tuple(out)
+    return known
+
+
+_BROADCASTS = {}    # (shape, shape) -> broadcast shape: the pairs of a program recur
 
 
 # ---- unary functions (include/tannic/functions.hpp:52-57: contiguous target) ----

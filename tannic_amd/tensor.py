@@ -106,6 +106,7 @@ _PAD = [(0,) * (abi.DIMENSIONS - r) for r in range(abi.DIMENSIONS + 1)]
 assert _TENSOR_T.size == C.sizeof(abi.tensor_t)
 
 
+_IMAGES = {}      # (shape, strides, dtype, environment) -> packed tensor_t without the address
 _STRIDES = {}     # shape -> (contiguous strides, number of elements); shapes recur, the table stays small
 
 
@@ -272,13 +273,21 @@ class Tensor:
         cached = self.__dict__.get("_descriptor")
         if cached is not None:
             return cached
-        # one packed image of ``tensor_t`` (offsets checked against the structure when ``abi`` is imported)
-        rank, env = len(self.shape), self.buffer.environment
-        pad = _PAD[rank]
-        layout = abi.SINGLETON if self.nelements == 1 else abi.CONTIGUOUS if self.is_contiguous() else abi.STRIDED
-        resource = env.id if env.kind == abi.DEVICE else abi.PAGEABLE
-        t = abi.tensor_t.from_buffer_copy(_TENSOR_T.pack(self.buffer.address + self.offset, rank, *self.shape, *pad, *self.strides, *pad, self.dtype.code,
-                                                         env.kind, resource, self.nelements, layout))
+        # One packed image of ``tensor_t`` per (shape, strides, dtype, environment), kept; a tensor's own descriptor is a copy
+        # of it with the address filled in (offsets checked against the structure when ``abi`` is imported).
+        env = self.buffer.environment
+        key = (self.shape, self.strides, self.dtype.code, env.kind, env.id if env.kind == abi.DEVICE else -1)
+        image = _IMAGES.get(key)
+        if image is None:
+            rank = len(self.shape)
+            pad = _PAD[rank]
+            layout = abi.SINGLETON if self.nelements == 1 else abi.CONTIGUOUS if self.is_contiguous() else abi.STRIDED
+            resource = env.id if env.kind == abi.DEVICE else abi.PAGEABLE
+            if len(_IMAGES) > 4096:
+                _IMAGES.clear()
+            image = _IMAGES[key] = _TENSOR_T.pack(0, rank, *self.shape, *pad, *self.strides, *pad, self.dtype.code, env.kind, resource, self.nelements, layout)
+        t = abi.tensor_t.from_buffer_copy(image)
+        t.address = self.buffer.address + self.offset
         self._descriptor = t
         self._reference = C.byref(t)
         return t
