@@ -2,12 +2,14 @@
 
 A replay must give what the eager calls give, every time: the graph is launched several times with the program's own
 eager work and waits between the launches, and each replay is compared bit for bit with the eager result."""
+import ctypes as C
+
 import numpy as np
 import pytest
 
 import support
 import tannic_amd as ta
-from tannic_amd import decoder_layer as dl, ops
+from tannic_amd import abi, decoder_layer as dl, ops
 
 pytestmark = pytest.mark.gpu
 
@@ -102,6 +104,24 @@ def test_products_that_share_k_replay_with_their_partial_sums(device):
         ops.matmul(c, d.transpose())
         ops.matmul(a, b.transpose())
     assert z.shape == y.shape
+
+
+def test_the_product_that_allocates_nothing_can_be_recorded(device):
+    """tannic_hip_gemm_noalloc with a destination that exists before the recording: the recording holds kernels only
+    (the partial sums of the shared K live in the library's static array), and replays equal tannic_hip_gemm."""
+    a = ta.tensor(support.normal(12, 0, (128, 4096), 1.0), ta.float16, device)
+    b = ta.tensor(support.normal(12, 1, (4096, 4096), 0.02), ta.float16, device).transpose()
+    want = ops.matmul(a, b).storage()
+    dst = ta.Tensor(ta.float16, (128, 4096)).initialize(device)
+    lib = ta.library()
+    with ta.Graph(device) as g:
+        status = lib.kernels["gemm_noalloc"](a.reference(), b.reference(), dst.reference(), device.stream())
+        assert status == abi.SUCCESS, lib.error_message()
+    for replay in range(3):
+        ops.copy_into(dst, ta.tensor(np.zeros((128, 4096)), ta.float16, device))
+        g.launch()
+        np.testing.assert_array_equal(dst.storage(), want, err_msg=f"replay {replay}")
+        ops.matmul(a, b)
 
 
 def test_calls_that_wait_are_refused_while_recording(device):
