@@ -8,6 +8,7 @@
 #include <cstdio>
 #include <cstdlib>
 #include <stdexcept>
+#include <string>
 
 #include "../../../include/tannic_hip.h"
 
@@ -100,7 +101,11 @@ status conv2d(const tensor_t* x, const tensor_t* w, const tensor_t* b, tensor_t*
 }
 bool allclose(const tensor_t* a, const tensor_t* b, stream_t q, double rtol, double atol) {
     const int r = tannic_hip_allclose(in(a), in(b), st(q), rtol, atol);
-    if (r < 0) throw std::runtime_error("Unsupported dtype");
+    if (r < 0) {
+        // the library's own words where it has said why (shapes differ, the stream is being recorded); the reference's otherwise
+        const std::string why = tannic_hip_last_error();
+        throw std::runtime_error(why.rfind("allclose", 0) == 0 ? why : "Unsupported dtype");
+    }
     return r == 1;
 }
 
@@ -129,4 +134,18 @@ status softmax(const tensor_t* x, const tensor_t* mask, tensor_t* d, stream_t q,
     return code(tannic_hip_softmax(in(x), mask ? in(mask) : nullptr, out(d), st(q), scale));
 }
 status rope(const tensor_t* x, const tensor_t* c, const tensor_t* s, tensor_t* d, stream_t q) { return code(tannic_hip_rope(in(x), in(c), in(s), out(d), st(q))); }
+
+Recording::Recording(int device) {
+    tannic_device_t dvc{};
+    dvc.id = device;
+    handle_ = tannic_hip_graph_begin(&dvc);
+    if (!handle_) throw std::runtime_error(std::string("Recording: ") + tannic_hip_last_error());
+}
+Recording::~Recording() { tannic_hip_graph_destroy(handle_); }
+void Recording::end() {
+    if (tannic_hip_graph_end(handle_) != TANNIC_SUCCESS) throw std::runtime_error(std::string("Recording::end: ") + tannic_hip_last_error());
+}
+void Recording::launch() {
+    if (tannic_hip_graph_launch(handle_) != TANNIC_SUCCESS) throw std::runtime_error(std::string("Recording::launch: ") + tannic_hip_last_error());
+}
 }  // namespace tannic_hip

@@ -131,4 +131,26 @@ status cast(const tensor_t*, tensor_t*, stream_t);
 status rms_norm(const tensor_t* x, const tensor_t* gain, tensor_t*, stream_t, float eps);
 status softmax(const tensor_t* x, const tensor_t* mask_or_null, tensor_t*, stream_t, float scale);
 status rope(const tensor_t* x, const tensor_t* cos, const tensor_t* sin, tensor_t*, stream_t);
+
+// A sequence of the front end's evaluations on one device recorded once and replayed as one HIP graph
+// (tannic_hip_graph_begin / end / launch / destroy):
+//     tannic_hip::Recording r(0);          // device 0's stream is recording
+//     Tensor y = f(x);                     // every backend call is recorded, none runs
+//     r.end();
+//     r.launch();                          // y holds f(x); write new values into x's memory and launch again
+// Tensors created between the constructor and end() keep their addresses and are rewritten by every launch; tensors that
+// existed before must outlive the launches.  Calls that wait for the device (copies to the host, allclose) throw while
+// the recording is open.  Throws std::runtime_error with the library's message when a step fails.
+class Recording {
+   public:
+    explicit Recording(int device = 0);
+    Recording(const Recording&) = delete;
+    Recording& operator=(const Recording&) = delete;
+    ~Recording();
+    void end();
+    void launch();
+
+   private:
+    void* handle_;
+};
 }  // namespace tannic_hip
