@@ -52,9 +52,9 @@ int gemm_mfma_16bit(const GemmProblem& p, int dtype, const void* a, const void* 
 int gemm_mfma_f32(const GemmProblem& p, const float* a, const float* b, float* c, hipStream_t stream, const GemmWorkspace* workspace = nullptr);
 // bm x bn tiles (256 x 256, 256 x 128, 128 x 128) filled by direct global -> LDS loads (gemm_dtl.hip); T is f16 or bf16
 template <class T> int gemm16_dtl(const GemmProblem& p, int bm, int bn, const void* a, const void* b, void* c, hipStream_t stream);
-// the 128 x 128 tiles with K shared between `splits` workgroups per tile (k_chunk elements each, a multiple of 64): fp32
+// the 128 x 128 (bm = 128) or 64 x 128 (bm = 64) tiles with K shared between `splits` workgroups per tile (k_chunk elements each, a multiple of 64): fp32
 // partial sums go to partials[split][batch][M][N], which the caller adds up
-template <class T> int gemm16_dtl_split(const GemmProblem& p, uint32_t splits, uint32_t k_chunk, float* partials, const void* a, const void* b, hipStream_t stream);
+template <class T> int gemm16_dtl_split(const GemmProblem& p, int bm, uint32_t splits, uint32_t k_chunk, float* partials, const void* a, const void* b, hipStream_t stream);
 // int8 x int8 -> int32 on the same tiles (v_mfma_i32_16x16x64_i8)
 int gemm_mfma_int8(const GemmProblem& p, const void* a, const void* b, void* c, hipStream_t stream);
 

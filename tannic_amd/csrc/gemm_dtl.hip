@@ -376,17 +376,25 @@ static bool operands_fit(const GemmProblem& p, int bm, int bn, bool& a_t, bool& 
 }
 
 template <class T>
-int gemm16_dtl_split(const GemmProblem& p, uint32_t splits, uint32_t k_chunk, float* partials, const void* a, const void* b, hipStream_t stream) {
+int gemm16_dtl_split(const GemmProblem& p, int bm, uint32_t splits, uint32_t k_chunk, float* partials, const void* a, const void* b, hipStream_t stream) {
     bool a_t, b_t;
-    if (!operands_fit<T>(p, 128, 128, a_t, b_t) || p.N % 4 != 0 || k_chunk % 64 != 0) return TANNIC_UNSUPPORTED_DTYPE;
+    if (!operands_fit<T>(p, bm, 128, a_t, b_t) || p.N % 4 != 0 || k_chunk % 64 != 0) return TANNIC_UNSUPPORTED_DTYPE;
     const SplitK sk{splits, k_chunk, partials};
+    if (bm == 64) {
+        // 64 x 128 tiles, six stages: a workgroup's share of K is short and its operands are in no cache, so what counts
+        // is how much of that share is on its way at once (operands contiguous along K only: a k-row tile is at least
+        // 128 wide)
+        if (a_t || b_t) return TANNIC_UNSUPPORTED_DTYPE;
+        return launch_dtl<T, 64, 128, 6, true>(p, a, b, nullptr, stream, sk);
+    }
+    if (bm != 128) return TANNIC_UNSUPPORTED_DTYPE;
     if constexpr (sizeof(T) == 2) {
         if (a_t || b_t) return gemm16_dtl_krows<T>(p, 128, 128, a_t, b_t, sk, a, b, nullptr, stream);
     }
     return launch_dtl<T, 128, 128, 4, true>(p, a, b, nullptr, stream, sk);
 }
-template int gemm16_dtl_split<f16>(const GemmProblem&, uint32_t, uint32_t, float*, const void*, const void*, hipStream_t);
-template int gemm16_dtl_split<bf16>(const GemmProblem&, uint32_t, uint32_t, float*, const void*, const void*, hipStream_t);
+template int gemm16_dtl_split<f16>(const GemmProblem&, int, uint32_t, uint32_t, float*, const void*, const void*, hipStream_t);
+template int gemm16_dtl_split<bf16>(const GemmProblem&, int, uint32_t, uint32_t, float*, const void*, const void*, hipStream_t);
 
 // Returns TANNIC_UNSUPPORTED_DTYPE when the problem is not this kernel's: the caller then takes the register-staged one.
 template <class T>

@@ -525,7 +525,7 @@ int run16_split(const GemmProblem& p, bool ak, bool bk, uint32_t splits, const v
         return TANNIC_ERROR;
     }
     int status = TANNIC_UNSUPPORTED_DTYPE;
-    if constexpr (sizeof(T) == 2 && BM == 128) status = gemm16_dtl_split<T>(p, sk.splits, sk.k_chunk, sk.partials, a, b, stream);
+    if constexpr (sizeof(T) == 2 && (BM == 128 || BM == 64)) status = gemm16_dtl_split<T>(p, BM, sk.splits, sk.k_chunk, sk.partials, a, b, stream);
     if (status != TANNIC_UNSUPPORTED_DTYPE) {}
     else if (ak && bk) status = launch16<T, BM, BN, 2, true, true, true>(p, a, b, c, stream, sk);
     else if (ak) status = launch16<T, BM, BN, 2, true, false, true>(p, a, b, c, stream, sk);
