@@ -228,3 +228,24 @@ def test_full_size_layer_is_causal(layer, device, form):
     before = layer[form]["out"].numpy()
     np.testing.assert_array_equal(again[0, :300], before[0, :300])
     assert np.abs(again[0, 300:].astype(np.float64) - before[0, 300:].astype(np.float64)).max() > 1e-2
+
+
+@pytest.mark.parametrize("form", ["composed", "one_pass"])
+def test_full_size_layer_replayed_as_a_graph_equals_the_eager_layer(layer, device, form):
+    """Both forms recorded once (58 and 19 backend calls, the products that share K with their partial sums among them)
+    and replayed three times, with an eager layer between replays: every replay equals the eager result bit for bit."""
+    L = layer
+    if form == "composed":
+        run = lambda: dl.forward(L["s"], L["w"], L["dx"], L["cos"], L["sin"], L["mask"], L["one"])
+        want = L["composed"]["out"].storage()
+    else:
+        run = lambda: dl.forward_fused(L["s"], L["packed"], L["dx"], L["cos"], L["sin"], L["mask"])
+        want = L["fused"]["out"].storage()
+    with ta.Graph(device) as graph:
+        out = run()
+    for replay in range(3):
+        graph.launch()
+        np.testing.assert_array_equal(out.storage(), want, err_msg=f"{form}, replay {replay}")
+        np.testing.assert_array_equal(run().storage(), want, err_msg=f"{form}, eager after replay {replay}")
+    graph.close()
+    gc.collect()
