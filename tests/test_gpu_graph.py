@@ -106,6 +106,49 @@ def test_products_that_share_k_replay_with_their_partial_sums(device):
     assert z.shape == y.shape
 
 
+def test_every_operator_family_replays(device):
+    """One recording that holds kernels of every family, those with library scratch among them (the gathered signal of
+    an fp32 convolution, the rearranged weights of a 16-bit one, partial results of a column reduction, partial sums of
+    a product): two replays with other eager work in between equal the eager results bit for bit."""
+    f16, f32 = ta.float16, ta.float32
+    img16 = ta.tensor(support.normal(13, 0, (4, 64, 28, 28), 1.0), f16, device)
+    ker16 = ta.tensor(support.normal(13, 1, (64, 64, 3, 3), 0.05), f16, device)
+    img32 = ta.tensor(support.normal(13, 2, (2, 6, 20, 20), 1.0), f32, device)
+    ker32 = ta.tensor(support.normal(13, 3, (5, 6, 3, 3), 0.3), f32, device)
+    bias32 = ta.tensor(support.normal(13, 4, (5,), 1.0), f32, device)
+    big = ta.tensor(support.normal(13, 5, (16, 2048, 96), 1.0), f32, device)
+    other = ta.tensor(support.normal(13, 6, (16, 2048, 96), 1.0), f32, device)
+    rows = ta.tensor(support.normal(13, 7, (300, 1000), 1.0), ta.bfloat16, device)
+    gain = ta.tensor(support.normal(13, 8, (1000,), 1.0), ta.bfloat16, device)
+    a = ta.tensor(support.normal(13, 9, (96, 4096), 1.0), f16, device)
+    b = ta.tensor(support.normal(13, 10, (2048, 4096), 0.02), f16, device)
+    rho = ta.tensor(support.uniform(13, 11, (40, 30), 0.5, 2.0), f32, device)
+    theta = ta.tensor(support.uniform(13, 12, (40, 30), -3.0, 3.0), f32, device)
+
+    def everything():
+        return [
+            ops.convolve2d(img16, ker16, None, 1, 1),
+            ops.convolve2d(img32, ker32, bias32, 2, 1),
+            ops.sum(big, 1), ops.mean(big, 0), ops.argmax(big, 1), ops.max(big, 2),
+            ops.gt(big, other), ops.add(ops.exp(ops.neg(ops.abs(big))), other),
+            ops.realify(ops.polar(rho, theta)),
+            ops.repeat(img32, 3, 1), ops.concatenate(big, other, 2), ops.triu(rho, 1), ops.outer(bias32, bias32),
+            ops.softmax(rows), ops.rms_norm(rows, gain), ops.cast(rows, f32),
+            ops.matmul(a, b.transpose()),
+        ]
+
+    want = [t.storage() for t in everything()]
+    with ta.Graph(device) as g:
+        recorded = everything()
+    for replay in range(2):
+        g.launch()
+        for i, (t, w) in enumerate(zip(recorded, want)):
+            np.testing.assert_array_equal(t.storage(), w, err_msg=f"replay {replay}, result {i}")
+        for t, w in zip(everything(), want):       # eager calls take the same scratch between replays
+            np.testing.assert_array_equal(t.storage(), w)
+        eager_noise(device)
+
+
 def test_the_product_that_allocates_nothing_can_be_recorded(device):
     """tannic_hip_gemm_noalloc with a destination that exists before the recording: the recording holds kernels only
     (the partial sums of the shared K live in the library's static array), and replays equal tannic_hip_gemm."""
