@@ -128,6 +128,25 @@ case("concat_expanded_with_transposed", "tests/cpu/test-concat.cpp:51-84", "conc
      [tv([1,1,3],[100,200,300],expand=[2,-1,-1]), tv([2,3,4],list(range(1,25)),transpose=[1,2])],
      t([2,5,3],[100,200,300,1,5,9,2,6,10,3,7,11,4,8,12,100,200,300,13,17,21,14,18,22,15,19,23,16,20,24]), axis=1)
 case("outer_vectors", "tests/cpu/test-outer-product.cpp:7-23", "outer", [t([2],[1.5,-2.0]), t([3],[4.0,0.0,-1.0])], t([2,3],[6.0,0.0,-1.5,-8.0,0.0,2.0]))
+# ---- strided views copied into contiguous tensors (reshape of a transposed tensor, reads of a permuted one)
+tr = [1.0 + b*48 + c*16 + i*4 + j for b in range(2) for i in range(4) for c in range(3) for j in range(4)]
+# rows copied from the reference file, checked against the closed form above
+assert tr[0:12] == [1,2,3,4,17,18,19,20,33,34,35,36] and tr[36:48] == [13,14,15,16,29,30,31,32,45,46,47,48]
+assert tr[48:60] == [49,50,51,52,65,66,67,68,81,82,83,84] and tr[84:96] == [61,62,63,64,77,78,79,80,93,94,95,96]
+case("repack_transposed_then_reshaped", "tests/cpu/test-non-contiguous.cpp:12-76", "repack", [tv([2,3,4,4],seq96,transpose=[1,2])], t([2,4,3,4],tr))
+pm = [1.0 + j*12 + k*4 + i for i in range(4) for j in range(2) for k in range(3)]      # the formula the reference test states
+case("repack_permuted_234_to_423", "tests/cpu/test-repeats.cpp:55-81", "repack", [tv([2,3,4],[float(v) for v in range(1,25)],permute=[2,0,1])], t([4,2,3],pm))
+# ---- complex views
+case("complexify_then_realify", "tests/cpu/test-complex.cpp:17-38", "complex_roundtrip", [t([2,2],[1,0,2,3])], t([2,2],[1,0,2,3]))
+freqs = [1.0,0.0, 1.0,0.0, 1.0,0.0,  0.5403,0.8415, 0.9989,0.0464, 1.0,0.0022,  -0.4161,0.9093, 0.9957,0.0927, 1.0,0.0043,
+         -0.9900,0.1411, 0.9903,0.1388, 1.0,0.0065,  -0.6536,-0.7568, 0.9828,0.1846, 1.0,0.0086,  0.2837,-0.9589, 0.9732,0.2300, 0.9999,0.0108,
+         0.9602,-0.2794, 0.9615,0.2749, 0.9999,0.0129,  0.7539,0.6570, 0.9477,0.3192, 0.9999,0.0151]
+rot = [1.0,2.0,-1.7451,4.6857,-7.5363,2.0499,-8.0588,-6.9323,1.6856,-13.3472,14.6275,-7.1435,16.3942,9.8106,0.7965,21.9174,
+       17.0,18.0,18.0511,20.8596,18.8703,23.8521,19.4457,26.9596,19.7704,30.1678,19.8364,33.4596,19.6365,36.8171,19.1643,40.2216,
+       33.0,34.0,34.9208,36.0770,36.8366,38.1591,38.7400,40.2535,40.6388,42.3526,42.5205,44.4600,44.4021,46.5759,46.2705,48.7049]
+# the sequence as pairs times the frequencies [8 positions... of 3 rows][2], complexified and transposed to [3, 8]: rotary embedding by complex product
+case("rotary_embedding_by_complex_product", "tests/cpu/test-complex.cpp:110-157", "complex_mul",
+     [t([1,1,3,8,2],[float(v) for v in range(1,49)]), tv([8,3,2],freqs,transpose=[0,1])], t([1,1,3,8,2],rot), rtol=1e-4, atol=1e-3)
 json.dump(dict(note="Inputs and expected outputs held by the reference's own tests (tests/cpu/*.cpp, tests/test-types.cpp), transcribed as data; "
                "'cite' names the reference file and lines. Cases with expected_expr compare against the same libm function the reference test evaluates.",
                cases=cases), open("tests/golden/reference_vectors.json","w"), indent=0)

@@ -76,6 +76,8 @@ def run(case, env):
         out = ops.outer(ins[0], ins[1])
     elif op == "repeat":
         out = ops.repeat(ins[0], case["repeats"], case["axis"])
+    elif op == "complex_roundtrip":
+        out = ops.realify(ops.complexify(ins[0]))
     elif op == "polar":
         out = ops.realify(ops.polar(ins[0], ins[1]))
     else:
