@@ -147,6 +147,10 @@ rot = [1.0,2.0,-1.7451,4.6857,-7.5363,2.0499,-8.0588,-6.9323,1.6856,-13.3472,14.
 # the sequence as pairs times the frequencies [8 positions... of 3 rows][2], complexified and transposed to [3, 8]: rotary embedding by complex product
 case("rotary_embedding_by_complex_product", "tests/cpu/test-complex.cpp:110-157", "complex_mul",
      [t([1,1,3,8,2],[float(v) for v in range(1,49)]), tv([8,3,2],freqs,transpose=[0,1])], t([1,1,3,8,2],rot), rtol=1e-4, atol=1e-3)
+# ---- assignment of a tensor to a slice (a strided copy into existing memory)
+assigned = list(freqs)
+assigned[2*6:5*6] = [1.0] * 18
+case("assign_tensor_to_slice", "tests/cpu/test-views.cpp:392-419", "assign_rows", [t([8,3,2],freqs), t([3,3,2],[1.0]*18)], t([8,3,2],assigned), rows=[2,5])
 json.dump(dict(note="Inputs and expected outputs held by the reference's own tests (tests/cpu/*.cpp, tests/test-types.cpp), transcribed as data; "
                "'cite' names the reference file and lines. Cases with expected_expr compare against the same libm function the reference test evaluates.",
                cases=cases), open("tests/golden/reference_vectors.json","w"), indent=0)

@@ -76,6 +76,10 @@ def run(case, env):
         out = ops.outer(ins[0], ins[1])
     elif op == "repeat":
         out = ops.repeat(ins[0], case["repeats"], case["axis"])
+    elif op == "assign_rows":
+        first, last = case["rows"]
+        ops.copy_into(ins[0][first:last], ins[1])
+        out = ins[0]
     elif op == "complex_roundtrip":
         out = ops.realify(ops.complexify(ins[0]))
     elif op == "polar":
