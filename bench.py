@@ -288,6 +288,29 @@ def decoder_layer_entry(b, iters, composed=True, one_pass=True):
     return entries
 
 
+def cpp_front_end_layer_entries(iters):
+    """The same layer written with the reference's own C++ front end (tests/frontend_decoder_layer.cpp, built where the
+    reference is mounted) and evaluated by this backend through the `cuda::` adapter: a child process, waited for.  It is
+    the product driven by the reference's caller, not the CPU checker; nothing of it runs on the host's cores but the
+    front end itself."""
+    import subprocess
+    binary = os.path.join(ROOT, "oracle", "_ref", "frontend_decoder_layer")
+    label = "decoder layer bfloat16 seq 512 through the reference's C++ front end"
+    if not os.path.exists(binary):
+        return [{"op": label, "skipped": "oracle/_ref/frontend_decoder_layer is not built (needs the reference's sources at build time)"}]
+    try:
+        done = subprocess.run([binary, "full", "", str(iters)], capture_output=True, text=True, timeout=200)
+        times = json.loads([line for line in done.stdout.splitlines() if line.startswith("{")][-1])
+    except Exception as error:
+        return [{"op": label, "skipped": f"{type(error).__name__}: {error}"[:100]}]
+    flops, out = times["flops"], []
+    for key, what in (("composed_eager", "composed, eager"), ("composed_replay", "composed, recorded and replayed"),
+                      ("one_pass_eager", "one-pass nodes, eager"), ("one_pass_replay", "one-pass nodes, recorded and replayed")):
+        us = times[key + "_us"]
+        out.append({"op": f"{label}: {what}", "us": us, "tflops": round(flops / us / 1e6, 2), "mfma_frac": round(flops / us / 1e6 / MFMA_PEAK_TFLOPS["bf16"], 4)})
+    return out
+
+
 def conv_entry(b, dtype, name, xs, ws, stride, pad, iters):
     ta = b.ta
     fan_in = ws[1] * ws[2] * ws[3]
@@ -448,6 +471,9 @@ def secondary(b, only):
             work += reduction_entries(b, dtype, 10)
     if only in (None, "layer", "layer-one-pass"):
         work.extend(decoder_layer_entry(b, 20, composed=only != "layer-one-pass", one_pass=only != "layer"))
+        if only != "layer-one-pass":
+            b.sync()
+            work.extend(cpp_front_end_layer_entries(20))
     return work
 
 
