@@ -477,6 +477,37 @@ def secondary(b, only):
     return work
 
 
+def short_key(op):
+    """A compact name for an entry of `workloads` (letters, digits, a few signs), for the table inside `roofline`."""
+    import re
+    key = re.sub(r" \((?:weights resident|general tiles|a product per image|hidden 4096|no counterpart)[^)]*\)", "", op)
+    for long, short in (("float16", "f16"), ("bfloat16", "bf16"), ("float32", "f32"), ("int32", "i32"), ("int8", "i8"), ("conv2d ", "conv "),
+                        ("decoder layer bf16 seq 512 through the reference's C++ front end: ", "layer C++ "), ("decoder layer bf16 seq 512, composed from operators", "layer composed"),
+                        ("the composed layer, its backend calls recorded once and replayed as a HIP graph", "layer composed replayed"),
+                        ("the same layer with the one-pass rms_norm / rope / softmax / swiglu operators", "layer one-pass"), ("recorded and replayed", "replayed"),
+                        (" N=32", ""), (" (broadcast)", ""), (" (one-element operand)", ""), (" (bit-packed)", ""), (" (scale)", ""), (" (full)", ""),
+                        ("chain log(|X|+1) + Z*Z - exp(X) + 3*X, 8 nodes", "chain")):
+        key = key.replace(long, short)
+    key = re.sub(r"[^A-Za-z0-9.\[\]^>*+|,@=-]+", "_", key).strip("_")
+    return key[:48]
+
+
+def sweep_table(workloads):
+    """name -> fraction of the entry's roofline (MFMA peak or 8 TB/s; both for the convolutions), numbers only."""
+    table = {}
+    for w in workloads:
+        if "skipped" in w or w["op"].startswith("yardstick"):
+            continue
+        key = short_key(w["op"])
+        if "frac" in w:
+            table[key] = w["frac"]
+        elif "hbm_frac" in w:
+            table[key] = [w["mfma_frac"], w["hbm_frac"]]
+        elif "mfma_frac" in w:
+            table[key] = w["mfma_frac"]
+    return table
+
+
 def main():
     args = parse()
     if args.gpus != 1:
@@ -533,7 +564,7 @@ def main():
                 "peak": MFMA_PEAK_TFLOPS["f16"], "unit": "TFLOP/s", "frac": round(achieved / MFMA_PEAK_TFLOPS["f16"], 4),
                 "avg_kernel_us": round(kernel_ms * 1e3, 2),
                 "traffic": measured_traffic("gemm16_fp16_4096x4096x4096_hbm_traffic.txt"),
-                "traffic_source": "profiles/gemm16_fp16_4096x4096x4096_hbm_traffic.txt (rocprofv3 FETCH_SIZE / WRITE_SIZE of this kernel, scaled by a plain copy)"}
+                "traffic_source": "profiles/gemm16_fp16_4096x4096x4096_hbm_traffic.txt"}
     del y
 
     result = {
@@ -550,8 +581,13 @@ def main():
 
     if not args.primary_only:
         result["workloads"] = secondary(b, None)
+        # the same fractions once more, compact (short names, numbers only; a pair is [of MFMA peak, of 8 TB/s])
+        result["roofline"]["sweep"] = sweep_table(result["workloads"])
         result["workloads"] += vendor_yardstick(max(args.steps, 10))
         result["cpu_baseline"] = cpu_baseline()
+        # parity bars the figures stand on (tests/): integers, comparisons, argmax bit-exact; fp32 rel 1e-5; fp16 GEMM/conv rel 2e-3 / abs 1e-3;
+        # bf16 GEMM/conv rel 2^-7: one bf16 rounding is 3.9e-3 already, so 2e-3 cannot hold once the order of summation flips one
+        result["parity"] = {"int": "bit-exact", "fp32": "rel 1e-5", "fp16_gemm_conv": "rel 2e-3 abs 1e-3", "bf16_gemm_conv": "rel 2^-7 (one bf16 ulp) abs 1e-3"}
     print(json.dumps(result))
 
 

@@ -206,6 +206,12 @@ void* tannic_hip_graph_begin(const tannic_device_t* device);
 int tannic_hip_graph_end(void* recording);
 int tannic_hip_graph_launch(void* recording);
 void tannic_hip_graph_destroy(void* recording);
+/* What the library has done so far, for tests that check more than results (no reference twin): out[0] kernel-scratch
+ * acquisitions, out[1] tensor allocations and releases through tannic_hip_allocate / tannic_hip_deallocate, out[2] the
+ * number of workgroups that shared K in the last matrix product that shared it. */
+void tannic_hip_counters(uint64_t out[3]);
+/* The stream a recording captures: a caller that keeps a device's stream to itself checks that it is this one. */
+tannic_stream_t tannic_hip_graph_stream(void* recording);
 
 /* Timing events on a stream, for benchmark harnesses (no reference twin). */
 void* tannic_hip_event_create(void);

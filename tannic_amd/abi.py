@@ -149,6 +149,8 @@ def runtime_signatures():
         "graph_end": (C.c_int, [C.c_void_p]),
         "graph_launch": (C.c_int, [C.c_void_p]),
         "graph_destroy": (None, [C.c_void_p]),
+        "graph_stream": (stream_t, [C.c_void_p]),
+        "counters": (None, [C.POINTER(C.c_uint64)]),
         "event_create": (C.c_void_p, []),
         "event_destroy": (None, [C.c_void_p]),
         "event_record": (C.c_int, [C.c_void_p, stream_t]),

@@ -208,6 +208,10 @@ struct FastDiv {
     }
 };
 
+// What tannic_hip_counters reports (for tests that check what a call did, not only what it returned).
+enum Counter { kCounterScratchAcquired = 0, kCounterMemoryCalls = 1, kCounterKShares = 2, kCounters = 3 };
+void count(Counter which, uint64_t value, bool set = false);
+
 // Work scratch obtained stream-ordered for the duration of one call.
 int scratch_acquire(void** ptr, size_t nbytes, hipStream_t stream);
 int scratch_release(void* ptr, hipStream_t stream);

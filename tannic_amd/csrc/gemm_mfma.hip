@@ -510,6 +510,7 @@ int run16_split(const GemmProblem& p, bool ak, bool bk, uint32_t splits, const v
     SplitK sk{};
     sk.k_chunk = (steps + splits - 1) / splits * kBK;
     sk.splits = (p.K + sk.k_chunk - 1) / sk.k_chunk;   // no block without a step
+    count(kCounterKShares, sk.splits, true);
     const uint64_t rows = static_cast<uint64_t>(p.batches) * p.M, quads_per_row = (p.N + 3) / 4;
     if (rows * quads_per_row >= (1ull << 31)) return TANNIC_UNSUPPORTED_DTYPE;
     const size_t bytes = static_cast<size_t>(sk.splits) * rows * p.N * sizeof(float);

@@ -111,6 +111,13 @@ constexpr size_t kScratchCacheLimit = size_t(2) << 30;
 
 void release_idle_memory();   // defined below, next to the kept tensor blocks
 
+// Whether some stream is being recorded right now: memory must not go back to the driver then (a stream-ordered free on
+// the capturing stream would become a node of the graph, a wait for the device would end the capture).
+static bool recording_open() {
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    return g_capturing && g_capturing->capturing;
+}
+
 // With g_scratch_mutex held: a block handed out while `stream` is being recorded is addressed by the graph's kernels.
 static void pin_for_recording(ScratchBlock& b, hipStream_t stream) {
     if (!g_capturing || !g_capturing->capturing || g_capturing->stream != stream) return;
@@ -120,7 +127,14 @@ static void pin_for_recording(ScratchBlock& b, hipStream_t stream) {
     b.pins += 1;
 }
 
+std::atomic<uint64_t> g_counters[kCounters];
+void count(Counter which, uint64_t value, bool set) {
+    if (set) g_counters[which].store(value, std::memory_order_relaxed);
+    else g_counters[which].fetch_add(value, std::memory_order_relaxed);
+}
+
 int scratch_acquire(void** ptr, size_t nbytes, hipStream_t stream) {
+    count(kCounterScratchAcquired, 1);
     int device = 0;
     TH_TRY(hipGetDevice(&device));
     {
@@ -142,9 +156,10 @@ int scratch_acquire(void** ptr, size_t nbytes, hipStream_t stream) {
     }
     const size_t size = ((nbytes + 0xFFFF) & ~size_t(0xFFFF)) ? ((nbytes + 0xFFFF) & ~size_t(0xFFFF)) : 0x10000;
     hipError_t err = hipMalloc(ptr, size);
-    if (err == hipErrorOutOfMemory) {
+    if (err == hipErrorOutOfMemory && !recording_open()) {
         // Idle memory the library itself holds may be all that is missing: the cached scratch blocks and the tensor
         // blocks kept for reuse go back to the driver (once every stream has passed their last use), then one more try.
+        // Not while a recording is open: the frees would be issued on, and the wait would break, the capturing stream.
         (void)hipGetLastError();
         release_idle_memory();
         err = hipMalloc(ptr, size);
@@ -303,6 +318,7 @@ void th::release_idle_memory() {
 extern "C" {
 
 void* tannic_hip_allocate(const tannic_device_t* device, size_t nbytes) {
+    count(kCounterMemoryCalls, 1);
     if (!device || tannic_hip_set_device(device->id) != TANNIC_SUCCESS) return nullptr;
     retain_pool_memory(device->id);
     Streams& streams = Streams::instance();
@@ -360,6 +376,7 @@ void* tannic_hip_allocate(const tannic_device_t* device, size_t nbytes) {
 }
 
 void* tannic_hip_deallocate(const tannic_device_t* device, void* address) {
+    count(kCounterMemoryCalls, 1);
     if (!device || !address) return nullptr;
     if (tannic_hip_set_device(device->id) != TANNIC_SUCCESS) return nullptr;
     Streams& streams = Streams::instance();
@@ -387,7 +404,9 @@ void* tannic_hip_deallocate(const tannic_device_t* device, void* address) {
                 g_mem_free.push_back(FreeBlock{address, info});
                 g_mem_kept += info.size;
                 kept = true;
-                while (g_mem_kept > kMemKeepLimit && !g_mem_free.empty()) {
+                // (over the limit the oldest kept blocks go back to the driver - later, if a recording is open now: see recording_open)
+                const bool recording_now = g_capturing && g_capturing->capturing;
+                while (!recording_now && g_mem_kept > kMemKeepLimit && !g_mem_free.empty()) {
                     evict.push_back(g_mem_free.front());
                     g_mem_kept -= g_mem_free.front().info.size;
                     g_mem_free.erase(g_mem_free.begin());
@@ -526,6 +545,16 @@ void* tannic_hip_graph_begin(const tannic_device_t* device) {
     g_recording_idle[r->id];
     g_capturing = r;
     return r;
+}
+
+void tannic_hip_counters(uint64_t out[3]) {
+    for (int i = 0; i < th::kCounters; ++i) out[i] = th::g_counters[i].load(std::memory_order_relaxed);
+}
+
+tannic_stream_t tannic_hip_graph_stream(void* recording) {
+    tannic_stream_t handle{};
+    handle.address = recording ? reinterpret_cast<uintptr_t>(static_cast<Recording*>(recording)->stream) : 0;
+    return handle;
 }
 
 int tannic_hip_graph_end(void* recording) {

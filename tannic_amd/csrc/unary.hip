@@ -61,8 +61,14 @@ struct UnaryF {
             // evaluated in double whatever the element type (src/cpu/ops-unary.cpp:141-149).  For a 16-bit result the
             // hardware's reciprocal square root (1 ulp in fp32) gives the same value except where the exact one lies within
             // 2^-24 of a rounding boundary of the 16-bit type, and runs at the memory stream's speed, which double does not.
-            if constexpr (is_16bit<T>::value) return narrow<T>(__builtin_amdgcn_rsqf(widen(x) + static_cast<float>(eps)));
-            else return narrow<T>(1.0 / sqrt(static_cast<double>(widen(x)) + eps));
+            // A sum below the smallest normal float (a bfloat16 subnormal with eps = 0) is one the instruction reads as zero:
+            // it is scaled by 2^24 first and the result by 2^12.
+            if constexpr (is_16bit<T>::value) {
+                const float t = widen(x) + static_cast<float>(eps);
+                const bool tiny = t > 0.0f && t < 1.17549435e-38f;
+                const float r = __builtin_amdgcn_rsqf(tiny ? t * 16777216.0f : t);
+                return narrow<T>(tiny ? r * 4096.0f : r);
+            } else return narrow<T>(1.0 / sqrt(static_cast<double>(widen(x)) + eps));
         } else if constexpr (K == U_ABS && std::is_integral_v<T>) {
             using U = std::make_unsigned_t<T>;
             return x < 0 ? static_cast<T>(static_cast<U>(0) - static_cast<U>(x)) : x;

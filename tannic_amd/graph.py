@@ -33,6 +33,11 @@ class Graph:
         self.handle = lib.graph_begin(self.device.reference)
         if not self.handle:
             raise BackendError(lib.error_message())
+        # the operators of this harness launch on the stream the device handed out once (Device.stream); a recording on
+        # any other stream would record nothing and the calls would run eagerly
+        if lib.graph_stream(self.handle).address != self.device.stream().address:
+            self.close()
+            raise BackendError("Graph: the backend records another stream than the one this device's operators use (a stream popped and not put back?)")
         return self
 
     def __exit__(self, kind, value, trace):

@@ -203,7 +203,13 @@ def test_both_forms_and_both_parameter_layouts_agree(layer):
     composed, fused = numbers(layer["composed"]["out"]), numbers(layer["fused"]["out"])
     assert np.isfinite(composed).all() and np.isfinite(fused).all()
     spread = composed.std()
-    # (measured: 0.087 of the output's spread at most, 0.010 on average; every stage is checked by itself above)
+    # Where the bounds come from.  The stage tests above hold the activation `act` of the composed form within 7 roundings
+    # of bfloat16 of the exact value and that of the one-pass form within 1: per element the two differ by d ~ 2^-9 * |act|
+    # times a few, of either sign.  The down projection adds 14336 such terms with the weights as factors, as it adds the
+    # terms of y itself: |y1 - y2| / std(y) ~ rms(d) / rms(act) ~ 0.01, which is the mean bound below (0.02; measured 0.010).
+    # Over the 2 M outputs the largest of these roughly Gaussian differences is about five times their spread (0.05), and
+    # each form rounds its output once more (2^-8 of values up to four spreads: 0.016 each): 0.08 - 0.09 expected
+    # (measured 0.087), 0.15 allowed.
     assert np.abs(composed - fused).max() <= 0.15 * spread, (np.abs(composed - fused).max(), spread)
     assert np.abs(composed - fused).mean() <= 0.02 * spread, (np.abs(composed - fused).mean(), spread)
     separate = {}

@@ -114,6 +114,18 @@ def test_unary_functions(device, dtype, view):
             support.assert_close(got.numpy(), want.numpy(), *tolerance_of(dtype), f"{op} {dtype} {view}")
 
 
+def test_rsqrt_of_bfloat16_subnormals_without_epsilon(device):
+    """A bfloat16 subnormal is a float subnormal, which the hardware's reciprocal square root reads as zero: the device
+    scales such inputs first.  The CPU path evaluates in double (src/cpu/ops-unary.cpp:141-149); one ulp apart at most."""
+    bits = np.array([0x0001, 0x0002, 0x0040, 0x007F, 0x0080, 0x0081, 0x0100, 0x3F80], dtype=np.uint16)
+    h = ta.Tensor(ta.bfloat16, bits.shape).initialize(ta.Host())
+    h.write_raw(bits)
+    d = h.to(device)
+    want, got = ops.rsqrt(h, 0.0).storage().astype(np.int32), ops.rsqrt(d, 0.0).storage().astype(np.int32)
+    assert np.isfinite(ta.types.bfloat16_bits_to_float32(got.astype(np.uint16))).all()
+    assert np.abs(want - got).max() <= 1, (want, got)
+
+
 def test_rsqrt_fp32_is_bit_exact(device):
     """The double-precision evaluation makes the fp32 result correctly rounded on both sides."""
     h, d = pair_of(ta.float32, 8, (100, 333), device, 0.01, 100)
