@@ -457,10 +457,10 @@ def secondary(b, only):
             work.append(conv_entry(b, dtype, "3->64 k7 s2 p3 @224 N=32", (32, 3, 224, 224), (64, 3, 7, 7), 2, 3, 5))
             work.append(conv_entry(b, dtype, "64->64 k3 s1 p1 @56 N=32", (32, 64, 56, 56), (64, 64, 3, 3), 1, 1, 5))
             work.append(conv_entry(b, dtype, "256->512 k1 s2 @56 N=32", (32, 256, 56, 56), (512, 256, 1, 1), 2, 0, 5))
-        # layers outside the benchmark's three, one for each of the more general 16-bit kernels the dispatcher falls back to
+        # layers outside the benchmark's three: 5x5 kernels and the more general 16-bit kernels the dispatcher falls back to
         # (named in the entry; which kernel ran is in the profile of this group)
-        work.append(conv_entry(b, ta.float16, "32->64 k5 s1 p2 @56 N=32 (weights resident in LDS: conv2d_resident)", (32, 32, 56, 56), (64, 32, 5, 5), 1, 2, 5))
-        work.append(conv_entry(b, ta.float16, "128->128 k5 s1 p2 @32 N=32 (general tiles: conv2d_mfma, 128 channels wide)", (32, 128, 32, 32), (128, 128, 5, 5), 1, 2, 5))
+        work.append(conv_entry(b, ta.float16, "32->64 k5 s1 p2 @56 N=32 (the 5x5 instance of the LDS-patch kernel: conv2d_k3)", (32, 32, 56, 56), (64, 32, 5, 5), 1, 2, 5))
+        work.append(conv_entry(b, ta.float16, "128->128 k5 s1 p2 @32 N=32 (the 5x5 instance of the LDS-patch kernel, four chunks)", (32, 128, 32, 32), (128, 128, 5, 5), 1, 2, 5))
         work.append(conv_entry(b, ta.float16, "512->128 k1 s1 @28 N=32 (a product per image: conv2d_pointwise)", (32, 512, 28, 28), (128, 512, 1, 1), 1, 0, 5))
         work.append(conv_entry(b, ta.float16, "24->48 k3 s1 p1 @30 N=32 (general tiles, nothing aligned: conv2d_mfma, 64 channels wide)", (32, 24, 30, 30), (48, 24, 3, 3), 1, 1, 5))
     if only in (None, "elementwise"):

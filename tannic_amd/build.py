@@ -50,7 +50,8 @@ UNITS = [
     ("conv2d_mfma.hip", "conv2d_mfma.o", []),
     ("conv2d_patch.hip", "conv2d_patch.o", []),
     ("conv2d_resident.hip", "conv2d_resident.o", []),
-    ("conv2d_k3.hip", "conv2d_k3.o", []),
+    ("conv2d_k3.hip", "conv2d_k3.o", ["-DTH_K3_PART=0"]),
+    ("conv2d_k3.hip", "conv2d_k5.o", ["-DTH_K3_PART=1"]),
     ("conv2d_k1.hip", "conv2d_k1.o", []),
     ("conv2d_pointwise.hip", "conv2d_pointwise.o", []),
     ("conv2d_stem.hip", "conv2d_stem.o", []),

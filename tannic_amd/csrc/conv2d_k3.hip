@@ -1,4 +1,4 @@
-// conv2d with a 3x3 kernel on MFMA, 16-bit signals — the common ResNet-style layer.
+// conv2d with a 3x3 (or 5x5) kernel on MFMA, 16-bit signals — the common ResNet-style layer.
 //
 // One block of 256 threads computes 64 output channels of R whole output rows
 // of one image (up to 128 * TN pixels).  The input channels are walked in chunks
@@ -10,7 +10,8 @@
 // hold chunk c+1 are written to the other stage and refilled with chunk c+2
 // from global memory, one memory operation between MFMAs.  With ONE_STAGE the
 // block has a single stage (chunk c+1 is written after the MFMAs of chunk c) and
-// half the registers, so that two blocks fit a compute unit and cover each other.
+// half the registers, so that two blocks fit a compute unit and cover each other;
+// a 5x5 kernel's weights (100 KB a chunk) leave room for one stage of one block.
 // Weights are read straight from the OIHW tensor: a thread loads the 8 channels x
 // 9 taps of one output channel (72 consecutive elements) and regroups them in
 // registers into nine 8-channel vectors.  The signal is read as 8 channels x 8
@@ -54,11 +55,9 @@ __device__ inline void k3_static_for(F&& f) {
 }
 
 constexpr int kK3Threads = 256;
-constexpr int kK3Taps = 9;
 constexpr int kK3BCO = 64;     // output channels per block
 constexpr int kK3CH = 32;      // input channels per chunk = elements per LDS record
 constexpr int kK3Passes = 2;   // micro-blocks per thread and chunk (one where two blocks share a compute unit)
-constexpr uint32_t kK3WeightElems = kK3Taps * kK3BCO * kK3CH;
 
 struct K3Plan {
     uint32_t R, IH, IWp, row_blocks, co_tiles;
@@ -74,10 +73,13 @@ __device__ const uint4k k3_zeros = {0, 0, 0, 0};
 
 __device__ inline uint32_t k3_offset(uint32_t rec, uint32_t slot) { return rec * kK3CH + ((slot ^ ((rec >> 2) & 3u)) * 8u); }
 
-template <class T, int TN, bool ONE_STAGE>
-__global__ __launch_bounds__(kK3Threads, ONE_STAGE ? 2 : 1) void conv2d_k3_kernel(const T* x, const T* w, const T* bias, T* y, ConvProblem p, K3Plan q) {
+// KH x KW: the kernel's size; BPC: blocks that share a compute unit (2 only with ONE_STAGE)
+template <class T, int TN, bool ONE_STAGE, int KH, int KW, int BPC>
+__global__ __launch_bounds__(kK3Threads, BPC) void conv2d_k3_kernel(const T* x, const T* w, const T* bias, T* y, ConvProblem p, K3Plan q) {
     constexpr int TM = kK3BCO / 32;
-    constexpr int PASSES = ONE_STAGE ? 1 : kK3Passes;   // micro-blocks per thread and chunk
+    constexpr int kK3Taps = KH * KW;
+    constexpr uint32_t kK3WeightElems = kK3Taps * kK3BCO * kK3CH;
+    constexpr int PASSES = BPC == 2 ? 1 : kK3Passes;   // micro-blocks per thread and chunk
     extern __shared__ __align__(16) unsigned char k3_lds[];
     T* lds = reinterpret_cast<T*>(k3_lds);
 
@@ -128,10 +130,10 @@ __global__ __launch_bounds__(kK3Threads, ONE_STAGE ? 2 : 1) void conv2d_k3_kerne
     auto fetch_p = [&](int ps, int cc, uint32_t chunk) {
         preg[ps][cc] = *reinterpret_cast<const uint4k*>(p_src[ps] + (static_cast<int64_t>(chunk) * kK3CH + cc) * p_cstep[ps]);
     };
-    // tap `tap` of the eight channels: elements cc * 9 + tap of the 72 loaded ones
+    // tap `tap` of the eight channels: elements cc * taps + tap of the 8 * taps loaded ones
     auto commit_w = [&](int tap, T* stage) {
-        uint16_t all[72], out[8];
-        __builtin_memcpy(all, wreg, 144);
+        uint16_t all[8 * kK3Taps], out[8];
+        __builtin_memcpy(all, wreg, 16 * kK3Taps);
 #pragma unroll
         for (int cc = 0; cc < 8; ++cc) out[cc] = all[cc * kK3Taps + tap];
         uint4k v;
@@ -219,7 +221,7 @@ __global__ __launch_bounds__(kK3Threads, ONE_STAGE ? 2 : 1) void conv2d_k3_kerne
     const uint32_t wlane = k3_offset(lane % 32, frag_slot);   // record i * 32 + lane % 32: same swizzle for every i and tap
     uint4k fw[2][2][TM], fx[2][2][TN];   // [buffer][half][...]
     auto read_fragments = [&](const T* stage, int tap, int into) {
-        const uint32_t tap_rec = (tap / 3) * q.IWp + tap % 3;
+        const uint32_t tap_rec = (tap / KW) * q.IWp + tap % KW;
 #pragma unroll
         for (int j = 0; j < TN; ++j) {
             const uint32_t xoff = k3_offset(pbase[j] + tap_rec, frag_slot);
@@ -327,9 +329,9 @@ __global__ __launch_bounds__(kK3Threads, ONE_STAGE ? 2 : 1) void conv2d_k3_kerne
     }
 }
 
-template <class T, int TN, bool ONE_STAGE>
+template <class T, int TN, bool ONE_STAGE, int KH, int KW, int BPC>
 int launch_k3(const ConvProblem& p, const K3Plan& q, size_t lds, uint32_t blocks, const void* x, const void* w, const void* bias, void* y, hipStream_t stream) {
-    auto kernel = conv2d_k3_kernel<T, TN, ONE_STAGE>;
+    auto kernel = conv2d_k3_kernel<T, TN, ONE_STAGE, KH, KW, BPC>;
     static std::atomic<uint64_t> configured{0};
     if (int rc = raise_lds_limit(reinterpret_cast<const void*>(kernel), 160 * 1024, configured)) return rc;
     hipLaunchKernelGGL(kernel, dim3(blocks), dim3(kK3Threads), lds, stream, static_cast<const T*>(x), static_cast<const T*>(w), static_cast<const T*>(bias),
@@ -337,46 +339,54 @@ int launch_k3(const ConvProblem& p, const K3Plan& q, size_t lds, uint32_t blocks
     return launch_status("conv2d_k3_kernel");
 }
 
-template <class T>
+template <class T, int KH, int KW>
 int run_k3(const ConvProblem& p, const void* x, const void* w, const void* bias, void* y, hipStream_t stream) {
-    if (p.KH != 3 || p.KW != 3) return TANNIC_UNSUPPORTED_DTYPE;
+    constexpr uint32_t TAPS = KH * KW, WEIGHT_ELEMS = TAPS * kK3BCO * kK3CH;
+    if (p.KH != KH || p.KW != KW) return TANNIC_UNSUPPORTED_DTYPE;
     if (p.C == 0 || p.C % kK3CH != 0 || p.W % 8 != 0) return TANNIC_UNSUPPORTED_DTYPE;
     // 16-byte loads: signal rows, channels and images start at multiples of 8 elements; the kernel tensor is plain OIHW
     if (p.xs[3] != 1 || p.xs[2] % 8 != 0 || p.xs[1] % 8 != 0 || p.xs[0] % 8 != 0 || reinterpret_cast<uintptr_t>(x) % 16 != 0) return TANNIC_UNSUPPORTED_DTYPE;
-    if (p.ws[3] != 1 || p.ws[2] != 3 || p.ws[1] != 9 || p.ws[0] != static_cast<int64_t>(p.C) * 9 || reinterpret_cast<uintptr_t>(w) % 16 != 0) return TANNIC_UNSUPPORTED_DTYPE;
+    if (p.ws[3] != 1 || p.ws[2] != KW || p.ws[1] != static_cast<int64_t>(TAPS) || p.ws[0] != static_cast<int64_t>(p.C) * TAPS || reinterpret_cast<uintptr_t>(w) % 16 != 0)
+        return TANNIC_UNSUPPORTED_DTYPE;
     if (p.N == 0 || p.O == 0 || p.HO == 0 || p.WO == 0) return TANNIC_SUCCESS;
     K3Plan q{};
     q.IWp = p.W + 2 * p.pad_w;
     const size_t budget = 158 * 1024;
     // the largest number of output rows whose tile fits: pixels, LDS, staging registers
-    int tn = 0;
+    int tn = 0, mode = 0;   // mode 0: two stages; 1: one stage, two blocks per compute unit; 2: one stage, one block
     double best = 0.0;
-    bool one_stage = false;
-    auto consider = [&](uint32_t R, bool single, double weight) {
-        const uint32_t IH = (R - 1) * p.stride_h + 3;
-        const size_t stage = (static_cast<size_t>(kK3WeightElems) + static_cast<size_t>(IH) * q.IWp * kK3CH) * sizeof(T);
+    auto consider = [&](uint32_t R, int m, double weight) {
+        const uint32_t IH = (R - 1) * p.stride_h + KH;
+        const size_t stage = (static_cast<size_t>(WEIGHT_ELEMS) + static_cast<size_t>(IH) * q.IWp * kK3CH) * sizeof(T);
         const uint64_t microblocks = 4ull * (p.W / 8) * IH;
         const int t = R * p.WO > 256 ? 4 : 2;
         const size_t out_bytes = static_cast<size_t>(kK3BCO) * (128 * t + 8) * sizeof(T);
-        if (microblocks > (single ? 1 : kK3Passes) * kK3Threads) return;
-        if (single ? (stage > budget / 2 || out_bytes > budget / 2 || t != 2) : 2 * stage > budget) return;
+        if (microblocks > (m == 1 ? 1 : kK3Passes) * kK3Threads) return;
+        if (m == 0 && 2 * stage > budget) return;
+        if (m == 1 && (stage > budget / 2 || out_bytes > budget / 2 || t != 2)) return;
+        if (m == 2 && (stage > budget || out_bytes > budget)) return;
         const double fill = static_cast<double>(R * p.WO) / (128.0 * t);              // lanes with a pixel
         const double rows = static_cast<double>(p.HO) / (((p.HO + R - 1) / R) * R);    // rows of the last block that exist
         const double halo = static_cast<double>(R * p.stride_h) / IH;                  // input rows read once
         const double score = weight * fill * rows * (0.5 + 0.5 * halo);
-        if (score >= best) { best = score; q.R = R; q.IH = IH; tn = t; one_stage = single; }
+        if (score >= best) { best = score; q.R = R; q.IH = IH; tn = t; mode = m; }
     };
-    for (uint32_t R = 1; R <= p.HO && R * p.WO <= 512; ++R) consider(R, false, 1.0);
+    constexpr bool SMALL = TAPS <= 9;   // a larger kernel's chunk of weights leaves room for one stage of one block only
+    if (SMALL)
+        for (uint32_t R = 1; R <= p.HO && R * p.WO <= 512; ++R) consider(R, 0, 1.0);
     // Few chunks: one stage per block and tiles of at most 256 pixels, so that two blocks share a compute unit and
     // one block's loads, LDS writes and result rows run under the other's MFMAs.  With more than four chunks the
     // LDS writes between the chunks, which a single stage cannot hide inside a block, cost more than that gains.
-    if (p.C <= 4 * kK3CH)
-        for (uint32_t R = 1; R <= p.HO && R * p.WO <= 256; ++R) consider(R, true, 1.25);
+    if (SMALL && p.C <= 4 * kK3CH)
+        for (uint32_t R = 1; R <= p.HO && R * p.WO <= 256; ++R) consider(R, 1, 1.25);
+    // 5x5: one stage, the whole LDS, tiles of at most 256 pixels (what the registers hold next to 25 taps of weights).
+    if (!SMALL)
+        for (uint32_t R = 1; R <= p.HO && R * p.WO <= 256; ++R) consider(R, 2, 1.0);
     if (best == 0.0) return TANNIC_UNSUPPORTED_DTYPE;
     q.row_blocks = (p.HO + q.R - 1) / q.R;
     q.co_tiles = (p.O + kK3BCO - 1) / kK3BCO;
     q.patch_records = q.IH * q.IWp;
-    q.stage_elems = kK3WeightElems + q.patch_records * kK3CH;
+    q.stage_elems = WEIGHT_ELEMS + q.patch_records * kK3CH;
     q.microblocks = 4 * (p.W / 8) * q.IH;
     q.div_colblocks = FastDiv(p.W / 8);
     q.div_wo = FastDiv(p.WO);
@@ -389,17 +399,38 @@ int run_k3(const ConvProblem& p, const void* x, const void* w, const void* bias,
     if (blocks >= (1ull << 31)) return TANNIC_UNSUPPORTED_DTYPE;
     const size_t stage_bytes = static_cast<size_t>(q.stage_elems) * sizeof(T);
     const size_t out_bytes = static_cast<size_t>(kK3BCO) * (128 * tn + 8) * sizeof(T);
-    const size_t held = (one_stage ? 1 : 2) * stage_bytes;
+    const size_t held = (mode == 0 ? 2 : 1) * stage_bytes;
     const size_t lds = held > out_bytes ? held : out_bytes;
-    if (one_stage) return launch_k3<T, 2, true>(p, q, lds, static_cast<uint32_t>(blocks), x, w, bias, y, stream);
-    if (tn == 4) return launch_k3<T, 4, false>(p, q, lds, static_cast<uint32_t>(blocks), x, w, bias, y, stream);
-    return launch_k3<T, 2, false>(p, q, lds, static_cast<uint32_t>(blocks), x, w, bias, y, stream);
+    const uint32_t nb = static_cast<uint32_t>(blocks);
+    if constexpr (SMALL) {
+        if (mode == 1) return launch_k3<T, 2, true, KH, KW, 2>(p, q, lds, nb, x, w, bias, y, stream);
+        if (tn == 4) return launch_k3<T, 4, false, KH, KW, 1>(p, q, lds, nb, x, w, bias, y, stream);
+        return launch_k3<T, 2, false, KH, KW, 1>(p, q, lds, nb, x, w, bias, y, stream);
+    } else {
+        return launch_k3<T, 2, true, KH, KW, 1>(p, q, lds, nb, x, w, bias, y, stream);
+    }
 }
 
-int conv2d_k3(const ConvProblem& p, int dtype, const void* x, const void* w, const void* bias, void* y, hipStream_t stream) {
-    if (dtype == TANNIC_FLOAT16) return run_k3<f16>(p, x, w, bias, y, stream);
-    if (dtype == TANNIC_BFLOAT16) return run_k3<bf16>(p, x, w, bias, y, stream);
+// This file is compiled in two parts (TH_K3_PART): 0 holds the 3x3 kernels and the entry point, 1 the 5x5 kernels.
+#ifndef TH_K3_PART
+#define TH_K3_PART 0
+#endif
+
+int conv2d_k5(const ConvProblem& p, int dtype, const void* x, const void* w, const void* bias, void* y, hipStream_t stream);
+
+#if TH_K3_PART == 1
+int conv2d_k5(const ConvProblem& p, int dtype, const void* x, const void* w, const void* bias, void* y, hipStream_t stream) {
+    if (dtype == TANNIC_FLOAT16) return run_k3<f16, 5, 5>(p, x, w, bias, y, stream);
+    if (dtype == TANNIC_BFLOAT16) return run_k3<bf16, 5, 5>(p, x, w, bias, y, stream);
     return TANNIC_UNSUPPORTED_DTYPE;
 }
+#else
+int conv2d_k3(const ConvProblem& p, int dtype, const void* x, const void* w, const void* bias, void* y, hipStream_t stream) {
+    if (p.KH == 5 && p.KW == 5) return conv2d_k5(p, dtype, x, w, bias, y, stream);
+    if (dtype == TANNIC_FLOAT16) return run_k3<f16, 3, 3>(p, x, w, bias, y, stream);
+    if (dtype == TANNIC_BFLOAT16) return run_k3<bf16, 3, 3>(p, x, w, bias, y, stream);
+    return TANNIC_UNSUPPORTED_DTYPE;
+}
+#endif
 
 }  // namespace th

@@ -49,6 +49,12 @@ CASES = {
     "k3_two_stages_160ch": ((1, 160, 12, 16), (64, 160, 3, 3), (1, 1), (1, 1)),
     "k3_two_stages_256ch_s2": ((2, 256, 16, 16), (40, 256, 3, 3), (2, 2), (1, 1)),
     "k3_one_stage_ragged_rows": ((2, 64, 19, 56), (64, 64, 3, 3), (1, 1), (1, 1)),
+    # 5x5 kernels over 32-channel chunks (one LDS stage, one block per compute unit): padding 2, stride 2, no padding with a
+    # ragged last row block, more output channels than a block holds
+    "k5_s1_p2": ((2, 32, 12, 16), (64, 32, 5, 5), (1, 1), (2, 2)),
+    "k5_s2_p2_96ch": ((1, 96, 17, 24), (40, 96, 5, 5), (2, 2), (2, 2)),
+    "k5_p0_two_co_tiles": ((1, 64, 11, 32), (130, 64, 5, 5), (1, 1), (0, 0)),
+    "k5_rect_stride_pad": ((2, 32, 13, 16), (16, 32, 5, 5), (2, 1), (1, 3)),
     # 1x1 kernels with the weights resident in registers: 64..256 channels in, multiples of 256 out, stride 1 and 2,
     # pixel counts that end inside a 64-pixel tile, several images per worker
     "k1_s2_256ch": ((2, 256, 24, 24), (256, 256, 1, 1), (2, 2), (0, 0)),
