@@ -35,7 +35,7 @@ struct Plan {
 };
 
 // Collapses `rank` dims.  strides[o][d] are element strides of operand o.
-// Returns false when the index space does not fit 31 bits.
+// Returns false when the index space cannot be addressed (see below); the launch checks the vector count.
 inline bool build_plan(Plan& p, int rank, const size_t* extent, const int64_t (*strides)[TANNIC_DIMENSIONS], int operands) {
     size_t ext[TANNIC_DIMENSIONS];
     int64_t st[kMaxOperands][TANNIC_DIMENSIONS];
@@ -63,11 +63,32 @@ inline bool build_plan(Plan& p, int rank, const size_t* extent, const int64_t (*
         for (int o = 0; o < operands; ++o) st[o][0] = 1;
         r = 1;
     }
+    // A thread's index counts 16-byte vectors and stays below 2^31 (what the multiply-shift division takes); the element
+    // count may go beyond that.  A dim of 2^31 elements or more (a large contiguous tensor collapses to one) is cut in
+    // two at a power of two, so that every extent fits; what cannot be cut that way is refused.
+    for (int d = 0; d < r; ++d) {
+        if (ext[d] < (1ull << 31)) continue;
+        if (r == TANNIC_DIMENSIONS) return false;
+        size_t inner = size_t(1) << 20;
+        while (inner > 1 && ext[d] % inner != 0) inner >>= 1;
+        if (ext[d] / inner >= (1ull << 31)) return false;
+        for (int e = r; e > d + 1; --e) {
+            ext[e] = ext[e - 1];
+            for (int o = 0; o < operands; ++o) st[o][e] = st[o][e - 1];
+        }
+        ext[d + 1] = inner;
+        ext[d] /= inner;
+        for (int o = 0; o < operands; ++o) {
+            st[o][d + 1] = st[o][d];
+            st[o][d] = st[o][d] * static_cast<int64_t>(inner);
+        }
+        ++r;
+        ++d;
+    }
     size_t total = 1;
     for (int d = 0; d < r; ++d) {
-        if (ext[d] >= (1ull << 31)) return false;
         total *= ext[d];
-        if (total >= (1ull << 31)) return false;
+        if (total >= (1ull << 36)) return false;
     }
     p.rank = r;
     for (int d = 0; d < TANNIC_DIMENSIONS; ++d) {
@@ -244,14 +265,18 @@ int launch_elementwise(F f, Plan p, hipStream_t stream) {
                                               : max_size<S0, D>();
     constexpr int VEC = widest >= 16 ? 1 : static_cast<int>(16 / widest);
     const int last = p.rank - 1;
-    uint32_t rows = 1;
+    uint64_t rows = 1;
     for (int d = 0; d < last; ++d) rows *= p.extent[d];
     bool vec = VEC > 1 && p.extent[last] % VEC == 0 && vector_ok(p, 0, f.a, VEC, false) &&
                vector_ok(p, 2, f.out, VEC, true);
     if (F::sources == 2) vec = vec && vector_ok(p, 1, f.b, VEC, false);
     p.row_vectors = vec ? p.extent[last] / VEC : p.extent[last];
     p.row_div = FastDiv(p.row_vectors);
-    p.total_vectors = rows * p.row_vectors;
+    if (rows * p.row_vectors >= (1ull << 31)) {
+        set_error_text("elementwise: more than 2^31 vectors (16 bytes each where the operands allow, single elements otherwise)");
+        return TANNIC_ERROR;
+    }
+    p.total_vectors = static_cast<uint32_t>(rows * p.row_vectors);
     if (p.total_vectors == 0) return TANNIC_SUCCESS;
     const bool repeats = p.rank > 1 || p.stride[0][last] == 0 || (F::sources == 2 && p.stride[1][last] == 0);
     // Two vectors per thread pay only when the blocks are many generations deep (1 GiB with a broadcast operand: 6 %

@@ -256,7 +256,7 @@ int run_compare(const tannic_tensor_t* a, const tannic_tensor_t* b, tannic_tenso
     contiguous_strides(rank, dst->shape.sizes, strides[2]);
     Plan plan;
     size_t one = 1;
-    if (!build_plan(plan, rank == 0 ? 1 : rank, rank == 0 ? &one : dst->shape.sizes, strides, 3)) {
+    if (dst->size >= (1ull << 31) || !build_plan(plan, rank == 0 ? 1 : rank, rank == 0 ? &one : dst->shape.sizes, strides, 3)) {
         set_error_text("compare: tensors of 2^31 elements or more are not supported");
         return TANNIC_ERROR;
     }
@@ -337,7 +337,7 @@ int run_allclose(const tannic_tensor_t* a, const tannic_tensor_t* b, hipStream_t
     }
     Plan plan;
     size_t one = 1;
-    if (!build_plan(plan, rank == 0 ? 1 : rank, rank == 0 ? &one : a->shape.sizes, strides, 3)) {
+    if (a->size >= (1ull << 31) || !build_plan(plan, rank == 0 ? 1 : rank, rank == 0 ? &one : a->shape.sizes, strides, 3)) {
         set_error_text("allclose: tensors of 2^31 elements or more are not supported");
         return -1;
     }

@@ -225,3 +225,33 @@ def test_byte_offsets_beyond_4_gib(device):
     assert (ops.argmax(cube, 1).numpy() == blocks.argmax(axis=1)).all()
     turned = ops.repack(cube.transpose(0, 2)).numpy()
     assert (turned[:, :, -3:] == blocks.transpose(2, 1, 0)[:, :, -3:]).all() and (turned[::7, ::11] == blocks.transpose(2, 1, 0)[::7, ::11]).all()
+
+
+def test_more_than_two_to_the_31_elements(device):
+    """An int8 tensor of 2^31 + 2^21 elements (the reference indexes with size_t throughout, src/cpu/ops-binary.cpp:48-61):
+    the elementwise engine counts 16-byte vectors, not elements, so add, a broadcast multiply, neg and a copy of a
+    transposed view take it; reductions index their source with 64-bit offsets and take it too.  Bit-exact."""
+    rows, width = 2048 + 2, 1 << 20
+    n = rows * width
+    assert n > 1 << 31
+    block = ((np.arange(1 << 22, dtype=np.int64) * 37 + 11) % 251 - 125).astype(np.int8)
+    x = np.resize(block, n)
+    dx = ta.tensor(x, ta.int8, device)
+    got = ops.add(dx, dx).numpy()
+    want = (x.astype(np.int16) * 2).astype(np.int8)
+    assert (got[-3_000_000:] == want[-3_000_000:]).all() and (got[:: 4099] == want[:: 4099]).all() and (got[1 << 31: (1 << 31) + 4096] == want[1 << 31: (1 << 31) + 4096]).all()
+    del got, want
+    got = ops.neg(dx).numpy()
+    assert (got[-3_000_000:] == -x[-3_000_000:]).all() and (got[:: 4099] == -x[:: 4099]).all()
+    del got
+    grid = dx.view(rows, 1024, 1024)
+    three = ta.tensor(np.full((1, 1024, 1), 3), ta.int8, device)
+    got = ops.mul(grid, three).numpy().reshape(-1)
+    want = (x.astype(np.int16) * 3).astype(np.int8)
+    assert (got[-3_000_000:] == want[-3_000_000:]).all() and (got[:: 4099] == want[:: 4099]).all()
+    del got, want
+    blocks = x.reshape(rows, 1024, 1024)
+    got = ops.sum(grid, 2).numpy()
+    np.testing.assert_array_equal(got, blocks.sum(axis=2, dtype=np.int64).astype(np.int8))
+    got = ops.argmax(grid, 0).numpy()
+    np.testing.assert_array_equal(got, blocks.argmax(axis=0))
