@@ -28,6 +28,7 @@
 #include "reductions.hpp"
 #include "transformations.hpp"
 #include "tannic_hip_functions.hpp"   // the operators this backend adds to the front end's surface
+#include "tannic_hip_serialization.hpp"   // tensors in the reference's file layout, host or device
 
 #include <cmath>
 
@@ -77,7 +78,7 @@ static Tensor computed(Shape shape, F&& f) {
 }
 static const float* values(Tensor const& host) { return reinterpret_cast<const float*>(host.bytes()); }
 
-int main() {
+int main(int argc, char** argv) {
     if (Devices::count() < 1) {
         std::printf("no device\n");
         return 2;
@@ -285,6 +286,56 @@ int main() {
         failures += same ? 0 : 1;
     }
 
+    // ---- tensors in the reference's file layout (include/tannic/serialization.hpp:26-66), through tannic_hip_serialization.hpp ----
+    {
+        auto check = [&](const char* what, bool ok) {
+            std::printf("%-50s %s\n", what, ok ? "ok" : "FAILED");
+            failures += ok ? 0 : 1;
+        };
+        try {
+            const std::vector<std::byte> image = hip::dumps(X);
+            // Header 15 bytes, Metadata 18 bytes, three extents, the data
+            const unsigned char head[] = {0x45, 0x52, 0x49, 0x43, 0x01, 0xCD, 0xAB};
+            uint64_t announced = 0, data = 0;
+            std::memcpy(&announced, image.data() + 7, 8);
+            std::memcpy(&data, image.data() + 15 + 9, 8);
+            check("file image: sizes and the header's fixed bytes", image.size() == 15 + 18 + 24 + X.nbytes() && std::memcmp(image.data(), head, 7) == 0 &&
+                                                                       announced == image.size() - 15 && data == X.nbytes() &&
+                                                                       static_cast<unsigned char>(image[15]) == 24 && static_cast<unsigned char>(image[15 + 17]) == 3);
+            Tensor back = hip::loads(image);
+            check("file image -> host tensor: the same bytes", back.dtype() == float32 && back.shape() == X.shape() && std::memcmp(back.bytes(), X.bytes(), X.nbytes()) == 0);
+            Tensor on_device = hip::loads(image, Device());
+            check("file image -> device tensor", allclose(on_device, X.to(Device()), 0, 0));
+            const std::vector<std::byte> again = hip::dumps(on_device);
+            check("device tensor -> file image: the same image", again == image);
+            Tensor packed = Tensor(I.to(Device()) > seeded(int32, {4, 9, 5}, 23, -50, 50).to(Device()));   // booleans: bit-packed data
+            Tensor packed_back = hip::loads(hip::dumps(packed));
+            Tensor packed_host = packed.to(Host{});
+            check("boolean tensor round trip (bit-packed)", packed_back.dtype() == boolean && packed_back.shape() == packed.shape() &&
+                                                                std::memcmp(packed_back.bytes(), packed_host.bytes(), (packed.nelements() + 7) / 8) == 0);
+            bool threw = false;
+            try { std::vector<std::byte> cut(image.begin(), image.end() - 5); (void)hip::loads(cut); } catch (std::exception const&) { threw = true; }
+            check("a truncated image is refused", threw);
+            threw = false;
+            try { std::vector<std::byte> bad = image; bad[0] = std::byte{0}; (void)hip::loads(bad); } catch (std::exception const&) { threw = true; }
+            check("an image with another magic is refused", threw);
+            threw = false;
+            try { (void)hip::dumps(Tensor(transpose(X, 0, 2))); } catch (std::exception const&) { threw = true; }
+            check("a transposed view is not written", threw);
+            if (argc > 1) {
+                // files shared with the Python reader and writer of the same layout
+                const std::string dir = argv[1];
+                hip::save(X.to(Device()) * 0.5f, dir + "/from_cpp.tannic");
+                Tensor theirs = hip::load(dir + "/from_python.tannic", Device());
+                Tensor expected = computed({2, 3, 4}, [](size_t i) { return 0.5 * i; });
+                check("a file written by the Python writer, loaded onto the device", theirs.dtype() == float32 && theirs.shape() == expected.shape() && allclose(theirs, expected.to(Device()), 0, 0));
+            }
+        } catch (std::exception const& ex) {
+            std::printf("%-50s FAILED exception: %s\n", "tensor files", ex.what());
+            failures += 1;
+        }
+    }
+
     for (auto& c : cases) {
         bool ok = false;
         std::string note;
@@ -304,6 +355,6 @@ int main() {
         std::fflush(stdout);
         failures += ok ? 0 : 1;
     }
-    std::printf("%d of %zu cases failed\n", failures, cases.size() + added.size() + 21);
+    std::printf("%d of %zu cases failed\n", failures, cases.size() + added.size() + 21 + 8 + (argc > 1 ? 1 : 0));
     return failures ? 1 : 0;
 }
