@@ -103,9 +103,10 @@ struct ArgOp {
     // rule; the lower-index tie-break only matters when partial results meet (combine)
     __device__ static inline A step(A acc, T v, uint32_t r) {
         const bool strictly = MAX ? gt(v, acc.value) : gt(acc.value, v);
-        acc.value = strictly ? v : acc.value;
-        acc.index = strictly ? r : acc.index;
-        return acc;
+        A out;   // the padding of a 16-bit value is left unset: carrying it along costs three instructions per element
+        out.value = strictly ? v : acc.value;
+        out.index = strictly ? r : acc.index;
+        return out;
     }
     __device__ static inline A combine(A x, A y) { return better(y.value, y.index, x) ? y : x; }
     __device__ static inline int64_t finish(A acc, uint32_t) { return static_cast<int64_t>(acc.index); }
@@ -140,6 +141,10 @@ struct ValueOp {
     __device__ static inline A step(A acc, T v, uint32_t) { return extreme<T, MAX>(acc, v); }
     __device__ static inline A combine(A x, A y) { return extreme<T, MAX>(x, y); }
 };
+
+// an index search over 16-bit elements: eight compare-and-select pairs per 16-byte load
+template <class Op> struct folds_slowly { static constexpr bool value = false; };
+template <class T, bool MAX, bool VALUE> struct folds_slowly<ArgOp<T, MAX, VALUE>> { static constexpr bool value = sizeof(T) == 2; };
 
 template <class Op, class = void> struct is_value_only { static constexpr bool value = false; };
 template <class Op> struct is_value_only<Op, std::enable_if_t<Op::value_only>> { static constexpr bool value = true; };
@@ -331,14 +336,48 @@ __global__ __launch_bounds__(kThreads) void reduce_columns_kernel(const typename
         const T* p = src + static_cast<size_t>(outer) * R * inner + col;
         const uint32_t stride = TY * gridDim.z;
         uint32_t r = blockIdx.z * TY + ty;
-        for (; r + 3 * stride < R; r += 4 * stride) {
-            Vec<T, VEC> x[4];
+        if constexpr (folds_slowly<Op>::value) {
+            // Groups of rows, two groups in turn: the loads of the next group are on their way while the current
+            // one is folded, so a lane keeps requests outstanding through the arithmetic (an index search over 16-bit
+            // elements spends some hundred instructions per group, and only two waves share a SIMD at two blocks per
+            // compute unit).  Folds of a few instructions per load stream better without it.
+            constexpr int G = 4;   // rows per group; two-row groups (as many loads outstanding as the plain loop) stream a tenth slower
+            const size_t hop = static_cast<size_t>(stride) * inner;
+            const T* q = p + static_cast<size_t>(r) * inner;
+            auto fetch = [&](Vec<T, VEC> (&x)[G]) {
 #pragma unroll
-            for (int k = 0; k < 4; ++k) x[k] = load_vec<T, VEC>(p + static_cast<size_t>(r + k * stride) * inner);
+                for (int k = 0; k < G; ++k) x[k] = load_vec<T, VEC>(q + k * hop);
+                q += G * hop;
+            };
+            auto fold = [&](const Vec<T, VEC> (&x)[G]) {
 #pragma unroll
-            for (int k = 0; k < 4; ++k)
+                for (int k = 0; k < G; ++k)
 #pragma unroll
-                for (int i = 0; i < VEC; ++i) acc[i] = Op::step(acc[i], x[k].v[i], r + k * stride);
+                    for (int i = 0; i < VEC; ++i) acc[i] = Op::step(acc[i], x[k].v[i], r + k * stride);
+                r += G * stride;
+            };
+            if (r + (G - 1) * stride < R) {
+                Vec<T, VEC> even[G], odd[G];
+                fetch(even);
+                for (;;) {
+                    if (!(r + (2 * G - 1) * stride < R)) { fold(even); break; }
+                    fetch(odd);
+                    fold(even);
+                    if (!(r + (2 * G - 1) * stride < R)) { fold(odd); break; }
+                    fetch(even);
+                    fold(odd);
+                }
+            }
+        } else {
+            for (; r + 3 * stride < R; r += 4 * stride) {
+                Vec<T, VEC> x[4];
+#pragma unroll
+                for (int k = 0; k < 4; ++k) x[k] = load_vec<T, VEC>(p + static_cast<size_t>(r + k * stride) * inner);
+#pragma unroll
+                for (int k = 0; k < 4; ++k)
+#pragma unroll
+                    for (int i = 0; i < VEC; ++i) acc[i] = Op::step(acc[i], x[k].v[i], r + k * stride);
+            }
         }
         for (; r < R; r += stride) {
             const Vec<T, VEC> x = load_vec<T, VEC>(p + static_cast<size_t>(r) * inner);
