@@ -157,11 +157,11 @@ def test_operand_with_fewer_batch_dims_steps_by_its_own_batch_stride(device):
 
 
 @pytest.mark.parametrize("shape", [(1024, 2048, 512), (2048, 4096, 256), (512, 4096, 1024), (512, 4096, 4096), (256, 2048, 8192), (4096, 4096, 128), (2304, 8192, 192), (2, 2048, 6144, 64), (25, 512, 1024, 64),
-                                   (264, 392, 2048), (2, 136, 784, 2048), (520, 4104, 4096)], ids=str)
+                                   (264, 392, 2048), (2, 136, 784, 2048), (520, 4104, 4096), (512, 2048, 16384)], ids=str)
 @pytest.mark.parametrize("dtype", [ta.float16, ta.bfloat16], ids=str)
 def test_operands_contiguous_along_m_or_n_on_direct_tiles(device, dtype, shape):
     """X . W, X^T . W and X^T . W^T with whole tiles along M and N (the last three shapes: with a last tile that reaches
-    past M and N, long K), at sizes that choose each tile of the direct-to-LDS
+    past M and N, long K; the last: a long K shared between many workgroups), at sizes that choose each tile of the direct-to-LDS
     kernel (128 x 128, 256 x 128, K shared between two and more workgroups, 256 x 256, more 256 x 256 tiles than compute units
     so that a workgroup walks several, batches): operand tiles kept as k-rows and
     read with the transposing LDS read.  Sums run over k in the same order as for X . W^T, so the four layouts agree

@@ -73,7 +73,7 @@ def test_products_without_shared_k_need_no_scratch(device):
 
 
 def test_a_product_whose_partial_sums_do_not_fit_is_refused(device):
-    """[128,16384] x [16384,8192]: 64 tiles of 128 x 128, K shared four ways: 4 x 128 x 8192 fp32 partial sums = 16 MiB."""
+    """[128,16384] x [16384,8192]: 64 tiles of 128 x 128 with K shared at least four ways: 4 x 128 x 8192 fp32 partial sums are 16 MiB already."""
     dx = ta.Tensor(ta.float16, (128, 16384)).initialize(device)
     dw = ta.Tensor(ta.float16, (8192, 16384)).initialize(device).transpose()
     status, message, _, _ = product("gemm_noalloc", device, dx, dw, (128, 8192), ta.float16)
