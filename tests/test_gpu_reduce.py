@@ -95,6 +95,21 @@ def test_argmax_argmin_max_min_bit_exact(device, dtype, name):
         support.assert_bit_exact(got.storage(), want.storage(), f"{op} {name} {dtype}")
 
 
+@pytest.mark.parametrize("extent", [3, 4, 15, 16, 17, 31, 32, 33, 47, 48, 49, 64, 65])
+@pytest.mark.parametrize("dtype", [ta.float16, ta.bfloat16], ids=str)
+def test_index_search_over_16bit_columns_at_the_group_boundaries(device, dtype, extent):
+    """[3, extent, 512]: 64 lanes across the columns, four rows of lanes, no sharing of R, so a lane walks rows
+    ty, ty + 4, ...: extents around 16, 32, 48 and 64 are one to four whole groups of four rows (the loop that folds a
+    group while the next is loading takes them in turn from two register sets), with and without rows left over."""
+    x = np.round(support.values_for(dtype, SEED, 11, (3, extent, 512), -4, 4).astype(np.float64))
+    x[1, extent // 2, 7] = np.nan
+    x[2, :, 9] = -np.inf
+    h, d = support.both(x, dtype, device)
+    for op in ("argmax", "argmin", "max", "min"):
+        want, got = getattr(ops, op)(h, 1), getattr(ops, op)(d, 1)
+        support.assert_bit_exact(got.storage(), want.storage(), f"{op} extent {extent} {dtype}")
+
+
 def test_argmax_with_nan_and_infinities(device):
     x = support.uniform(SEED, 5, (64, 700))
     x[0, :] = np.nan
