@@ -156,6 +156,13 @@ __global__ __launch_bounds__(kK3Threads, BPC) void conv2d_k3_kernel(const T* x, 
     };
 
     // ---- prologue: chunk 0 into stage 0, chunk 1 into registers ------------------------------------
+    // (the bias goes first: loads return in order, and the accumulators are seeded while the tiles are on their way)
+    float bias_v[TM];
+#pragma unroll
+    for (int i = 0; i < TM; ++i) {
+        const uint32_t co = co0 + i * 32 + lane % 32;
+        bias_v[i] = (p.has_bias && co < p.O) ? static_cast<float>(widen(bias[static_cast<int64_t>(co) * p.bs])) : 0.0f;
+    }
 #pragma unroll
     for (int k = 0; k < kK3Taps; ++k) fetch_w(k, 0);
 #pragma unroll
@@ -185,12 +192,14 @@ __global__ __launch_bounds__(kK3Threads, BPC) void conv2d_k3_kernel(const T* x, 
         if (qp < npix_tile) q.div_wo.divmod(qp, r, ow);
         pbase[j] = r * p.stride_h * q.IWp + ow * p.stride_w;
     }
-    float bias_v[TM];
+    float16k acc[TM][TN];
 #pragma unroll
-    for (int i = 0; i < TM; ++i) {
-        const uint32_t co = co0 + i * 32 + lane % 32;
-        bias_v[i] = (p.has_bias && co < p.O) ? static_cast<float>(widen(bias[static_cast<int64_t>(co) * p.bs])) : 0.0f;
-    }
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[i][j][v] = bias_v[i];
+    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int k = 0; k < kK3Taps; ++k) commit_w(k, lds);
 #pragma unroll
@@ -205,13 +214,6 @@ __global__ __launch_bounds__(kK3Threads, BPC) void conv2d_k3_kernel(const T* x, 
 #pragma unroll
             for (int cc = 0; cc < 8; ++cc) fetch_p(ps, cc, 1);
     }
-    float16k acc[TM][TN];
-#pragma unroll
-    for (int i = 0; i < TM; ++i)
-#pragma unroll
-        for (int j = 0; j < TN; ++j)
-#pragma unroll
-            for (int v = 0; v < 16; ++v) acc[i][j][v] = bias_v[i];
     __syncthreads();
 
     // ---- chunks ------------------------------------------------------------------------------------
