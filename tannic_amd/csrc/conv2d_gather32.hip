@@ -33,9 +33,19 @@ struct Tap32 {
     uint16_t kh, kw;
 };
 
+template <int N, class F, int I = 0>
+__device__ inline void g32_static_for(F&& f) {
+    if constexpr (I < N) {
+        f(std::integral_constant<int, I>{});
+        g32_static_for<N, F, I + 1>(static_cast<F&&>(f));
+    }
+}
+
 __device__ inline uint32_t g32_offset(uint32_t row, uint32_t chunk) { return row * kG32BK + ((chunk ^ ((row >> 2) & 3u)) * 4u); }
 
-template <int BCO, bool W_VECTOR>
+// MAPW: 32-bit words of the per-pixel map "tap (kh, kw) lies inside the image" (KH * KW <= 31: one, <= 63: two; the last
+// bit stays clear and stands for "no such k").  0: larger kernels, every tap is range-tested as it is gathered.
+template <int BCO, bool W_VECTOR, int MAPW>
 __global__ __launch_bounds__(kG32Threads) void conv2d_gather32_kernel(const float* x, const float* w, const float* bias, float* y, ConvProblem p,
                                                                        uint32_t K, uint32_t pixels, uint32_t co_tiles) {
     constexpr int BP = kG32BP, BK = kG32BK;
@@ -54,11 +64,11 @@ __global__ __launch_bounds__(kG32Threads) void conv2d_gather32_kernel(const floa
         if (k < K) {
             const uint32_t ci = k / khw, r = k % khw, kh = r / p.KW, kw = r % p.KW;
             t.offset = static_cast<int32_t>(ci * p.xs[1] + kh * p.xs[2] + kw * p.xs[3]);
-            t.kh = static_cast<uint16_t>(kh);
+            t.kh = static_cast<uint16_t>(MAPW ? r : kh);     // with a map: the tap's bit
             t.kw = static_cast<uint16_t>(kw);
         } else {
             t.offset = 0;
-            t.kh = 0xFFFF;
+            t.kh = MAPW ? 32 * MAPW - 1 : 0xFFFF;
             t.kw = 0;
         }
         taps[k] = t;
@@ -79,6 +89,18 @@ __global__ __launch_bounds__(kG32Threads) void conv2d_gather32_kernel(const floa
     const int32_t base_w = static_cast<int32_t>((prem % p.WO) * p.stride_w) - static_cast<int32_t>(p.pad_w);
     const float* xp = x + static_cast<int64_t>(n_img) * p.xs[0] + static_cast<int64_t>(base_h) * p.xs[2] + static_cast<int64_t>(base_w) * p.xs[3];
     const uint32_t H = pixel_live ? p.H : 0;   // a dead pixel fails every range test
+    // which taps of this pixel's window lie inside the image, and an offset that is always safe to read (the image's
+    // first element) for those that do not
+    uint64_t inside = 0;
+    const int32_t safe = -static_cast<int32_t>(static_cast<int64_t>(base_h) * p.xs[2] + static_cast<int64_t>(base_w) * p.xs[3]);
+    if constexpr (MAPW > 0) {
+        // columns first (one bit per kw), then that pattern once per row of the window that lies inside
+        uint32_t columns = 0;
+        for (uint32_t kw = 0; kw < p.KW; ++kw) columns |= static_cast<uint32_t>(static_cast<uint32_t>(base_w + static_cast<int32_t>(kw)) < p.W) << kw;
+        for (uint32_t kh = 0; kh < p.KH; ++kh)
+            if (static_cast<uint32_t>(base_h + static_cast<int32_t>(kh)) < H) inside |= static_cast<uint64_t>(columns) << (kh * p.KW);
+    }
+    const uint32_t inside_low = static_cast<uint32_t>(inside);
 
     uint32_t w_row[W_CHUNKS], w_chunk[W_CHUNKS];
 #pragma unroll
@@ -88,66 +110,95 @@ __global__ __launch_bounds__(kG32Threads) void conv2d_gather32_kernel(const floa
         w_chunk[i] = id % 4;
     }
 
-    // Values of the coming step.  Whether a value counts is recorded in bit masks and applied only when the registers
-    // are written to LDS, so that nothing waits for the loads before the MFMAs of the current step have been issued.
-    float gx[8];
-    uint32_t gx_live = 0;
-    float gw[W_CHUNKS][4];
-    uint32_t gw_live = 0;   // one bit per weight element: chunk i, element q -> bit 4 i + q
+    // Values on their way, two sets: the set of step s + 1 was asked for during step s - 1 and goes to LDS during step s,
+    // while the other set is asked for step s + 2.  Whether a value counts is recorded in bit masks and applied when the
+    // registers are written to LDS.  All of this is issued BETWEEN the MFMAs of a step (see the loop), so that a
+    // wavefront's address arithmetic, loads and LDS writes run while its own MFMAs occupy the matrix pipe.
+    struct Fetched {
+        float gx[8];
+        uint32_t gx_live;
+        float gw[W_CHUNKS][4];
+        uint32_t gw_live;   // one bit per weight element: chunk i, element q -> bit 4 i + q
+    };
+    Fetched sets[2];
+    Tap32 tap_of[8];       // the eight table entries of the step being asked for
 
-    auto fetch = [&](uint32_t step) {
+    auto read_taps = [&](uint32_t step) {
         const uint32_t kbase = step * BK + kq * 8;
-        gx_live = 0;
-        gw_live = 0;
 #pragma unroll
-        for (int j = 0; j < 8; ++j) {
-            const Tap32 t = taps[kbase + j];
+        for (int j = 0; j < 8; ++j) tap_of[j] = taps[kbase + j];
+    };
+    auto fetch_x = [&](Fetched& f, int j) {
+        const Tap32 t = tap_of[j];
+        if (j == 0) f.gx_live = 0;
+        if constexpr (MAPW > 0) {
+            // all ones when the tap's bit of the map is set; a tap outside reads the image's first element and is zeroed later
+            const uint32_t all = MAPW == 1 ? static_cast<uint32_t>(__builtin_amdgcn_sbfe(static_cast<int32_t>(inside_low), t.kh, 1u))
+                                           : 0u - static_cast<uint32_t>((inside >> t.kh) & 1u);
+            const int32_t offset = static_cast<int32_t>((static_cast<uint32_t>(t.offset) & all) | (static_cast<uint32_t>(safe) & ~all));
+            f.gx[j] = xp[offset];
+            f.gx_live |= all & (1u << j);
+        } else {
             const uint32_t ih = static_cast<uint32_t>(base_h + static_cast<int32_t>(t.kh));
             const uint32_t iw = static_cast<uint32_t>(base_w + static_cast<int32_t>(t.kw));
             const bool ok = t.kh != 0xFFFF && ih < H && iw < p.W;   // unsigned: negative coordinates are huge
             // a tap outside the image reads the tensor's first element (valid memory) and is zeroed later
-            gx[j] = *(ok ? xp + t.offset : x);
-            gx_live |= static_cast<uint32_t>(ok) << j;
+            f.gx[j] = *(ok ? xp + t.offset : x);
+            f.gx_live |= static_cast<uint32_t>(ok) << j;
         }
+    };
+    auto fetch_w = [&](Fetched& f, uint32_t step, int i) {
+        const uint32_t co = co0 + w_row[i];
+        const uint32_t k = step * BK + w_chunk[i] * 4;
+        const uint32_t sco = co < p.O ? co : p.O - 1;
+        const float* src = w + static_cast<int64_t>(sco) * K;
+        if (i == 0) f.gw_live = 0;
+        if constexpr (W_VECTOR) {
+            const float4g v = *reinterpret_cast<const float4g*>(src + (k < K ? k : 0));
+            __builtin_memcpy(f.gw[i], &v, 16);
+            f.gw_live |= (k < K ? 0xFu : 0u) << (4 * i);
+        } else {
 #pragma unroll
-        for (int i = 0; i < W_CHUNKS; ++i) {
-            const uint32_t co = co0 + w_row[i];
-            const uint32_t k = step * BK + w_chunk[i] * 4;
-            const uint32_t sco = co < p.O ? co : p.O - 1;
-            const float* src = w + static_cast<int64_t>(sco) * K;
-            if constexpr (W_VECTOR) {
-                const float4g v = *reinterpret_cast<const float4g*>(src + (k < K ? k : 0));
-                __builtin_memcpy(gw[i], &v, 16);
-                gw_live |= (k < K ? 0xFu : 0u) << (4 * i);
-            } else {
-#pragma unroll
-                for (int q = 0; q < 4; ++q) {
-                    gw[i][q] = src[k + q < K ? k + q : 0];
-                    gw_live |= static_cast<uint32_t>(k + q < K) << (4 * i + q);
-                }
+            for (int q = 0; q < 4; ++q) {
+                f.gw[i][q] = src[k + q < K ? k + q : 0];
+                f.gw_live |= static_cast<uint32_t>(k + q < K) << (4 * i + q);
             }
         }
     };
-    auto commit = [&](uint32_t buf) {
+    auto commit_x = [&](const Fetched& f, uint32_t buf) {
         float* xt = sX + buf * BP * BK;
-        float* wt = sW + buf * BCO * BK;
         float masked[8];
 #pragma unroll
-        for (int j = 0; j < 8; ++j) masked[j] = (gx_live >> j) & 1u ? gx[j] : 0.0f;
+        for (int j = 0; j < 8; ++j) {
+            const uint32_t all = static_cast<uint32_t>(__builtin_amdgcn_sbfe(static_cast<int32_t>(f.gx_live), j, 1u));
+            masked[j] = __builtin_bit_cast(float, __builtin_bit_cast(uint32_t, f.gx[j]) & all);
+        }
         float4g lo, hi;
         __builtin_memcpy(&lo, &masked[0], 16);
         __builtin_memcpy(&hi, &masked[4], 16);
         *reinterpret_cast<float4g*>(xt + g32_offset(pc, kq * 2)) = lo;
         *reinterpret_cast<float4g*>(xt + g32_offset(pc, kq * 2 + 1)) = hi;
+    };
+    auto commit_w = [&](const Fetched& f, uint32_t buf, int i) {
+        float* wt = sW + buf * BCO * BK;
+        float e[4];
 #pragma unroll
-        for (int i = 0; i < W_CHUNKS; ++i) {
-            float e[4];
+        for (int q = 0; q < 4; ++q) e[q] = (f.gw_live >> (4 * i + q)) & 1u ? f.gw[i][q] : 0.0f;
+        float4g v;
+        __builtin_memcpy(&v, e, 16);
+        *reinterpret_cast<float4g*>(wt + g32_offset(w_row[i], w_chunk[i])) = v;
+    };
+    auto fetch_all = [&](Fetched& f, uint32_t step) {
+        read_taps(step);
 #pragma unroll
-            for (int q = 0; q < 4; ++q) e[q] = (gw_live >> (4 * i + q)) & 1u ? gw[i][q] : 0.0f;
-            float4g v;
-            __builtin_memcpy(&v, e, 16);
-            *reinterpret_cast<float4g*>(wt + g32_offset(w_row[i], w_chunk[i])) = v;
-        }
+        for (int j = 0; j < 8; ++j) fetch_x(f, j);
+#pragma unroll
+        for (int i = 0; i < W_CHUNKS; ++i) fetch_w(f, step, i);
+    };
+    auto commit_all = [&](const Fetched& f, uint32_t buf) {
+        commit_x(f, buf);
+#pragma unroll
+        for (int i = 0; i < W_CHUNKS; ++i) commit_w(f, buf, i);
     };
 
     const int wave = threadIdx.x / 64, lane = threadIdx.x % 64;
@@ -168,46 +219,57 @@ __global__ __launch_bounds__(kG32Threads) void conv2d_gather32_kernel(const floa
         }
 
     __syncthreads();   // tap table complete
-    fetch(0);
-    commit(0);
+    const uint32_t last = ksteps - 1;
+    fetch_all(sets[0], 0);
+    commit_all(sets[0], 0);
+    fetch_all(sets[1], last < 1 ? last : 1);
     __syncthreads();
 
-    for (uint32_t step = 0; step < ksteps; ++step) {
-        const uint32_t cur = step & 1;
-        if (step + 1 < ksteps) fetch(step + 1);   // in flight while this step is multiplied
-        const float* wt = sW + cur * BCO * BK;
-        const float* xt = sX + cur * BP * BK;
+    // One step: the MFMAs of LDS buffer PAR.  Between them: the fragments of the second half of the step are read, set
+    // PAR is asked for step + 2 (past the end: the last step once more, never used), and set 1 - PAR (step + 1) goes
+    // to the other buffer.  Every step issues the same operations, so that the waits for the loads count them exactly.
+    constexpr int PER_E = TM * TN, MFMAS = (BK / 8) * 4 * PER_E;
+    auto one_step = [&](auto par_, uint32_t step) {
+        constexpr int PAR = decltype(par_)::value;
+        const float* wt = sW + PAR * BCO * BK;
+        const float* xt = sX + PAR * BP * BK;
+        const uint32_t ask = step + 2 < ksteps ? step + 2 : last;
+        float4g fw[2][TM], fx[2][TN];
+        auto read_fragments = [&](int ks) {
 #pragma unroll
-        for (int ks = 0; ks < BK / 8; ++ks) {
-            float4g fw[TM], fx[TN];
+            for (int i = 0; i < TM; ++i) fw[ks][i] = *reinterpret_cast<const float4g*>(wt + g32_offset(wco + i * 32 + frag_row, ks * 2 + frag_chunk));
 #pragma unroll
-            for (int i = 0; i < TM; ++i) fw[i] = *reinterpret_cast<const float4g*>(wt + g32_offset(wco + i * 32 + frag_row, ks * 2 + frag_chunk));
-#pragma unroll
-            for (int j = 0; j < TN; ++j) fx[j] = *reinterpret_cast<const float4g*>(xt + g32_offset(wp + j * 32 + frag_row, ks * 2 + frag_chunk));
-#pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                float a[TM], b[TN];
-#pragma unroll
-                for (int i = 0; i < TM; ++i) {
-                    float t4[4];
-                    __builtin_memcpy(t4, &fw[i], 16);
-                    a[i] = t4[e];
-                }
-#pragma unroll
-                for (int j = 0; j < TN; ++j) {
-                    float t4[4];
-                    __builtin_memcpy(t4, &fx[j], 16);
-                    b[j] = t4[e];
-                }
-#pragma unroll
-                for (int i = 0; i < TM; ++i)
-#pragma unroll
-                    for (int j = 0; j < TN; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i], b[j], acc[i][j], 0, 0, 0);
-            }
-        }
-        if (step + 1 < ksteps) commit(cur ^ 1);
+            for (int j = 0; j < TN; ++j) fx[ks][j] = *reinterpret_cast<const float4g*>(xt + g32_offset(wp + j * 32 + frag_row, ks * 2 + frag_chunk));
+        };
+        read_fragments(0);
+        read_taps(ask);
+        __builtin_amdgcn_sched_barrier(0);
+        g32_static_for<MFMAS>([&](auto m_) {
+            constexpr int m = decltype(m_)::value;
+            constexpr int ks = m / (4 * PER_E), e = (m / PER_E) % 4, i = (m % PER_E) / TN, j = m % TN;
+            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fw[ks][i][e], fx[ks][j][e], acc[i][j], 0, 0, 0);
+            // the other work of the step, spread over its MFMAs: the loads of step + 2 first, the stores of step + 1
+            // last (their loads went out early in the step before: they have had nearly two steps to arrive)
+            constexpr int PIECES = 1 + 8 + W_CHUNKS + 1 + W_CHUNKS;    // fragments, taps, weights, commit x, commit w..
+            constexpr int first = m * PIECES / MFMAS, end = (m + 1) * PIECES / MFMAS;
+            g32_static_for<end - first>([&](auto o_) {
+                constexpr int o = first + decltype(o_)::value;
+                if constexpr (o == 0) read_fragments(1);
+                else if constexpr (o < 1 + 8) fetch_x(sets[PAR], o - 1);
+                else if constexpr (o < 1 + 8 + W_CHUNKS) fetch_w(sets[PAR], ask, o - 1 - 8);
+                else if constexpr (o == 1 + 8 + W_CHUNKS) commit_x(sets[1 - PAR], 1 - PAR);
+                else commit_w(sets[1 - PAR], 1 - PAR, o - 2 - 8 - W_CHUNKS);
+            });
+            __builtin_amdgcn_sched_barrier(0);
+        });
         __syncthreads();
+    };
+    uint32_t step = 0;
+    for (; step + 1 < ksteps; step += 2) {
+        one_step(std::integral_constant<int, 0>{}, step);
+        one_step(std::integral_constant<int, 1>{}, step + 1);
     }
+    if (step < ksteps) one_step(std::integral_constant<int, 0>{}, step);
 
     // store: the lane's pixel column, rows = output channels
 #pragma unroll
@@ -226,18 +288,26 @@ __global__ __launch_bounds__(kG32Threads) void conv2d_gather32_kernel(const floa
     }
 }
 
-template <int BCO, bool WV>
-int launch_gather32(const ConvProblem& p, uint32_t K, uint32_t pixels, const void* x, const void* w, const void* bias, void* y, hipStream_t stream) {
+template <int BCO, bool WV, int MAPW>
+int launch_gather32_mapped(const ConvProblem& p, uint32_t K, uint32_t pixels, const void* x, const void* w, const void* bias, void* y, hipStream_t stream) {
     const uint32_t ksteps = (K + kG32BK - 1) / kG32BK;
     const size_t lds = sizeof(float) * 2 * (BCO + kG32BP) * kG32BK + sizeof(Tap32) * ksteps * kG32BK;
     const uint32_t co_tiles = (p.O + BCO - 1) / BCO, p_tiles = (pixels + kG32BP - 1) / kG32BP;
-    auto kernel = conv2d_gather32_kernel<BCO, WV>;
+    auto kernel = conv2d_gather32_kernel<BCO, WV, MAPW>;
     static std::atomic<uint64_t> configured{0};
     const size_t most = sizeof(float) * 2 * (BCO + kG32BP) * kG32BK + sizeof(Tap32) * kG32MaxTableK;
     if (int rc = raise_lds_limit(reinterpret_cast<const void*>(kernel), most, configured)) return rc;
     hipLaunchKernelGGL(kernel, dim3(co_tiles * p_tiles), dim3(kG32Threads), lds, stream, static_cast<const float*>(x), static_cast<const float*>(w),
                        static_cast<const float*>(bias), static_cast<float*>(y), p, K, pixels, co_tiles);
     return launch_status("conv2d_gather32_kernel");
+}
+
+template <int BCO, bool WV>
+int launch_gather32(const ConvProblem& p, uint32_t K, uint32_t pixels, const void* x, const void* w, const void* bias, void* y, hipStream_t stream) {
+    const uint64_t taps = static_cast<uint64_t>(p.KH) * p.KW;
+    if (taps <= 31) return launch_gather32_mapped<BCO, WV, 1>(p, K, pixels, x, w, bias, y, stream);
+    if (taps <= 63) return launch_gather32_mapped<BCO, WV, 2>(p, K, pixels, x, w, bias, y, stream);
+    return launch_gather32_mapped<BCO, WV, 0>(p, K, pixels, x, w, bias, y, stream);
 }
 
 int conv2d_gather32(const ConvProblem& p, int dtype, const void* x, const void* w, const void* bias, void* y, hipStream_t stream) {

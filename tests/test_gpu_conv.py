@@ -63,6 +63,13 @@ CASES = {
     "k1_s1_192ch": ((1, 192, 10, 16), (256, 192, 1, 1), (1, 1), (0, 0)),
     "k1_s2_odd_rows": ((1, 64, 15, 24), (256, 64, 1, 1), (2, 2), (0, 0)),
     "k1_s2_many_images": ((40, 64, 8, 8), (256, 64, 1, 1), (2, 2), (0, 0)),
+    # window sizes on both sides of 31 and 63 taps (the fp32 kernel keeps a per-pixel map of the taps inside the image in
+    # one or two words, or tests every tap), and windows that lie wholly in the padding
+    "k1x31_one_word": ((1, 2, 4, 40), (5, 2, 1, 31), (1, 1), (0, 15)),
+    "k4x8_two_words": ((1, 3, 9, 20), (6, 3, 4, 8), (1, 2), (2, 3)),
+    "k7x9_last_bit": ((1, 2, 12, 14), (4, 2, 7, 9), (1, 1), (3, 4)),
+    "k8x8_every_tap_tested": ((1, 2, 12, 12), (4, 2, 8, 8), (2, 1), (4, 3)),
+    "window_in_the_padding": ((1, 2, 5, 5), (3, 2, 2, 2), (1, 1), (3, 3)),
 }
 
 
