@@ -157,6 +157,13 @@ __global__ __launch_bounds__(kG32Threads) void conv2d_gather32_kernel(const floa
             const float4g v = *reinterpret_cast<const float4g*>(src + (k < K ? k : 0));
             __builtin_memcpy(f.gw[i], &v, 16);
             f.gw_live |= (k < K ? 0xFu : 0u) << (4 * i);
+        } else if (k + 4 <= K) {
+            // rows of the weights start at any multiple of four bytes: one load of sixteen bytes all the same, which the
+            // compiler splits where the hardware would not take it
+            typedef float float4u __attribute__((ext_vector_type(4), aligned(4)));
+            const float4u v = *reinterpret_cast<const float4u*>(src + k);
+            __builtin_memcpy(f.gw[i], &v, 16);
+            f.gw_live |= 0xFu << (4 * i);
         } else {
 #pragma unroll
             for (int q = 0; q < 4; ++q) {
