@@ -31,6 +31,7 @@ typedef _Float16 half8k __attribute__((ext_vector_type(8)));
 typedef __bf16 bfloat8k __attribute__((ext_vector_type(8)));
 typedef float float16k __attribute__((ext_vector_type(16)));
 typedef unsigned int uint4k __attribute__((ext_vector_type(4)));
+typedef unsigned int uint4k_any __attribute__((ext_vector_type(4), aligned(2)));   // 16 bytes at any element of a 16-bit tensor
 
 template <class T> __device__ inline float16k k3_mfma(uint4k a, uint4k b, float16k c) {
     if constexpr (std::is_same_v<T, f16>) {
@@ -65,7 +66,7 @@ struct K3Plan {
     uint32_t stage_elems;     // elements of one LDS stage: weights + patch
     uint32_t microblocks;     // 4 * (W / 8) * IH
     uint32_t vector_store;    // rows of the result can be written 16 bytes at a time
-    FastDiv div_colblocks, div_wo, div_row_blocks, div_co_tiles, div_pad;
+    FastDiv div_colblocks, div_wo, div_row_blocks, div_co_tiles, div_pad, div_w, div_w4;   // the last two: W and 4 W (flat staging)
 };
 
 // what a micro-block outside the image reads: its eight loads all come from here
@@ -73,8 +74,13 @@ __device__ const uint4k k3_zeros = {0, 0, 0, 0};
 
 __device__ inline uint32_t k3_offset(uint32_t rec, uint32_t slot) { return rec * kK3CH + ((slot ^ ((rec >> 2) & 3u)) * 8u); }
 
-// KH x KW: the kernel's size; BPC: blocks that share a compute unit (2 only with ONE_STAGE)
-template <class T, int TN, bool ONE_STAGE, int KH, int KW, int BPC>
+// KH x KW: the kernel's size; BPC: blocks that share a compute unit (2 only with ONE_STAGE).
+// FLAT: rows of any width at any alignment.  The rows of the patch that lie inside the image are one contiguous run of a
+// channel plane; it is cut into pieces of eight elements from its first element on (the last piece moved back so that
+// it ends with the run), a micro-block is eight channels of a piece, loaded with 16-byte loads at whatever address that
+// is, and its eight columns go to the records of their (row, column), which may be on two or three rows of the patch.
+// Rows of the patch outside the image are zeroed once.  Without FLAT a micro-block is eight aligned columns of one row.
+template <class T, int TN, bool ONE_STAGE, int KH, int KW, int BPC, bool FLAT>
 __global__ __launch_bounds__(kK3Threads, BPC) void conv2d_k3_kernel(const T* x, const T* w, const T* bias, T* y, ConvProblem p, K3Plan q) {
     constexpr int TM = kK3BCO / 32;
     constexpr int kK3Taps = KH * KW;
@@ -104,22 +110,42 @@ __global__ __launch_bounds__(kK3Threads, BPC) void conv2d_k3_kernel(const T* x, 
     const T* p_src[PASSES];
     int64_t p_cstep[PASSES];
     uint32_t p_dst[PASSES], p_slot[PASSES];
+    uint32_t p_row[PASSES], p_col[PASSES];   // FLAT: patch row and column of the micro-block's first element
     bool p_mine[PASSES];
+    // FLAT: the rows of the patch inside the image, [first_in, end_in) of IH
+    const int32_t ih_first = static_cast<int32_t>(oh0 * p.stride_h) - static_cast<int32_t>(p.pad_h);
+    const uint32_t row_lo = ih_first < 0 ? 0u : static_cast<uint32_t>(ih_first);
+    const uint32_t row_hi = static_cast<uint32_t>(ih_first + static_cast<int32_t>(q.IH)) < p.H ? static_cast<uint32_t>(ih_first + static_cast<int32_t>(q.IH)) : p.H;
+    const uint32_t first_in = row_lo - static_cast<uint32_t>(ih_first), end_in = row_hi - static_cast<uint32_t>(ih_first);
 #pragma unroll
     for (int ps = 0; ps < PASSES; ++ps) {
         const uint32_t mb = threadIdx.x + kK3Threads * ps;
         const uint32_t cb = mb % 4, t1 = mb / 4;
-        uint32_t prow, colb;
-        q.div_colblocks.divmod(t1, prow, colb);
-        const int32_t ih = static_cast<int32_t>(oh0 * p.stride_h + prow) - static_cast<int32_t>(p.pad_h);
-        p_mine[ps] = mb < q.microblocks;
-        const bool live = p_mine[ps] && ih >= 0 && ih < static_cast<int32_t>(p.H);
-        // rows outside the image are zeros in LDS: their micro-blocks load zeros
-        p_src[ps] = live ? x + static_cast<int64_t>(n) * p.xs[0] + static_cast<int64_t>(cb * 8) * p.xs[1] + static_cast<int64_t>(ih) * p.xs[2] + colb * 8
-                         : reinterpret_cast<const T*>(&k3_zeros);
-        p_cstep[ps] = live ? p.xs[1] : 0;
-        p_dst[ps] = prow * q.IWp + p.pad_w + colb * 8;   // first of the eight records
         p_slot[ps] = cb;
+        if constexpr (FLAT) {
+            const uint32_t run = (row_hi - row_lo) * p.W;           // elements; at least 8 (checked by the host)
+            p_mine[ps] = t1 * 8 < run;
+            const uint32_t e0 = !p_mine[ps] ? 0 : t1 * 8 + 8 <= run ? t1 * 8 : run - 8;
+            uint32_t r0, c0;
+            q.div_w.divmod(e0, r0, c0);
+            p_row[ps] = first_in + r0;
+            p_col[ps] = c0;
+            p_dst[ps] = 0;
+            p_src[ps] = x + static_cast<int64_t>(n) * p.xs[0] + static_cast<int64_t>(cb * 8) * p.xs[1] + static_cast<int64_t>(row_lo) * p.xs[2] + e0;
+            p_cstep[ps] = p.xs[1];
+        } else {
+            uint32_t prow, colb;
+            q.div_colblocks.divmod(t1, prow, colb);
+            const int32_t ih = static_cast<int32_t>(oh0 * p.stride_h + prow) - static_cast<int32_t>(p.pad_h);
+            p_mine[ps] = mb < q.microblocks;
+            const bool live = p_mine[ps] && ih >= 0 && ih < static_cast<int32_t>(p.H);
+            // rows outside the image are zeros in LDS: their micro-blocks load zeros
+            p_src[ps] = live ? x + static_cast<int64_t>(n) * p.xs[0] + static_cast<int64_t>(cb * 8) * p.xs[1] + static_cast<int64_t>(ih) * p.xs[2] + colb * 8
+                             : reinterpret_cast<const T*>(&k3_zeros);
+            p_cstep[ps] = live ? p.xs[1] : 0;
+            p_dst[ps] = prow * q.IWp + p.pad_w + colb * 8;   // first of the eight records
+            p_row[ps] = p_col[ps] = 0;
+        }
     }
 
     uint4k wreg[kK3Taps];
@@ -128,7 +154,8 @@ __global__ __launch_bounds__(kK3Threads, BPC) void conv2d_k3_kernel(const T* x, 
         wreg[k] = *reinterpret_cast<const uint4k*>(w_src + static_cast<int64_t>(chunk) * (kK3CH * kK3Taps) + k * 8);
     };
     auto fetch_p = [&](int ps, int cc, uint32_t chunk) {
-        preg[ps][cc] = *reinterpret_cast<const uint4k*>(p_src[ps] + (static_cast<int64_t>(chunk) * kK3CH + cc) * p_cstep[ps]);
+        if constexpr (FLAT) preg[ps][cc] = *reinterpret_cast<const uint4k_any*>(p_src[ps] + (static_cast<int64_t>(chunk) * kK3CH + cc) * p_cstep[ps]);
+        else preg[ps][cc] = *reinterpret_cast<const uint4k*>(p_src[ps] + (static_cast<int64_t>(chunk) * kK3CH + cc) * p_cstep[ps]);
     };
     // tap `tap` of the eight channels: elements cc * taps + tap of the 8 * taps loaded ones
     auto commit_w = [&](int tap, T* stage) {
@@ -152,7 +179,15 @@ __global__ __launch_bounds__(kK3Threads, BPC) void conv2d_k3_kernel(const T* x, 
         }
         uint4k v;
         __builtin_memcpy(&v, out, 16);
-        *reinterpret_cast<uint4k*>(stage + kK3WeightElems + k3_offset(p_dst[ps] + px, p_slot[ps])) = v;
+        uint32_t rec = p_dst[ps] + px;
+        if constexpr (FLAT) {
+            // column px of the piece: up to two rows further down (rows are at least four columns wide)
+            uint32_t row = p_row[ps], col = p_col[ps] + px;
+            if (col >= p.W) { col -= p.W; ++row; }
+            if (col >= p.W) { col -= p.W; ++row; }
+            rec = row * q.IWp + p.pad_w + col;
+        }
+        *reinterpret_cast<uint4k*>(stage + kK3WeightElems + k3_offset(rec, p_slot[ps])) = v;
     };
 
     // ---- prologue: chunk 0 into stage 0, chunk 1 into registers ------------------------------------
@@ -180,6 +215,17 @@ __global__ __launch_bounds__(kK3Threads, BPC) void conv2d_k3_kernel(const T* x, 
             const uint32_t slot = e % 4, side = e / 4;
             const uint32_t col = side < p.pad_w ? side : p.W + side;
             *reinterpret_cast<uint4k*>(lds + st * q.stage_elems + kK3WeightElems + k3_offset(row * q.IWp + col, slot)) = uint4k{0, 0, 0, 0};
+        }
+        if constexpr (FLAT) {
+            // the rows of the patch above and below the image: no micro-block ever writes them
+            const uint32_t outside = q.IH - (end_in - first_in), slots = outside * 4 * p.W;
+            for (uint32_t i = threadIdx.x; i < (ONE_STAGE ? 1 : 2) * slots; i += kK3Threads) {
+                const uint32_t st = i >= slots ? 1 : 0, r = i - st * slots;
+                uint32_t k, e;
+                q.div_w4.divmod(r, k, e);
+                const uint32_t row = k < first_in ? k : end_in + (k - first_in);
+                *reinterpret_cast<uint4k*>(lds + st * q.stage_elems + kK3WeightElems + k3_offset(row * q.IWp + p.pad_w + e / 4, e % 4)) = uint4k{0, 0, 0, 0};
+            }
         }
     }
     // the lane's pixels: group wave + 4 * j, pixel lane % 32 of the group
@@ -314,14 +360,31 @@ __global__ __launch_bounds__(kK3Threads, BPC) void conv2d_k3_kernel(const T* x, 
     const uint32_t rows_here = p.HO - oh0 < q.R ? p.HO - oh0 : q.R;
     const uint32_t npix = rows_here * p.WO;
     T* ybase = y + static_cast<int64_t>(n) * p.ys[0] + static_cast<int64_t>(oh0) * p.ys[2];
-    for (uint32_t c = wave; c < kK3BCO; c += 4) {
-        if (co0 + c >= p.O) break;
-        T* yrow = ybase + static_cast<int64_t>(co0 + c) * p.ys[1];
-        const T* srow = out + c * PITCH;
-        if (q.vector_store) {
-            // rows of the tile follow each other in memory: npix contiguous elements, a multiple of 8
+    // one loop per way of storing, so that each stays a plain loop over the wavefront's sixteen channels
+    if (q.vector_store == 1) {
+        // rows of the tile follow each other in memory: npix contiguous elements, a multiple of 8, 16-byte aligned
+        for (uint32_t c = wave; c < kK3BCO; c += 4) {
+            if (co0 + c >= p.O) break;
+            T* yrow = ybase + static_cast<int64_t>(co0 + c) * p.ys[1];
+            const T* srow = out + c * PITCH;
             for (uint32_t pix = lane * 8; pix < npix; pix += 64 * 8) *reinterpret_cast<uint4k*>(yrow + pix) = *reinterpret_cast<const uint4k*>(srow + pix);
-        } else {
+        }
+    } else if (q.vector_store == 2) {
+        // the same at any alignment and length: whole pieces of eight, then the last few one by one
+        for (uint32_t c = wave; c < kK3BCO; c += 4) {
+            if (co0 + c >= p.O) break;
+            T* yrow = ybase + static_cast<int64_t>(co0 + c) * p.ys[1];
+            const T* srow = out + c * PITCH;
+            for (uint32_t pix = lane * 8; pix < npix; pix += 64 * 8) {
+                if (pix + 8 <= npix) *reinterpret_cast<uint4k_any*>(yrow + pix) = *reinterpret_cast<const uint4k*>(srow + pix);
+                else for (uint32_t e = pix; e < npix; ++e) yrow[e] = srow[e];
+            }
+        }
+    } else {
+        for (uint32_t c = wave; c < kK3BCO; c += 4) {
+            if (co0 + c >= p.O) break;
+            T* yrow = ybase + static_cast<int64_t>(co0 + c) * p.ys[1];
+            const T* srow = out + c * PITCH;
             for (uint32_t pix = lane; pix < npix; pix += 64) {
                 uint32_t r, ow;
                 q.div_wo.divmod(pix, r, ow);
@@ -331,9 +394,9 @@ __global__ __launch_bounds__(kK3Threads, BPC) void conv2d_k3_kernel(const T* x, 
     }
 }
 
-template <class T, int TN, bool ONE_STAGE, int KH, int KW, int BPC>
-int launch_k3(const ConvProblem& p, const K3Plan& q, size_t lds, uint32_t blocks, const void* x, const void* w, const void* bias, void* y, hipStream_t stream) {
-    auto kernel = conv2d_k3_kernel<T, TN, ONE_STAGE, KH, KW, BPC>;
+template <class T, int TN, bool ONE_STAGE, int KH, int KW, int BPC, bool FLAT>
+int launch_k3_as(const ConvProblem& p, const K3Plan& q, size_t lds, uint32_t blocks, const void* x, const void* w, const void* bias, void* y, hipStream_t stream) {
+    auto kernel = conv2d_k3_kernel<T, TN, ONE_STAGE, KH, KW, BPC, FLAT>;
     static std::atomic<uint64_t> configured{0};
     if (int rc = raise_lds_limit(reinterpret_cast<const void*>(kernel), 160 * 1024, configured)) return rc;
     hipLaunchKernelGGL(kernel, dim3(blocks), dim3(kK3Threads), lds, stream, static_cast<const T*>(x), static_cast<const T*>(w), static_cast<const T*>(bias),
@@ -341,13 +404,25 @@ int launch_k3(const ConvProblem& p, const K3Plan& q, size_t lds, uint32_t blocks
     return launch_status("conv2d_k3_kernel");
 }
 
+template <class T, int TN, bool ONE_STAGE, int KH, int KW, int BPC>
+int launch_k3(bool flat, const ConvProblem& p, const K3Plan& q, size_t lds, uint32_t blocks, const void* x, const void* w, const void* bias, void* y, hipStream_t stream) {
+    if (flat) return launch_k3_as<T, TN, ONE_STAGE, KH, KW, BPC, true>(p, q, lds, blocks, x, w, bias, y, stream);
+    return launch_k3_as<T, TN, ONE_STAGE, KH, KW, BPC, false>(p, q, lds, blocks, x, w, bias, y, stream);
+}
+
 template <class T, int KH, int KW>
 int run_k3(const ConvProblem& p, const void* x, const void* w, const void* bias, void* y, hipStream_t stream) {
     constexpr uint32_t TAPS = KH * KW, WEIGHT_ELEMS = TAPS * kK3BCO * kK3CH;
     if (p.KH != KH || p.KW != KW) return TANNIC_UNSUPPORTED_DTYPE;
-    if (p.C == 0 || p.C % kK3CH != 0 || p.W % 8 != 0) return TANNIC_UNSUPPORTED_DTYPE;
-    // 16-byte loads: signal rows, channels and images start at multiples of 8 elements; the kernel tensor is plain OIHW
-    if (p.xs[3] != 1 || p.xs[2] % 8 != 0 || p.xs[1] % 8 != 0 || p.xs[0] % 8 != 0 || reinterpret_cast<uintptr_t>(x) % 16 != 0) return TANNIC_UNSUPPORTED_DTYPE;
+    if (p.C == 0 || p.C % kK3CH != 0 || p.xs[3] != 1) return TANNIC_UNSUPPORTED_DTYPE;
+    // 16-byte loads.  Aligned staging: rows a multiple of 8 wide, rows, channels and images starting at multiples of 8
+    // elements.  Otherwise flat staging: rows that follow each other in memory (a channel plane is one run), at least four
+    // columns, and at least eight elements of the image in every block's patch (its rows inside the image: KH - pad_h or more).
+    const bool aligned = p.W % 8 == 0 && p.xs[2] % 8 == 0 && p.xs[1] % 8 == 0 && p.xs[0] % 8 == 0 && reinterpret_cast<uintptr_t>(x) % 16 == 0;
+    const bool flat = !aligned;
+    if (flat && (p.xs[2] != static_cast<int64_t>(p.W) || p.W < 4 || p.pad_h >= KH || p.H < KH - p.pad_h || static_cast<uint64_t>(KH - p.pad_h) * p.W < 8 ||
+                 reinterpret_cast<uintptr_t>(x) % sizeof(T) != 0))
+        return TANNIC_UNSUPPORTED_DTYPE;
     if (p.ws[3] != 1 || p.ws[2] != KW || p.ws[1] != static_cast<int64_t>(TAPS) || p.ws[0] != static_cast<int64_t>(p.C) * TAPS || reinterpret_cast<uintptr_t>(w) % 16 != 0)
         return TANNIC_UNSUPPORTED_DTYPE;
     if (p.N == 0 || p.O == 0 || p.HO == 0 || p.WO == 0) return TANNIC_SUCCESS;
@@ -360,7 +435,7 @@ int run_k3(const ConvProblem& p, const void* x, const void* w, const void* bias,
     auto consider = [&](uint32_t R, int m, double weight) {
         const uint32_t IH = (R - 1) * p.stride_h + KH;
         const size_t stage = (static_cast<size_t>(WEIGHT_ELEMS) + static_cast<size_t>(IH) * q.IWp * kK3CH) * sizeof(T);
-        const uint64_t microblocks = 4ull * (p.W / 8) * IH;
+        const uint64_t microblocks = flat ? 4ull * ((static_cast<uint64_t>(p.W) * IH + 7) / 8) : 4ull * (p.W / 8) * IH;
         const int t = R * p.WO > 256 ? 4 : 2;
         const size_t out_bytes = static_cast<size_t>(kK3BCO) * (128 * t + 8) * sizeof(T);
         if (microblocks > (m == 1 ? 1 : kK3Passes) * kK3Threads) return;
@@ -395,8 +470,12 @@ int run_k3(const ConvProblem& p, const void* x, const void* w, const void* bias,
     q.div_row_blocks = FastDiv(q.row_blocks);
     q.div_co_tiles = FastDiv(q.co_tiles);
     q.div_pad = FastDiv(p.pad_w ? 8 * p.pad_w : 1);
-    q.vector_store = p.ys[3] == 1 && p.ys[2] == static_cast<int64_t>(p.WO) && p.ys[1] % 8 == 0 && p.ys[0] % 8 == 0 && (q.R * p.WO) % 8 == 0 &&
-                     (static_cast<uint64_t>(p.HO) * p.WO) % 8 == 0 && reinterpret_cast<uintptr_t>(y) % 16 == 0;
+    q.div_w = FastDiv(p.W);
+    q.div_w4 = FastDiv(4 * p.W);
+    const bool rows_follow = p.ys[3] == 1 && p.ys[2] == static_cast<int64_t>(p.WO);
+    q.vector_store = rows_follow && p.ys[1] % 8 == 0 && p.ys[0] % 8 == 0 && (q.R * p.WO) % 8 == 0 && (static_cast<uint64_t>(p.HO) * p.WO) % 8 == 0 &&
+                             reinterpret_cast<uintptr_t>(y) % 16 == 0 ? 1
+                     : rows_follow && reinterpret_cast<uintptr_t>(y) % sizeof(T) == 0 ? 2 : 0;
     const uint64_t blocks = static_cast<uint64_t>(p.N) * q.row_blocks * q.co_tiles;
     if (blocks >= (1ull << 31)) return TANNIC_UNSUPPORTED_DTYPE;
     const size_t stage_bytes = static_cast<size_t>(q.stage_elems) * sizeof(T);
@@ -405,11 +484,11 @@ int run_k3(const ConvProblem& p, const void* x, const void* w, const void* bias,
     const size_t lds = held > out_bytes ? held : out_bytes;
     const uint32_t nb = static_cast<uint32_t>(blocks);
     if constexpr (SMALL) {
-        if (mode == 1) return launch_k3<T, 2, true, KH, KW, 2>(p, q, lds, nb, x, w, bias, y, stream);
-        if (tn == 4) return launch_k3<T, 4, false, KH, KW, 1>(p, q, lds, nb, x, w, bias, y, stream);
-        return launch_k3<T, 2, false, KH, KW, 1>(p, q, lds, nb, x, w, bias, y, stream);
+        if (mode == 1) return launch_k3<T, 2, true, KH, KW, 2>(flat, p, q, lds, nb, x, w, bias, y, stream);
+        if (tn == 4) return launch_k3<T, 4, false, KH, KW, 1>(flat, p, q, lds, nb, x, w, bias, y, stream);
+        return launch_k3<T, 2, false, KH, KW, 1>(flat, p, q, lds, nb, x, w, bias, y, stream);
     } else {
-        return launch_k3<T, 2, true, KH, KW, 1>(p, q, lds, nb, x, w, bias, y, stream);
+        return launch_k3<T, 2, true, KH, KW, 1>(flat, p, q, lds, nb, x, w, bias, y, stream);
     }
 }
 

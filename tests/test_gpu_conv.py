@@ -70,6 +70,19 @@ CASES = {
     "k7x9_last_bit": ((1, 2, 12, 14), (4, 2, 7, 9), (1, 1), (3, 4)),
     "k8x8_every_tap_tested": ((1, 2, 12, 12), (4, 2, 8, 8), (2, 1), (4, 3)),
     "window_in_the_padding": ((1, 2, 5, 5), (3, 2, 2, 2), (1, 1), (3, 3)),
+    # 32-channel chunks with rows that are not a multiple of 8 wide (28, 14, 7 ... as deeper in a ResNet): the patch's
+    # rows are staged as one run of the channel plane, cut into pieces of eight wherever they fall
+    "k3_w28_128ch": ((2, 128, 28, 28), (64, 128, 3, 3), (1, 1), (1, 1)),
+    "k3_w14_256ch_two_stages": ((2, 256, 14, 14), (64, 256, 3, 3), (1, 1), (1, 1)),
+    "k3_w7_64ch": ((3, 64, 7, 7), (64, 64, 3, 3), (1, 1), (1, 1)),
+    "k3_w14_s2": ((2, 64, 14, 14), (40, 64, 3, 3), (2, 2), (1, 1)),
+    "k3_w12_p0": ((1, 32, 9, 12), (16, 32, 3, 3), (1, 1), (0, 0)),
+    "k3_w9_rect_stride": ((2, 32, 11, 9), (70, 32, 3, 3), (2, 1), (1, 0)),
+    "k3_w5_two_rows_a_piece": ((2, 32, 6, 5), (16, 32, 3, 3), (1, 1), (1, 1)),
+    "k3_w4_three_rows_a_piece": ((1, 32, 4, 4), (8, 32, 3, 3), (1, 1), (1, 1)),
+    "k3_w30_tall": ((1, 32, 40, 30), (64, 32, 3, 3), (1, 1), (1, 1)),
+    "k5_w14": ((1, 64, 14, 14), (32, 64, 5, 5), (1, 1), (2, 2)),
+    "k5_w7_s2": ((2, 32, 7, 7), (16, 32, 5, 5), (2, 2), (2, 2)),
 }
 
 
@@ -123,6 +136,18 @@ def test_strided_signal_view(device):
     want = ops.convolve2d(hx.permute(0, 3, 1, 2), hw, None, 1, 1).numpy()
     got = ops.convolve2d(dx.permute(0, 3, 1, 2), dw, None, 1, 1).numpy()
     support.assert_close(got, want, 1e-5, 54 * 2.0 ** -24 * 16, "NHWC view")
+
+
+@pytest.mark.parametrize("dtype", [ta.float16, ta.bfloat16], ids=str)
+def test_channel_slice_of_a_larger_signal(device, dtype):
+    """Channels 3..34 of a [2, 40, 14, 14] signal: planes that start at odd multiples of 196 elements, images 40 planes apart;
+    and the same from a width of 16 (aligned rows, but the slice starts in the middle of nothing aligned to 16 bytes)."""
+    for width in (14, 16):
+        hx, dx = support.both(support.values_for(dtype, SEED, 6, (2, 40, 14, width), -2, 2), dtype, device)
+        hw, dw = support.both(support.values_for(dtype, SEED, 7, (24, 32, 3, 3), -0.2, 0.2), dtype, device)
+        want = ops.convolve2d(hx[:, 3:35], hw, None, 1, 1).numpy()
+        got = ops.convolve2d(dx[:, 3:35], dw, None, 1, 1).numpy()
+        support.assert_close(got, want, 2e-3 if dtype is ta.float16 else 2.0 ** -7, 1e-3, f"channel slice, width {width}")
 
 
 def test_status_codes(device):
