@@ -42,6 +42,63 @@ __global__ __launch_bounds__(256) void conv_subsample4_kernel(const T* x, T* out
     *reinterpret_cast<Quad*>(out + static_cast<int64_t>(row) * p.WO + quad * 4) = bits;
 }
 
+// Pixel counts that are not a multiple of 16 bytes (14 x 14, 7 x 7 ...): the product wants its rows of pixels to start at
+// multiples of 16 bytes, so the sampled pixels of every (image, channel) go to rows of `pitch` elements (the count rounded
+// up; the rest zeros), channel by channel with the images side by side, so that ONE product O x C . C x (N * pitch) does the
+// whole batch on whole tiles (a product per image would have 200 or 56 columns); its rows are then copied to where they belong.
+// out[(c * N + n) * pitch + pix] = x[n][c][oh * stride_h][ow * stride_w], pix = oh * WO + ow; 16 bytes per thread.
+template <class T, bool PLANE>
+__global__ __launch_bounds__(256) void conv_repitch_kernel(const T* x, T* out, ConvProblem p, uint32_t pixels, uint32_t pitch, FastDiv div_groups, FastDiv div_c,
+                                                           FastDiv div_wo, uint32_t total) {
+    constexpr int E = 16 / sizeof(T);
+    const uint32_t idx = blockIdx.x * 256 + threadIdx.x;
+    if (idx >= total) return;
+    uint32_t row, group, n, c, oh, ow;
+    div_groups.divmod(idx, row, group);
+    div_c.divmod(row, n, c);
+    const T* plane = x + static_cast<int64_t>(n) * p.xs[0] + static_cast<int64_t>(c) * p.xs[1];
+    uint4 bits;
+    if (PLANE && group * E + E <= pixels) {
+        // no stride, rows that follow each other: the pixels of a channel are one run of memory
+        typedef unsigned int uint4_any __attribute__((ext_vector_type(4), aligned(2)));   // 16 bytes at any element
+        const uint4_any run = *reinterpret_cast<const uint4_any*>(plane + group * E);
+        __builtin_memcpy(&bits, &run, 16);
+    } else {
+        div_wo.divmod(group * E, oh, ow);
+        T v[E];
+#pragma unroll
+        for (int e = 0; e < E; ++e) {
+            const bool live = group * E + e < pixels;
+            v[e] = live ? plane[static_cast<int64_t>(oh * p.stride_h) * p.xs[2] + static_cast<int64_t>(ow * p.stride_w) * p.xs[3]] : T{};
+            if (++ow == p.WO) { ow = 0; ++oh; }
+        }
+        __builtin_memcpy(&bits, v, 16);
+    }
+    *reinterpret_cast<uint4*>(out + (static_cast<size_t>(c) * p.N + n) * pitch + group * E) = bits;
+}
+
+// y[n][o][pix] = rows[(o * N + n) * pitch + pix] for pix < pixels; 16 bytes per thread, stored at whatever address they belong.
+template <class T>
+__global__ __launch_bounds__(256) void conv_unpitch_kernel(const T* rows, T* y, ConvProblem p, uint32_t pixels, uint32_t pitch, FastDiv div_groups, FastDiv div_o,
+                                                           uint32_t total) {
+    constexpr int E = 16 / sizeof(T);
+    typedef unsigned int uint4_any __attribute__((ext_vector_type(4), aligned(2)));   // 16 bytes at any element
+    const uint32_t idx = blockIdx.x * 256 + threadIdx.x;
+    if (idx >= total) return;
+    uint32_t row, group, n, o;
+    div_groups.divmod(idx, row, group);
+    div_o.divmod(row, n, o);
+    const uint4_any bits = *reinterpret_cast<const uint4_any*>(rows + (static_cast<size_t>(o) * p.N + n) * pitch + group * E);
+    T* dst = y + static_cast<int64_t>(n) * p.ys[0] + static_cast<int64_t>(o) * p.ys[1] + group * E;
+    if (group * E + E <= pixels) {
+        *reinterpret_cast<uint4_any*>(dst) = bits;
+    } else {
+        T v[E];
+        __builtin_memcpy(v, &bits, 16);
+        for (uint32_t e = 0; group * E + e < pixels; ++e) dst[e] = v[e];
+    }
+}
+
 template <class T>
 int product(const GemmProblem& g, int dtype, const void* a, const void* b, void* c, hipStream_t stream) {
     if constexpr (std::is_same_v<T, float>) return gemm_mfma_f32(g, static_cast<const float*>(a), static_cast<const float*>(b), static_cast<float*>(c), stream);
@@ -77,6 +134,53 @@ int run_pointwise(const ConvProblem& p, int dtype, const void* x, const void* w,
     g.c_bs[0] = p.ys[0];
     g.row_bias = bias;
     const bool dense = p.stride_h == 1 && p.stride_w == 1;
+    constexpr int E = 16 / sizeof(T);   // elements per 16 bytes
+    if (pixels % E != 0) {
+        // rows of pixels that do not start at multiples of 16 bytes: through rows of a rounded-up pitch (see conv_repitch_kernel)
+        if (p.ws[0] % E != 0 || p.C % E != 0 || reinterpret_cast<uintptr_t>(w) % 16 != 0) return TANNIC_UNSUPPORTED_DTYPE;
+        const uint32_t pitch = static_cast<uint32_t>((pixels + E - 1) / E * E), groups = pitch / E;
+        const uint64_t in_rows = static_cast<uint64_t>(p.N) * p.C, out_rows = static_cast<uint64_t>(p.N) * p.O;
+        if (in_rows * groups >= (1ull << 31) || out_rows * groups >= (1ull << 31) || static_cast<uint64_t>(p.N) * pitch >= (1ull << 31)) return TANNIC_UNSUPPORTED_DTYPE;
+        T* dense_x = nullptr;
+        T* rows = nullptr;
+        if (scratch_acquire(reinterpret_cast<void**>(&dense_x), in_rows * pitch * sizeof(T), stream) != TANNIC_SUCCESS) return TANNIC_ERROR;
+        if (scratch_acquire(reinterpret_cast<void**>(&rows), out_rows * pitch * sizeof(T), stream) != TANNIC_SUCCESS) {
+            scratch_release(dense_x, stream);
+            return TANNIC_ERROR;
+        }
+        const uint32_t total_in = static_cast<uint32_t>(in_rows * groups), total_out = static_cast<uint32_t>(out_rows * groups);
+        const bool plane = dense && p.xs[3] == 1 && p.xs[2] == static_cast<int64_t>(p.W) && reinterpret_cast<uintptr_t>(x) % sizeof(T) == 0;
+        if (plane)
+            hipLaunchKernelGGL((conv_repitch_kernel<T, true>), dim3((total_in + 255) / 256), dim3(256), 0, stream, static_cast<const T*>(x), dense_x, p,
+                               static_cast<uint32_t>(pixels), pitch, FastDiv(groups), FastDiv(p.C), FastDiv(p.WO), total_in);
+        else
+            hipLaunchKernelGGL((conv_repitch_kernel<T, false>), dim3((total_in + 255) / 256), dim3(256), 0, stream, static_cast<const T*>(x), dense_x, p,
+                               static_cast<uint32_t>(pixels), pitch, FastDiv(groups), FastDiv(p.C), FastDiv(p.WO), total_in);
+        int status = launch_status("conv_repitch_kernel");
+        if (status == TANNIC_SUCCESS) {
+            const uint64_t columns = static_cast<uint64_t>(p.N) * pitch;
+            g.N = static_cast<uint32_t>(columns);
+            g.b_rs = static_cast<int64_t>(columns);
+            g.c_rs = static_cast<int64_t>(columns);
+            g.batch_rank = 0;
+            g.batches = 1;
+            g.batch_extent[0] = 1;
+            g.b_bs[0] = g.c_bs[0] = 0;
+            status = product<T>(g, dtype, w, dense_x, rows, stream);
+            if (status == TANNIC_UNSUPPORTED_DTYPE) {
+                set_error_text("conv2d: internal: the 1x1 product refused a problem its caller had checked");
+                status = TANNIC_ERROR;
+            }
+        }
+        if (status == TANNIC_SUCCESS) {
+            hipLaunchKernelGGL((conv_unpitch_kernel<T>), dim3((total_out + 255) / 256), dim3(256), 0, stream, rows, static_cast<T*>(y), p,
+                               static_cast<uint32_t>(pixels), pitch, FastDiv(groups), FastDiv(p.O), total_out);
+            status = launch_status("conv_unpitch_kernel");
+        }
+        scratch_release(rows, stream);
+        scratch_release(dense_x, stream);
+        return status;
+    }
     if (dense) {
         if (p.xs[3] != 1 || p.xs[2] != static_cast<int64_t>(p.W)) return TANNIC_UNSUPPORTED_DTYPE;
         g.b_rs = p.xs[1];
@@ -84,7 +188,6 @@ int run_pointwise(const ConvProblem& p, int dtype, const void* x, const void* w,
         return product<T>(g, dtype, w, x, y, stream);
     }
     // strided: gather first.  The product's own conditions are checked before any work is queued.
-    constexpr int E = 16 / sizeof(T);   // elements per 16 bytes
     if (p.WO % 4 != 0 || pixels % E != 0 || p.ws[0] % E != 0 || p.C % E != 0 || reinterpret_cast<uintptr_t>(w) % 16 != 0) return TANNIC_UNSUPPORTED_DTYPE;
     const uint64_t rows = static_cast<uint64_t>(p.N) * p.C * p.HO, quads = rows * (p.WO / 4);
     if (quads >= (1ull << 31)) return TANNIC_UNSUPPORTED_DTYPE;

@@ -83,6 +83,13 @@ CASES = {
     "k3_w30_tall": ((1, 32, 40, 30), (64, 32, 3, 3), (1, 1), (1, 1)),
     "k5_w14": ((1, 64, 14, 14), (32, 64, 5, 5), (1, 1), (2, 2)),
     "k5_w7_s2": ((2, 32, 7, 7), (16, 32, 5, 5), (2, 2), (2, 2)),
+    # 1x1 kernels over pixel counts that are not a multiple of 16 bytes (196, 49, 45, 55): the product per image runs on
+    # rows of a rounded-up pitch
+    "k1_14x14_c512": ((2, 512, 14, 14), (64, 512, 1, 1), (1, 1), (0, 0)),
+    "k1_7x7_c256": ((3, 256, 7, 7), (40, 256, 1, 1), (1, 1), (0, 0)),
+    "k1_s2_14_to_7": ((2, 128, 14, 14), (72, 128, 1, 1), (2, 2), (0, 0)),
+    "k1_5x9": ((2, 64, 5, 9), (24, 64, 1, 1), (1, 1), (0, 0)),
+    "k1_s2x1_to_5x11": ((1, 64, 9, 11), (16, 64, 1, 1), (2, 1), (0, 0)),
 }
 
 
