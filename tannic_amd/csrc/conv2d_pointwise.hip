@@ -100,6 +100,24 @@ __global__ __launch_bounds__(256) void conv_unpitch_kernel(const T* rows, T* y, 
 }
 
 template <class T>
+static int launch_unpitch(const ConvProblem& p, const void* rows, void* y, uint32_t pixels, uint32_t pitch, hipStream_t stream) {
+    constexpr int E = 16 / sizeof(T);
+    const uint32_t groups = pitch / E;
+    const uint64_t total = static_cast<uint64_t>(p.N) * p.O * groups;
+    if (total >= (1ull << 31) || pitch % E != 0) return TANNIC_UNSUPPORTED_DTYPE;
+    hipLaunchKernelGGL((conv_unpitch_kernel<T>), dim3((total + 255) / 256), dim3(256), 0, stream, static_cast<const T*>(rows), static_cast<T*>(y), p, pixels, pitch,
+                       FastDiv(groups), FastDiv(p.O), static_cast<uint32_t>(total));
+    return launch_status("conv_unpitch_kernel");
+}
+
+int conv_unpitch_rows(const ConvProblem& p, int dtype, const void* rows, void* y, uint32_t pixels, uint32_t pitch, hipStream_t stream) {
+    if (dtype == TANNIC_FLOAT16) return launch_unpitch<f16>(p, rows, y, pixels, pitch, stream);
+    if (dtype == TANNIC_BFLOAT16) return launch_unpitch<bf16>(p, rows, y, pixels, pitch, stream);
+    if (dtype == TANNIC_FLOAT32) return launch_unpitch<float>(p, rows, y, pixels, pitch, stream);
+    return TANNIC_UNSUPPORTED_DTYPE;
+}
+
+template <class T>
 int product(const GemmProblem& g, int dtype, const void* a, const void* b, void* c, hipStream_t stream) {
     if constexpr (std::is_same_v<T, float>) return gemm_mfma_f32(g, static_cast<const float*>(a), static_cast<const float*>(b), static_cast<float*>(c), stream);
     else return gemm_mfma_16bit(g, dtype, a, b, c, stream);
@@ -148,7 +166,7 @@ int run_pointwise(const ConvProblem& p, int dtype, const void* x, const void* w,
             scratch_release(dense_x, stream);
             return TANNIC_ERROR;
         }
-        const uint32_t total_in = static_cast<uint32_t>(in_rows * groups), total_out = static_cast<uint32_t>(out_rows * groups);
+        const uint32_t total_in = static_cast<uint32_t>(in_rows * groups);
         const bool plane = dense && p.xs[3] == 1 && p.xs[2] == static_cast<int64_t>(p.W) && reinterpret_cast<uintptr_t>(x) % sizeof(T) == 0;
         if (plane)
             hipLaunchKernelGGL((conv_repitch_kernel<T, true>), dim3((total_in + 255) / 256), dim3(256), 0, stream, static_cast<const T*>(x), dense_x, p,
@@ -172,11 +190,7 @@ int run_pointwise(const ConvProblem& p, int dtype, const void* x, const void* w,
                 status = TANNIC_ERROR;
             }
         }
-        if (status == TANNIC_SUCCESS) {
-            hipLaunchKernelGGL((conv_unpitch_kernel<T>), dim3((total_out + 255) / 256), dim3(256), 0, stream, rows, static_cast<T*>(y), p,
-                               static_cast<uint32_t>(pixels), pitch, FastDiv(groups), FastDiv(p.O), total_out);
-            status = launch_status("conv_unpitch_kernel");
-        }
+        if (status == TANNIC_SUCCESS) status = launch_unpitch<T>(p, rows, y, static_cast<uint32_t>(pixels), pitch, stream);
         scratch_release(rows, stream);
         scratch_release(dense_x, stream);
         return status;

@@ -394,7 +394,7 @@ static bool operands_fit(const GemmProblem& p, int bm, int bn, bool& a_t, bool& 
 template <class T>
 int gemm16_dtl_split(const GemmProblem& p, int bm, uint32_t splits, uint32_t k_chunk, float* partials, const void* a, const void* b, hipStream_t stream) {
     bool a_t, b_t;
-    if (p.row_bias || !operands_fit<T>(p, bm, 128, a_t, b_t) || p.N % 4 != 0 || k_chunk % 64 != 0) return TANNIC_UNSUPPORTED_DTYPE;
+    if (!operands_fit<T>(p, bm, 128, a_t, b_t) || p.N % 4 != 0 || k_chunk % 64 != 0) return TANNIC_UNSUPPORTED_DTYPE;   // (a row start value is added with the partial sums)
     const SplitK sk{splits, k_chunk, partials};
     if (bm == 64) {
         // 64 x 128 tiles, six stages: a workgroup's share of K is short and its operands are in no cache, so what counts

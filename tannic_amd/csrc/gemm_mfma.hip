@@ -227,7 +227,8 @@ __global__ __launch_bounds__(128 * WAVES_N) void gemm16_kernel(const T* A, const
 #pragma unroll
     for (int i = 0; i < TM; ++i) {
         const uint32_t row = tm * BM + (wave / WAVES_N) * WM + i * 32 + lane % 32;
-        const float start = (p.row_bias && row < p.M) ? static_cast<float>(widen(static_cast<const T*>(p.row_bias)[row])) : 0.0f;
+        // (blocks that share K leave the start value to the pass that adds up their partial sums)
+        const float start = (!SPLIT && p.row_bias && row < p.M) ? static_cast<float>(widen(static_cast<const T*>(p.row_bias)[row])) : 0.0f;
 #pragma unroll
         for (int j = 0; j < TN; ++j)
 #pragma unroll
@@ -475,7 +476,9 @@ __global__ __launch_bounds__(256) void gemm_split_reduce_kernel(const float* par
     const uint32_t batch = r / p.M, m = r % p.M;
     const size_t share = static_cast<size_t>(p.batches) * p.M * p.N;
     const float* src = partials + static_cast<size_t>(r) * p.N + col;
-    float sum[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+    // the row's start value (the bias of a convolution) first, then the shares of K in their order
+    const float start = p.row_bias ? static_cast<float>(widen(static_cast<const T*>(p.row_bias)[m])) : 0.0f;
+    float sum[4] = {start, start, start, start};
     const uint32_t live = p.N - col < 4 ? p.N - col : 4;
     if (p.N % 4 == 0) {   // rows of the partial sums start at multiples of 16 bytes
         for (uint32_t sp = 0; sp < splits; ++sp) {
@@ -611,7 +614,7 @@ int run16(const GemmProblem& p, const void* a, const void* b, void* c, hipStream
         if ((bm == 128 && !tall) || (bm == 256 && p.M <= 192)) continue;
         const uint64_t tiles = static_cast<uint64_t>((p.M + bm - 1) / bm) * ((p.N + 127) / 128) * p.batches;
         for (uint32_t splits : {1u, 2u, 4u, 8u, 16u}) {
-            if (splits > 1 && (bm == 256 || p.row_bias || splits > p.K / (sizeof(T) == 4 ? 64 : 256))) break;
+            if (splits > 1 && (bm == 256 || splits > p.K / (sizeof(T) == 4 ? 64 : 256))) break;
             const double blocks = static_cast<double>(tiles) * splits;
             const double rounds = static_cast<double>((static_cast<uint64_t>(blocks) + 255) / 256);
             // a step costs more the more compute units pull operands through the L2s at the same time

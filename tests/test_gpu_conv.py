@@ -90,6 +90,11 @@ CASES = {
     "k1_s2_14_to_7": ((2, 128, 14, 14), (72, 128, 1, 1), (2, 2), (0, 0)),
     "k1_5x9": ((2, 64, 5, 9), (24, 64, 1, 1), (1, 1), (0, 0)),
     "k1_s2x1_to_5x11": ((1, 64, 9, 11), (16, 64, 1, 1), (2, 1), (0, 0)),
+    # few output pixels per image under a long K: the whole batch unfolded side by side, one product
+    "unfolded_k3_7x7": ((5, 128, 7, 7), (40, 128, 3, 3), (1, 1), (1, 1)),
+    "unfolded_k3_s2_14_to_7": ((6, 64, 14, 14), (48, 64, 3, 3), (2, 2), (1, 1)),
+    "unfolded_k5_9x9": ((8, 32, 9, 9), (16, 32, 5, 5), (1, 1), (2, 2)),
+    "unfolded_k3x2_100_pixels": ((3, 96, 10, 11), (24, 96, 3, 2), (1, 1), (1, 0)),
 }
 
 
