@@ -57,7 +57,7 @@ UNITS = [
     ("conv2d_stem.hip", "conv2d_stem.o", []),
     ("conv2d_gather32.hip", "conv2d_gather32.o", []),
     ("conv2d_unfold.hip", "conv2d_unfold.o", []),
-    ("conv2d_unfold16.hip", "conv2d_unfold16.o", []),
+    ("conv2d_unfold_batch.hip", "conv2d_unfold_batch.o", []),
 ]
 
 

@@ -334,7 +334,9 @@ int conv2d_gather32(const ConvProblem& p, int dtype, const void* x, const void* 
     if (reach >= (1ull << 31)) return TANNIC_UNSUPPORTED_DTYPE;
     const uint32_t K = static_cast<uint32_t>(K64), pixels = static_cast<uint32_t>(pixels64);
     const bool wv = K % 4 == 0 && reinterpret_cast<uintptr_t>(w) % 16 == 0;
-    if (p.O > 64) return wv ? launch_gather32<128, true>(p, K, pixels, x, w, bias, y, stream) : launch_gather32<128, false>(p, K, pixels, x, w, bias, y, stream);
+    // 128 output channels per block only while that leaves a block for (nearly) every compute unit
+    const uint64_t wide_blocks = (pixels64 + kG32BP - 1) / kG32BP * ((p.O + 127) / 128);
+    if (p.O > 64 && wide_blocks >= 200) return wv ? launch_gather32<128, true>(p, K, pixels, x, w, bias, y, stream) : launch_gather32<128, false>(p, K, pixels, x, w, bias, y, stream);
     return wv ? launch_gather32<64, true>(p, K, pixels, x, w, bias, y, stream) : launch_gather32<64, false>(p, K, pixels, x, w, bias, y, stream);
 }
 

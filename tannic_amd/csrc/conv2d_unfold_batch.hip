@@ -1,11 +1,11 @@
-// conv2d for 16-bit signals with few output pixels per image and many channels (the last stages of a ResNet: 3x3 over
-// 7 x 7 with 512 channels): unfold the whole batch, then ONE matrix product.
+// conv2d for fp16 / bf16 / fp32 signals with few output pixels per image and many channels (the last stages of a ResNet:
+// 3x3 over 7 x 7 with 512 channels): unfold the whole batch, then ONE matrix product.
 //
 // A tile of the patch kernels (conv2d_k3.hip) is one image's pixels, 49 of them in a tile made for 256, and every block
 // regroups the weights of its 64 output channels again, 590 KB for 512 channels.  With so few pixels the unfolded
 // operand is small instead (K x N x pixels: 16.5 MB for the layer above at batch 32), so it is written out,
 //   col[k][n * pitch + pix] = x[n][c][oh * stride_h + kh - pad_h][ow * stride_w + kw - pad_w]   (zero in the padding),
-// k = (c, kh, kw) in the kernel tensor's own order, pitch = pixels rounded up to 8, images side by side, and
+// k = (c, kh, kw) in the kernel tensor's own order, pitch = pixels rounded up to 16 bytes, images side by side, and
 // rows (O x N * pitch) = w (O x K) . col runs on the matrix-multiply kernels with the bias as per-row start value; the
 // rows are then copied to y[n][o][pix] (conv_unpitch_rows).  Sums run over k in the reference's order (src/cpu/conv2d.cpp:45-60).
 #include "conv_common.hpp"
@@ -13,44 +13,48 @@
 
 namespace th {
 
-// 16 bytes (eight pixels of one k and image) per thread
+// 16 bytes (eight or four pixels of one k and image) per thread
 template <class T>
-__global__ __launch_bounds__(256) void conv_unfold16_kernel(const T* x, T* col, ConvProblem p, uint32_t pixels, uint32_t pitch, FastDiv div_groups, FastDiv div_n,
+__global__ __launch_bounds__(256) void conv_unfold_batch_kernel(const T* x, T* col, ConvProblem p, uint32_t pixels, uint32_t pitch, FastDiv div_groups, FastDiv div_n,
                                                             FastDiv div_wo, FastDiv div_taps, FastDiv div_kw, uint32_t total) {
+    constexpr int E = 16 / sizeof(T);
     const uint32_t idx = blockIdx.x * 256 + threadIdx.x;
     if (idx >= total) return;
-    uint32_t row, group, k, n, c, tap, kh, kw, oh, ow;
-    div_groups.divmod(idx, row, group);
-    div_n.divmod(row, k, n);
-    div_taps.divmod(k, c, tap);
+    // neighbouring threads: the pixel groups, then the taps of one (channel, image) — they all read the same few rows of one plane
+    uint32_t rest, plane_id, group, n, c, tap, kh, kw, oh, ow;
+    div_groups.divmod(idx, rest, group);
+    div_taps.divmod(rest, plane_id, tap);
+    div_n.divmod(plane_id, c, n);
     div_kw.divmod(tap, kh, kw);
+    const uint32_t row = (c * div_taps.d + tap) * p.N + n;   // k * N + n
     const T* plane = x + static_cast<int64_t>(n) * p.xs[0] + static_cast<int64_t>(c) * p.xs[1];
-    div_wo.divmod(group * 8, oh, ow);
-    T v[8];
+    div_wo.divmod(group * E, oh, ow);
+    T v[E];
 #pragma unroll
-    for (int e = 0; e < 8; ++e) {
+    for (int e = 0; e < E; ++e) {
         const uint32_t ih = oh * p.stride_h + kh - p.pad_h, iw = ow * p.stride_w + kw - p.pad_w;   // unsigned: above and left of the image are huge
-        const bool inside = group * 8 + e < pixels && ih < p.H && iw < p.W;
+        const bool inside = group * E + e < pixels && ih < p.H && iw < p.W;
         v[e] = inside ? plane[static_cast<int64_t>(ih) * p.xs[2] + static_cast<int64_t>(iw) * p.xs[3]] : T{};
         if (++ow == p.WO) { ow = 0; ++oh; }
     }
     uint4 bits;
     __builtin_memcpy(&bits, v, 16);
-    *reinterpret_cast<uint4*>(col + static_cast<size_t>(row) * pitch + group * 8) = bits;
+    *reinterpret_cast<uint4*>(col + static_cast<size_t>(row) * pitch + group * E) = bits;
 }
 
 template <class T>
-static int run_unfold16(const ConvProblem& p, int dtype, const void* x, const void* w, const void* bias, void* y, hipStream_t stream) {
+static int run_unfold_batch(const ConvProblem& p, int dtype, const void* x, const void* w, const void* bias, void* y, hipStream_t stream) {
     if (p.has_bias && p.bs != 1 && p.O > 1) return TANNIC_UNSUPPORTED_DTYPE;   // the product reads its row bias as a dense vector
     if (p.N == 0 || p.O == 0 || p.HO == 0 || p.WO == 0) return TANNIC_SUCCESS;
+    constexpr int E = 16 / sizeof(T);
     const uint64_t K = static_cast<uint64_t>(p.C) * p.KH * p.KW, pixels = static_cast<uint64_t>(p.HO) * p.WO;
     // Where this pays: few pixels per image (a tile of the patch kernels would be mostly empty), a long K, and enough
     // columns in all for whole tiles of the product.
-    if (pixels > 100 || K < 512 || K % 8 != 0 || K >= (1u << 24)) return TANNIC_UNSUPPORTED_DTYPE;
-    const uint32_t pitch = static_cast<uint32_t>((pixels + 7) / 8 * 8);
+    if (pixels > 100 || K < 512 || K % E != 0 || K >= (1u << 24)) return TANNIC_UNSUPPORTED_DTYPE;
+    const uint32_t pitch = static_cast<uint32_t>((pixels + E - 1) / E * E);
     const uint64_t columns = static_cast<uint64_t>(p.N) * pitch;
-    if (columns < 256 || columns >= (1ull << 31) || K * p.N * (pitch / 8) >= (1ull << 31)) return TANNIC_UNSUPPORTED_DTYPE;
-    if (K * columns * sizeof(T) > (256ull << 20)) return TANNIC_UNSUPPORTED_DTYPE;
+    if (columns < 256 || columns >= (1ull << 31) || K * p.N * (pitch / E) >= (1ull << 31)) return TANNIC_UNSUPPORTED_DTYPE;
+    if (K * columns * sizeof(T) > (512ull << 20)) return TANNIC_UNSUPPORTED_DTYPE;
     // the kernel tensor as a K-contiguous O x K matrix, the result as pixel-contiguous rows
     if (p.ws[3] != 1 || p.ws[2] != static_cast<int64_t>(p.KW) || p.ws[1] != static_cast<int64_t>(p.KH) * p.KW || p.ws[0] != static_cast<int64_t>(K) ||
         reinterpret_cast<uintptr_t>(w) % 16 != 0)
@@ -61,10 +65,10 @@ static int run_unfold16(const ConvProblem& p, int dtype, const void* x, const vo
     if (scratch_acquire(reinterpret_cast<void**>(&scratch), col_bytes + static_cast<size_t>(p.O) * columns * sizeof(T), stream) != TANNIC_SUCCESS) return TANNIC_ERROR;
     T* col = reinterpret_cast<T*>(scratch);
     T* rows = reinterpret_cast<T*>(scratch + col_bytes);
-    const uint32_t groups = pitch / 8, total = static_cast<uint32_t>(K * p.N * groups);
-    hipLaunchKernelGGL((conv_unfold16_kernel<T>), dim3((total + 255) / 256), dim3(256), 0, stream, static_cast<const T*>(x), col, p, static_cast<uint32_t>(pixels), pitch,
+    const uint32_t groups = pitch / E, total = static_cast<uint32_t>(K * p.N * groups);
+    hipLaunchKernelGGL((conv_unfold_batch_kernel<T>), dim3((total + 255) / 256), dim3(256), 0, stream, static_cast<const T*>(x), col, p, static_cast<uint32_t>(pixels), pitch,
                        FastDiv(groups), FastDiv(p.N), FastDiv(p.WO), FastDiv(p.KH * p.KW), FastDiv(p.KW), total);
-    int status = launch_status("conv_unfold16_kernel");
+    int status = launch_status("conv_unfold_batch_kernel");
     if (status == TANNIC_SUCCESS) {
         GemmProblem g{};
         g.M = p.O;
@@ -82,7 +86,8 @@ static int run_unfold16(const ConvProblem& p, int dtype, const void* x, const vo
             g.a_bs[d] = g.b_bs[d] = g.c_bs[d] = 0;
         }
         g.row_bias = bias;
-        status = gemm_mfma_16bit(g, dtype, w, col, rows, stream);
+        if constexpr (std::is_same_v<T, float>) status = gemm_mfma_f32(g, static_cast<const float*>(w), reinterpret_cast<const float*>(col), reinterpret_cast<float*>(rows), stream);
+        else status = gemm_mfma_16bit(g, dtype, w, col, rows, stream);
         if (status == TANNIC_UNSUPPORTED_DTYPE) {
             set_error_text("conv2d: internal: the unfolded product refused a problem its caller had checked");
             status = TANNIC_ERROR;
@@ -93,10 +98,11 @@ static int run_unfold16(const ConvProblem& p, int dtype, const void* x, const vo
     return status;
 }
 
-int conv2d_unfold16(const ConvProblem& p, int dtype, const void* x, const void* w, const void* bias, void* y, hipStream_t stream) {
+int conv2d_unfold_batch(const ConvProblem& p, int dtype, const void* x, const void* w, const void* bias, void* y, hipStream_t stream) {
     if (p.KH == 1 && p.KW == 1) return TANNIC_UNSUPPORTED_DTYPE;   // conv2d_pointwise.hip: no unfolding needed
-    if (dtype == TANNIC_FLOAT16) return run_unfold16<f16>(p, dtype, x, w, bias, y, stream);
-    if (dtype == TANNIC_BFLOAT16) return run_unfold16<bf16>(p, dtype, x, w, bias, y, stream);
+    if (dtype == TANNIC_FLOAT16) return run_unfold_batch<f16>(p, dtype, x, w, bias, y, stream);
+    if (dtype == TANNIC_BFLOAT16) return run_unfold_batch<bf16>(p, dtype, x, w, bias, y, stream);
+    if (dtype == TANNIC_FLOAT32) return run_unfold_batch<float>(p, dtype, x, w, bias, y, stream);
     return TANNIC_UNSUPPORTED_DTYPE;
 }
 
