@@ -332,6 +332,38 @@ def conv_entry(b, dtype, name, xs, ws, stride, pad, iters):
             "mfma_frac": round(tflops / peak, 4), "hbm_frac": round(nbytes / ms / 1e6 / HBM_PEAK_GBS, 4)}
 
 
+# the 23 distinct convolution shapes of ResNet-50 (stem, and per stage the 1x1 / 3x3 / 1x1 of a bottleneck, its strided
+# first block and its projection): (name, C, H, O, kernel, stride, pad)
+RESNET50_LAYERS = [
+    ("conv1 3->64 k7 s2 @224", 3, 224, 64, 7, 2, 3),
+    ("conv2 64->64 k1 @56", 64, 56, 64, 1, 1, 0), ("conv2 64->64 k3 @56", 64, 56, 64, 3, 1, 1), ("conv2 64->256 k1 @56", 64, 56, 256, 1, 1, 0),
+    ("conv2 256->64 k1 @56", 256, 56, 64, 1, 1, 0), ("conv3 256->128 k1 @56", 256, 56, 128, 1, 1, 0), ("conv3 128->128 k3 s2 @56", 128, 56, 128, 3, 2, 1),
+    ("conv3 128->128 k3 @28", 128, 28, 128, 3, 1, 1), ("conv3 128->512 k1 @28", 128, 28, 512, 1, 1, 0), ("conv3 512->128 k1 @28", 512, 28, 128, 1, 1, 0),
+    ("conv3 256->512 k1 s2 @56", 256, 56, 512, 1, 2, 0), ("conv4 512->256 k1 @28", 512, 28, 256, 1, 1, 0), ("conv4 256->256 k3 s2 @28", 256, 28, 256, 3, 2, 1),
+    ("conv4 256->256 k3 @14", 256, 14, 256, 3, 1, 1), ("conv4 256->1024 k1 @14", 256, 14, 1024, 1, 1, 0), ("conv4 1024->256 k1 @14", 1024, 14, 256, 1, 1, 0),
+    ("conv4 512->1024 k1 s2 @28", 512, 28, 1024, 1, 2, 0), ("conv5 1024->512 k1 @14", 1024, 14, 512, 1, 1, 0), ("conv5 512->512 k3 s2 @14", 512, 14, 512, 3, 2, 1),
+    ("conv5 512->512 k3 @7", 512, 7, 512, 3, 1, 1), ("conv5 512->2048 k1 @7", 512, 7, 2048, 1, 1, 0), ("conv5 2048->512 k1 @7", 2048, 7, 512, 1, 1, 0),
+    ("conv5 1024->2048 k1 s2 @14", 1024, 14, 2048, 1, 2, 0),
+]
+
+
+def resnet50_entry(b, dtype, batch, iters):
+    """Every distinct convolution of ResNet-50 once, at `batch` images: the sum of their times, and the slowest three."""
+    global SECONDARY_PREHEAT_SECONDS
+    keep, SECONDARY_PREHEAT_SECONDS = SECONDARY_PREHEAT_SECONDS, 0.02
+    try:
+        rows = [conv_entry(b, dtype, name, (batch, c, h, h), (o, c, k, k), s, pad, iters) for name, c, h, o, k, s, pad in RESNET50_LAYERS]
+    finally:
+        SECONDARY_PREHEAT_SECONDS = keep
+    us = sum(r["us"] for r in rows)
+    flops = sum(r["tflops"] * r["us"] * 1e6 for r in rows)
+    peak = MFMA_PEAK_TFLOPS["f32" if dtype is b.ta.float32 else "f16"]
+    slowest = sorted(rows, key=lambda r: -r["us"])[:3]
+    return {"op": f"conv2d {dtype} the 23 distinct layers of ResNet-50 N={batch}, one after the other", "us": round(us, 1), "tflops": round(flops / us / 1e6, 2),
+            "mfma_frac": round(flops / us / 1e6 / peak, 4), "layers": len(rows),
+            "slowest": [f"{r['op'].split(' ', 2)[2]}: {r['us']} us" for r in slowest]}
+
+
 def elementwise_entries(b, dtype, iters):
     ta, abi, ops = b.ta, b.abi, b.ops
     shape = (64, 4096, 1024)
@@ -463,6 +495,9 @@ def secondary(b, only):
         work.append(conv_entry(b, ta.float16, "128->128 k5 s1 p2 @32 N=32 (the 5x5 instance of the LDS-patch kernel, four chunks)", (32, 128, 32, 32), (128, 128, 5, 5), 1, 2, 5))
         work.append(conv_entry(b, ta.float16, "512->128 k1 s1 @28 N=32 (a product per image: conv2d_pointwise)", (32, 512, 28, 28), (128, 512, 1, 1), 1, 0, 5))
         work.append(conv_entry(b, ta.float16, "24->48 k3 s1 p1 @30 N=32 (general tiles, nothing aligned: conv2d_mfma, 64 channels wide)", (32, 24, 30, 30), (48, 24, 3, 3), 1, 1, 5))
+        # widths of 28, 14 and 7, pixel counts of 196 and 49, up to 2048 channels: what lies behind the three layers above
+        work.append(resnet50_entry(b, ta.float16, 32, 5))
+        work.append(resnet50_entry(b, ta.float32, 32, 3))
     if only in (None, "elementwise"):
         for dtype in (ta.float32, ta.float16, ta.int32):
             work += elementwise_entries(b, dtype, 10)
