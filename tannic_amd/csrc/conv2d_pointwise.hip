@@ -45,7 +45,8 @@ __global__ __launch_bounds__(256) void conv_subsample4_kernel(const T* x, T* out
 // Pixel counts that are not a multiple of 16 bytes (14 x 14, 7 x 7 ...): the product wants its rows of pixels to start at
 // multiples of 16 bytes, so the sampled pixels of every (image, channel) go to rows of `pitch` elements (the count rounded
 // up; the rest zeros), channel by channel with the images side by side, so that ONE product O x C . C x (N * pitch) does the
-// whole batch on whole tiles (a product per image would have 200 or 56 columns); its rows are then copied to where they belong.
+// whole batch on whole tiles (a product per image would have 200 or 56 columns); the product stores its columns image by
+// image (GemmProblem::c_group), straight into y.
 // out[(c * N + n) * pitch + pix] = x[n][c][oh * stride_h][ow * stride_w], pix = oh * WO + ow; 16 bytes per thread.
 template <class T, bool PLANE>
 __global__ __launch_bounds__(256) void conv_repitch_kernel(const T* x, T* out, ConvProblem p, uint32_t pixels, uint32_t pitch, FastDiv div_groups, FastDiv div_c,
@@ -75,46 +76,6 @@ __global__ __launch_bounds__(256) void conv_repitch_kernel(const T* x, T* out, C
         __builtin_memcpy(&bits, v, 16);
     }
     *reinterpret_cast<uint4*>(out + (static_cast<size_t>(c) * p.N + n) * pitch + group * E) = bits;
-}
-
-// y[n][o][pix] = rows[(o * N + n) * pitch + pix] for pix < pixels; 16 bytes per thread, stored at whatever address they belong.
-template <class T>
-__global__ __launch_bounds__(256) void conv_unpitch_kernel(const T* rows, T* y, ConvProblem p, uint32_t pixels, uint32_t pitch, FastDiv div_groups, FastDiv div_o,
-                                                           uint32_t total) {
-    constexpr int E = 16 / sizeof(T);
-    typedef unsigned int uint4_any __attribute__((ext_vector_type(4), aligned(2)));   // 16 bytes at any element
-    const uint32_t idx = blockIdx.x * 256 + threadIdx.x;
-    if (idx >= total) return;
-    uint32_t row, group, n, o;
-    div_groups.divmod(idx, row, group);
-    div_o.divmod(row, n, o);
-    const uint4_any bits = *reinterpret_cast<const uint4_any*>(rows + (static_cast<size_t>(o) * p.N + n) * pitch + group * E);
-    T* dst = y + static_cast<int64_t>(n) * p.ys[0] + static_cast<int64_t>(o) * p.ys[1] + group * E;
-    if (group * E + E <= pixels) {
-        *reinterpret_cast<uint4_any*>(dst) = bits;
-    } else {
-        T v[E];
-        __builtin_memcpy(v, &bits, 16);
-        for (uint32_t e = 0; group * E + e < pixels; ++e) dst[e] = v[e];
-    }
-}
-
-template <class T>
-static int launch_unpitch(const ConvProblem& p, const void* rows, void* y, uint32_t pixels, uint32_t pitch, hipStream_t stream) {
-    constexpr int E = 16 / sizeof(T);
-    const uint32_t groups = pitch / E;
-    const uint64_t total = static_cast<uint64_t>(p.N) * p.O * groups;
-    if (total >= (1ull << 31) || pitch % E != 0) return TANNIC_UNSUPPORTED_DTYPE;
-    hipLaunchKernelGGL((conv_unpitch_kernel<T>), dim3((total + 255) / 256), dim3(256), 0, stream, static_cast<const T*>(rows), static_cast<T*>(y), p, pixels, pitch,
-                       FastDiv(groups), FastDiv(p.O), static_cast<uint32_t>(total));
-    return launch_status("conv_unpitch_kernel");
-}
-
-int conv_unpitch_rows(const ConvProblem& p, int dtype, const void* rows, void* y, uint32_t pixels, uint32_t pitch, hipStream_t stream) {
-    if (dtype == TANNIC_FLOAT16) return launch_unpitch<f16>(p, rows, y, pixels, pitch, stream);
-    if (dtype == TANNIC_BFLOAT16) return launch_unpitch<bf16>(p, rows, y, pixels, pitch, stream);
-    if (dtype == TANNIC_FLOAT32) return launch_unpitch<float>(p, rows, y, pixels, pitch, stream);
-    return TANNIC_UNSUPPORTED_DTYPE;
 }
 
 template <class T>
@@ -160,12 +121,7 @@ int run_pointwise(const ConvProblem& p, int dtype, const void* x, const void* w,
         const uint64_t in_rows = static_cast<uint64_t>(p.N) * p.C, out_rows = static_cast<uint64_t>(p.N) * p.O;
         if (in_rows * groups >= (1ull << 31) || out_rows * groups >= (1ull << 31) || static_cast<uint64_t>(p.N) * pitch >= (1ull << 31)) return TANNIC_UNSUPPORTED_DTYPE;
         T* dense_x = nullptr;
-        T* rows = nullptr;
         if (scratch_acquire(reinterpret_cast<void**>(&dense_x), in_rows * pitch * sizeof(T), stream) != TANNIC_SUCCESS) return TANNIC_ERROR;
-        if (scratch_acquire(reinterpret_cast<void**>(&rows), out_rows * pitch * sizeof(T), stream) != TANNIC_SUCCESS) {
-            scratch_release(dense_x, stream);
-            return TANNIC_ERROR;
-        }
         const uint32_t total_in = static_cast<uint32_t>(in_rows * groups);
         const bool plane = dense && p.xs[3] == 1 && p.xs[2] == static_cast<int64_t>(p.W) && reinterpret_cast<uintptr_t>(x) % sizeof(T) == 0;
         if (plane)
@@ -179,19 +135,22 @@ int run_pointwise(const ConvProblem& p, int dtype, const void* x, const void* w,
             const uint64_t columns = static_cast<uint64_t>(p.N) * pitch;
             g.N = static_cast<uint32_t>(columns);
             g.b_rs = static_cast<int64_t>(columns);
-            g.c_rs = static_cast<int64_t>(columns);
             g.batch_rank = 0;
             g.batches = 1;
             g.batch_extent[0] = 1;
             g.b_bs[0] = g.c_bs[0] = 0;
-            status = product<T>(g, dtype, w, dense_x, rows, stream);
+            // the columns of image n go to y[n]: rows p.ys[1] apart, images p.ys[0]
+            g.c_rs = p.ys[1];
+            g.c_group = pitch;
+            g.c_group_live = static_cast<uint32_t>(pixels);
+            g.c_group_stride = p.ys[0];
+            g.c_group_div = FastDiv(pitch);
+            status = product<T>(g, dtype, w, dense_x, y, stream);
             if (status == TANNIC_UNSUPPORTED_DTYPE) {
                 set_error_text("conv2d: internal: the 1x1 product refused a problem its caller had checked");
                 status = TANNIC_ERROR;
             }
         }
-        if (status == TANNIC_SUCCESS) status = launch_unpitch<T>(p, rows, y, static_cast<uint32_t>(pixels), pitch, stream);
-        scratch_release(rows, stream);
         scratch_release(dense_x, stream);
         return status;
     }

@@ -6,8 +6,9 @@
 // operand is small instead (K x N x pixels: 16.5 MB for the layer above at batch 32), so it is written out,
 //   col[k][n * pitch + pix] = x[n][c][oh * stride_h + kh - pad_h][ow * stride_w + kw - pad_w]   (zero in the padding),
 // k = (c, kh, kw) in the kernel tensor's own order, pitch = pixels rounded up to 16 bytes, images side by side, and
-// rows (O x N * pitch) = w (O x K) . col runs on the matrix-multiply kernels with the bias as per-row start value; the
-// rows are then copied to y[n][o][pix] (conv_unpitch_rows).  Sums run over k in the reference's order (src/cpu/conv2d.cpp:45-60).
+// (O x N * pitch) = w (O x K) . col runs on the matrix-multiply kernels with the bias as per-row start value and its
+// columns stored image by image, straight into y (GemmProblem::c_group).  Sums run over k in the reference's order
+// (src/cpu/conv2d.cpp:45-60).
 #include "conv_common.hpp"
 #include "gemm_common.hpp"
 
@@ -60,11 +61,8 @@ static int run_unfold_batch(const ConvProblem& p, int dtype, const void* x, cons
         reinterpret_cast<uintptr_t>(w) % 16 != 0)
         return TANNIC_UNSUPPORTED_DTYPE;
     if (p.ys[3] != 1 || p.ys[2] != static_cast<int64_t>(p.WO)) return TANNIC_UNSUPPORTED_DTYPE;
-    const size_t col_bytes = (static_cast<size_t>(K) * columns * sizeof(T) + 255) & ~size_t(255);
-    unsigned char* scratch = nullptr;
-    if (scratch_acquire(reinterpret_cast<void**>(&scratch), col_bytes + static_cast<size_t>(p.O) * columns * sizeof(T), stream) != TANNIC_SUCCESS) return TANNIC_ERROR;
-    T* col = reinterpret_cast<T*>(scratch);
-    T* rows = reinterpret_cast<T*>(scratch + col_bytes);
+    T* col = nullptr;
+    if (scratch_acquire(reinterpret_cast<void**>(&col), static_cast<size_t>(K) * columns * sizeof(T), stream) != TANNIC_SUCCESS) return TANNIC_ERROR;
     const uint32_t groups = pitch / E, total = static_cast<uint32_t>(K * p.N * groups);
     hipLaunchKernelGGL((conv_unfold_batch_kernel<T>), dim3((total + 255) / 256), dim3(256), 0, stream, static_cast<const T*>(x), col, p, static_cast<uint32_t>(pixels), pitch,
                        FastDiv(groups), FastDiv(p.N), FastDiv(p.WO), FastDiv(p.KH * p.KW), FastDiv(p.KW), total);
@@ -78,7 +76,12 @@ static int run_unfold_batch(const ConvProblem& p, int dtype, const void* x, cons
         g.a_cs = 1;
         g.b_rs = static_cast<int64_t>(columns);
         g.b_cs = 1;
-        g.c_rs = static_cast<int64_t>(columns);
+        // the columns of image n go to y[n]: rows p.ys[1] apart, images p.ys[0]
+        g.c_rs = p.ys[1];
+        g.c_group = pitch;
+        g.c_group_live = static_cast<uint32_t>(pixels);
+        g.c_group_stride = p.ys[0];
+        g.c_group_div = FastDiv(pitch);
         g.batch_rank = 0;
         g.batches = 1;
         for (int d = 0; d < 6; ++d) {
@@ -86,15 +89,14 @@ static int run_unfold_batch(const ConvProblem& p, int dtype, const void* x, cons
             g.a_bs[d] = g.b_bs[d] = g.c_bs[d] = 0;
         }
         g.row_bias = bias;
-        if constexpr (std::is_same_v<T, float>) status = gemm_mfma_f32(g, static_cast<const float*>(w), reinterpret_cast<const float*>(col), reinterpret_cast<float*>(rows), stream);
-        else status = gemm_mfma_16bit(g, dtype, w, col, rows, stream);
+        if constexpr (std::is_same_v<T, float>) status = gemm_mfma_f32(g, static_cast<const float*>(w), reinterpret_cast<const float*>(col), static_cast<float*>(y), stream);
+        else status = gemm_mfma_16bit(g, dtype, w, col, y, stream);
         if (status == TANNIC_UNSUPPORTED_DTYPE) {
             set_error_text("conv2d: internal: the unfolded product refused a problem its caller had checked");
             status = TANNIC_ERROR;
         }
     }
-    if (status == TANNIC_SUCCESS) status = conv_unpitch_rows(p, dtype, rows, y, static_cast<uint32_t>(pixels), pitch, stream);
-    scratch_release(scratch, stream);
+    scratch_release(col, stream);
     return status;
 }
 

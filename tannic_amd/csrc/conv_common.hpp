@@ -29,8 +29,6 @@ int conv2d_gather32(const ConvProblem& p, int dtype, const void* x, const void* 
 int conv2d_unfold(const ConvProblem& p, int dtype, const void* x, const void* w, const void* bias, void* y, hipStream_t stream);
 // few output pixels per image under many channels (fp16, bf16, fp32): the whole batch unfolded side by side, one product
 int conv2d_unfold_batch(const ConvProblem& p, int dtype, const void* x, const void* w, const void* bias, void* y, hipStream_t stream);
-// y[n][o][pix] = rows[(o * N + n) * pitch + pix] for pix < pixels (conv2d_pointwise.hip); dtype float16, bfloat16 or float32
-int conv_unpitch_rows(const ConvProblem& p, int dtype, const void* rows, void* y, uint32_t pixels, uint32_t pitch, hipStream_t stream);
 int conv2d_mfma(const ConvProblem& p, int dtype, const void* x, const void* w, const void* bias, void* y, hipStream_t stream);
 
 }  // namespace th

@@ -65,6 +65,9 @@ int describe_gemm(const tannic_tensor_t* a, const tannic_tensor_t* b, const tann
     p.b_cs = b->strides.sizes[b->rank - 1];
     p.c_rs = c->strides.sizes[c->rank - 2];
     p.row_bias = nullptr;
+    p.c_group = p.c_group_live = 0;
+    p.c_group_stride = 0;
+    p.c_group_div = FastDiv(1);
     p.batch_rank = c->rank - 2;
     p.batches = 1;
     for (int d = 0; d < 6; ++d) {

@@ -21,7 +21,39 @@ struct GemmProblem {
     int64_t a_bs[6], b_bs[6], c_bs[6];
     // optional (MFMA 16-bit kernels only): one value of C's type per row of C, added before rounding
     const void* row_bias;
+    // optional (MFMA f16 / bf16 / fp32 kernels, no batches): the columns of C come in groups of c_group (a multiple of 16
+    // bytes of elements; 0: off).  Column j of group g goes to C + g * c_group_stride + row * c_rs + j when j < c_group_live
+    // and nowhere otherwise; nothing about these addresses needs to be aligned.  (A convolution over a whole batch as one
+    // product: a group is an image, its live columns the image's pixels.)
+    uint32_t c_group, c_group_live;
+    int64_t c_group_stride;
+    FastDiv c_group_div;
 };
+
+// Where the piece of E elements that starts at column `col` (a multiple of E) of row `row` goes, and how many of its elements exist.
+template <class T>
+__device__ inline T* grouped_piece(T* c, const GemmProblem& p, uint32_t row, uint32_t col, int E, uint32_t& live) {
+    uint32_t g, j;
+    p.c_group_div.divmod(col, g, j);
+    live = j >= p.c_group_live ? 0u : p.c_group_live - j < static_cast<uint32_t>(E) ? p.c_group_live - j : static_cast<uint32_t>(E);
+    return c + static_cast<int64_t>(g) * p.c_group_stride + static_cast<int64_t>(row) * p.c_rs + j;
+}
+
+// `live` of the E elements at `bits` (16 bytes) to dst, which may have any alignment
+template <class T>
+__device__ inline void store_piece_anywhere(T* dst, const void* bits, uint32_t live) {
+    constexpr uint32_t E = 16 / sizeof(T);
+    typedef unsigned int uint4_any __attribute__((ext_vector_type(4), aligned(2)));
+    if (live == E) {
+        uint4_any v;
+        __builtin_memcpy(&v, bits, 16);
+        *reinterpret_cast<uint4_any*>(dst) = v;
+    } else {
+        T e[E];
+        __builtin_memcpy(e, bits, 16);
+        for (uint32_t i = 0; i < live; ++i) dst[i] = e[i];
+    }
+}
 
 __host__ __device__ inline void batch_offsets(const GemmProblem& p, uint32_t batch, int64_t& oa, int64_t& ob, int64_t& oc) {
     oa = ob = oc = 0;

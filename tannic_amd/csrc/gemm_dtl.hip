@@ -311,6 +311,20 @@ __global__ __launch_bounds__(256, BLOCKS_PER_CU) void gemm16_dtl_kernel(const T*
     constexpr int PIECES = WN / 8, LANES_PER_ROW = PIECES <= 4 ? 4 : PIECES <= 8 ? 8 : 16, ROWS_PER_PASS = 64 / LANES_PER_ROW;
     static_assert(PIECES <= 16, "a wavefront's block is at most 128 columns wide");
     const uint32_t piece = lane % LANES_PER_ROW, col = n0 + wn + piece * 8;
+    if (p.c_group) {
+        // columns in groups (an image each): the lane's piece belongs to one group, at one place in it, for every row
+        uint32_t live = 0;
+        T* first = piece < PIECES && col < p.N ? grouped_piece(c, p, 0, col, 8, live) : c;
+#pragma unroll
+        for (int r0 = 0; r0 < WM; r0 += ROWS_PER_PASS) {
+            const uint32_t r = r0 + lane / LANES_PER_ROW, row = m0 + wm + r;
+            if (live && row < p.M) {
+                const uint4v bits = *reinterpret_cast<const uint4v*>(stage + r * PITCH + piece * 8);
+                store_piece_anywhere(first + static_cast<int64_t>(row) * p.c_rs, &bits, live);
+            }
+        }
+        return;
+    }
 #pragma unroll
     for (int r0 = 0; r0 < WM; r0 += ROWS_PER_PASS) {
         const uint32_t r = r0 + lane / LANES_PER_ROW, row = m0 + wm + r;
@@ -418,7 +432,8 @@ int gemm16_dtl(const GemmProblem& p, int bm, int bn, const void* a, const void* 
     bool a_t, b_t;
     if (!operands_fit<T>(p, bm, bn, a_t, b_t)) return TANNIC_UNSUPPORTED_DTYPE;
     constexpr int quad = 16 / sizeof(typename DtlTypes<T>::Out);   // results per 16-byte store
-    if (p.N % quad != 0 || p.c_rs % quad != 0 || reinterpret_cast<uintptr_t>(c) % 16 != 0) return TANNIC_UNSUPPORTED_DTYPE;
+    if (p.c_group && (sizeof(T) != 2 || p.N % 8 != 0)) return TANNIC_UNSUPPORTED_DTYPE;   // column groups: 16-bit results, whole pieces of eight
+    if (!p.c_group && (p.N % quad != 0 || p.c_rs % quad != 0 || reinterpret_cast<uintptr_t>(c) % 16 != 0)) return TANNIC_UNSUPPORTED_DTYPE;
     for (int d = 0; d < p.batch_rank; ++d)
         if (p.c_bs[d] % quad != 0) return TANNIC_UNSUPPORTED_DTYPE;
     if constexpr (sizeof(T) == 2) {

@@ -382,6 +382,26 @@ __global__ __launch_bounds__(128 * WAVES_N) void gemm16_kernel(const T* A, const
     if constexpr (sizeof(T) == 4) {
         // four consecutive columns per lane are 16 bytes already
         const bool quads = p.c_rs % 4 == 0 && p.N % 4 == 0 && reinterpret_cast<uintptr_t>(c) % 16 == 0;
+        if (p.c_group) {
+            // columns in groups (an image each): every piece of four finds its own place
+#pragma unroll
+            for (int i = 0; i < TM; ++i) {
+                const uint32_t row = m0 + wm + i * 32 + lane % 32;
+                if (row >= p.M) continue;
+#pragma unroll
+                for (int j = 0; j < TN; ++j)
+#pragma unroll
+                    for (int g = 0; g < 4; ++g) {
+                        const uint32_t col = n0 + wn + j * 32 + g * 8 + 4 * (lane / 32);
+                        if (col >= p.N) continue;
+                        uint32_t live;
+                        T* dst = grouped_piece(c, p, row, col, 4, live);
+                        const float4 four{acc[i][j][g * 4], acc[i][j][g * 4 + 1], acc[i][j][g * 4 + 2], acc[i][j][g * 4 + 3]};
+                        if (live) store_piece_anywhere(dst, &four, live);
+                    }
+            }
+            return;
+        }
 #pragma unroll
         for (int i = 0; i < TM; ++i) {
             const uint32_t row = m0 + wm + i * 32 + lane % 32;
@@ -403,7 +423,7 @@ __global__ __launch_bounds__(128 * WAVES_N) void gemm16_kernel(const T* A, const
         }
         return;
     }
-    const bool vector_ok = p.c_rs % 8 == 0 && p.N % 8 == 0 && reinterpret_cast<uintptr_t>(c) % 16 == 0;
+    const bool vector_ok = p.c_group ? p.N % 8 == 0 : p.c_rs % 8 == 0 && p.N % 8 == 0 && reinterpret_cast<uintptr_t>(c) % 16 == 0;
     if (vector_ok) {
         constexpr int PITCH = WN + 8;                       // elements: rows stay 16-byte aligned and shift by four banks
         T* stage = lds + wave * (WM * PITCH);
@@ -423,6 +443,18 @@ __global__ __launch_bounds__(128 * WAVES_N) void gemm16_kernel(const T* A, const
         // same wavefront reads what it wrote: LDS operations of a wavefront complete in order
         constexpr int LANES_PER_ROW = WN / 8, ROWS_PER_PASS = 64 / LANES_PER_ROW;
         const uint32_t col = n0 + wn + (lane % LANES_PER_ROW) * 8;
+        if (p.c_group) {
+            // columns in groups (an image each): the lane's piece belongs to one group, at one place in it, for every row
+            uint32_t live = 0;
+            T* first = col < p.N ? grouped_piece(c, p, 0, col, 8, live) : c;
+#pragma unroll
+            for (int r0 = 0; r0 < WM; r0 += ROWS_PER_PASS) {
+                const uint32_t r = r0 + lane / LANES_PER_ROW, row = m0 + wm + r;
+                const uint4v bits = *reinterpret_cast<const uint4v*>(stage + r * PITCH + (lane % LANES_PER_ROW) * 8);
+                if (live && row < p.M) store_piece_anywhere(first + static_cast<int64_t>(row) * p.c_rs, &bits, live);
+            }
+            return;
+        }
 #pragma unroll
         for (int r0 = 0; r0 < WM; r0 += ROWS_PER_PASS) {
             const uint32_t r = r0 + lane / LANES_PER_ROW, row = m0 + wm + r;
@@ -438,7 +470,7 @@ __global__ __launch_bounds__(128 * WAVES_N) void gemm16_kernel(const T* A, const
 #pragma unroll
                 for (int v = 0; v < 16; ++v) {
                     const uint32_t col = n0 + wn + j * 32 + 8 * (v / 4) + 4 * (lane / 32) + v % 4;
-                    if (row < p.M && col < p.N) c[static_cast<int64_t>(row) * p.c_rs + col] = narrow_result<T>(acc[i][j][v]);
+                    if (row < p.M && col < p.N) c[static_cast<int64_t>(row) * p.c_rs + col] = narrow_result<T>(acc[i][j][v]);   // (never with column groups: their N is whole pieces)
                 }
         }
     }
@@ -492,6 +524,12 @@ __global__ __launch_bounds__(256) void gemm_split_reduce_kernel(const float* par
     int64_t oa, ob, oc;
     batch_offsets(p, batch, oa, ob, oc);
     T* dst = C + oc + static_cast<int64_t>(m) * p.c_rs + col;
+    if (p.c_group) {
+        uint32_t there;
+        dst = grouped_piece(C, p, m, col, 4, there);
+        for (uint32_t e = 0; e < there; ++e) dst[e] = narrow_result<T>(sum[e]);
+        return;
+    }
     if (live == 4 && reinterpret_cast<uintptr_t>(dst) % (4 * sizeof(T)) == 0) {
         T out[4];
 #pragma unroll

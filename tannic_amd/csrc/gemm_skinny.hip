@@ -261,7 +261,7 @@ static int launch_stream(const GemmProblem& p, const void* a, const void* b, voi
 
 template <class T>
 int run_skinny(const GemmProblem& p, const void* a, const void* b, void* c, hipStream_t stream) {
-    if (p.M == 0 || p.M > 32 || p.N == 0 || p.K == 0 || p.batches == 0 || p.batches > 65535 || p.row_bias) return TANNIC_UNSUPPORTED_DTYPE;
+    if (p.M == 0 || p.M > 32 || p.N == 0 || p.K == 0 || p.batches == 0 || p.batches > 65535 || p.row_bias || p.c_group) return TANNIC_UNSUPPORTED_DTYPE;
     // both operands K-contiguous; 16-byte chunks along K
     if (p.a_cs != 1 || p.b_rs != 1) return TANNIC_UNSUPPORTED_DTYPE;
     auto mult8 = [](int64_t v) { return v % 8 == 0; };
