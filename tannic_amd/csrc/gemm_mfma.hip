@@ -46,9 +46,9 @@ struct Operand {
 // touches the loaded values (and waits for them) early.
 // Both loaders expose their work as single memory operations (fetch_one /
 // commit_one) so that the main loop can spread them between MFMAs.
-// ALIGNED = false: the operand's address, leading dimension or K is not a multiple of 16 bytes, so a chunk is gathered
-// element by element (each element checked against K, rows past K's end of a chunk read as zero) - eight loads where
-// the aligned loader issues one, which still leaves the product on the matrix cores.
+// ALIGNED = false: the operand's address, leading dimension or K is not a multiple of 16 bytes.  A chunk that lies inside
+// K is still one 16-byte load, at an address that is a multiple of the element size only; the chunk that straddles K's
+// end is gathered element by element (each checked against K; what lies past it reads as zero).
 template <class T, int ROWS, int THREADS, bool ALIGNED = true>
 struct KMajorLoader {
     static constexpr int ROWS_PER_PASS = THREADS / 8;
@@ -71,10 +71,16 @@ struct KMajorLoader {
         } else {
             using U = std::conditional_t<sizeof(T) == 2, uint16_t, uint32_t>;
             const U* from = reinterpret_cast<const U*>(base + static_cast<int64_t>(srow) * op.row_stride);
-            U piece[kChunkOf<T>];
+            if (k_left >= static_cast<uint32_t>(kChunkOf<T>)) {
+                // the whole chunk lies inside K: one 16-byte load at whatever address that is (the hardware splits what it must)
+                typedef unsigned int uint4_any __attribute__((ext_vector_type(4), aligned(2)));
+                regs[i] = *reinterpret_cast<const uint4_any*>(from);
+            } else {
+                U piece[kChunkOf<T>];
 #pragma unroll
-            for (int e = 0; e < kChunkOf<T>; ++e) piece[e] = static_cast<uint32_t>(e) < k_left ? from[e] : U(0);
-            __builtin_memcpy(&regs[i], piece, 16);
+                for (int e = 0; e < kChunkOf<T>; ++e) piece[e] = static_cast<uint32_t>(e) < k_left ? from[e] : U(0);
+                __builtin_memcpy(&regs[i], piece, 16);
+            }
         }
     }
     template <bool MASK>
@@ -369,10 +375,10 @@ __global__ __launch_bounds__(128 * WAVES_N) void gemm16_kernel(const T* A, const
                     const uint32_t col = n0 + wn + j * 32 + g * 8 + 4 * (lane / 32);
                     if (quads) {
                         if (col < p.N) *reinterpret_cast<float4*>(rp + col) = float4{acc[i][j][g * 4], acc[i][j][g * 4 + 1], acc[i][j][g * 4 + 2], acc[i][j][g * 4 + 3]};
-                    } else {
-#pragma unroll
-                        for (int e = 0; e < 4; ++e)
-                            if (col + e < p.N) rp[col + e] = acc[i][j][g * 4 + e];
+                    } else if (col < p.N) {
+                        // rows that start anywhere, or end inside a piece: 16 bytes at whatever address, the last piece element by element
+                        const float4 four{acc[i][j][g * 4], acc[i][j][g * 4 + 1], acc[i][j][g * 4 + 2], acc[i][j][g * 4 + 3]};
+                        store_piece_anywhere(rp + col, &four, p.N - col < 4 ? p.N - col : 4u);
                     }
                 }
         }
@@ -414,17 +420,19 @@ __global__ __launch_bounds__(128 * WAVES_N) void gemm16_kernel(const T* A, const
                     const uint32_t col = n0 + wn + j * 32 + g * 8 + 4 * (lane / 32);
                     if (quads) {
                         if (col < p.N) *reinterpret_cast<float4*>(rp + col) = float4{acc[i][j][g * 4], acc[i][j][g * 4 + 1], acc[i][j][g * 4 + 2], acc[i][j][g * 4 + 3]};
-                    } else {
-#pragma unroll
-                        for (int e = 0; e < 4; ++e)
-                            if (col + e < p.N) rp[col + e] = acc[i][j][g * 4 + e];
+                    } else if (col < p.N) {
+                        const float4 four{acc[i][j][g * 4], acc[i][j][g * 4 + 1], acc[i][j][g * 4 + 2], acc[i][j][g * 4 + 3]};
+                        store_piece_anywhere(rp + col, &four, p.N - col < 4 ? p.N - col : 4u);
                     }
                 }
         }
         return;
     }
-    const bool vector_ok = p.c_group ? p.N % 8 == 0 : p.c_rs % 8 == 0 && p.N % 8 == 0 && reinterpret_cast<uintptr_t>(c) % 16 == 0;
-    if (vector_ok) {
+    // Rounded into LDS (each wavefront its own block) and written as pieces of 16 bytes: aligned stores when every row of C
+    // starts at a multiple of 16 bytes and is whole pieces long, otherwise stores at whatever address a piece has (the last
+    // piece of a row element by element): a result whose rows are 4098 long no longer costs 80 % more than one of 4096.
+    const bool aligned_rows = p.c_rs % 8 == 0 && p.N % 8 == 0 && reinterpret_cast<uintptr_t>(c) % 16 == 0;
+    {
         constexpr int PITCH = WN + 8;                       // elements: rows stay 16-byte aligned and shift by four banks
         T* stage = lds + wave * (WM * PITCH);
 #pragma unroll
@@ -455,23 +463,21 @@ __global__ __launch_bounds__(128 * WAVES_N) void gemm16_kernel(const T* A, const
             }
             return;
         }
+        if (!aligned_rows) {
+            const uint32_t live = col >= p.N ? 0u : p.N - col < 8 ? p.N - col : 8u;
+#pragma unroll
+            for (int r0 = 0; r0 < WM; r0 += ROWS_PER_PASS) {
+                const uint32_t r = r0 + lane / LANES_PER_ROW, row = m0 + wm + r;
+                const uint4v bits = *reinterpret_cast<const uint4v*>(stage + r * PITCH + (lane % LANES_PER_ROW) * 8);
+                if (live && row < p.M) store_piece_anywhere(c + static_cast<int64_t>(row) * p.c_rs + col, &bits, live);
+            }
+            return;
+        }
 #pragma unroll
         for (int r0 = 0; r0 < WM; r0 += ROWS_PER_PASS) {
             const uint32_t r = r0 + lane / LANES_PER_ROW, row = m0 + wm + r;
             const uint4v bits = *reinterpret_cast<const uint4v*>(stage + r * PITCH + (lane % LANES_PER_ROW) * 8);
             if (row < p.M && col < p.N) *reinterpret_cast<uint4v*>(c + static_cast<int64_t>(row) * p.c_rs + col) = bits;
-        }
-    } else {
-#pragma unroll
-        for (int i = 0; i < TM; ++i) {
-            const uint32_t row = m0 + wm + i * 32 + lane % 32;
-#pragma unroll
-            for (int j = 0; j < TN; ++j)
-#pragma unroll
-                for (int v = 0; v < 16; ++v) {
-                    const uint32_t col = n0 + wn + j * 32 + 8 * (v / 4) + 4 * (lane / 32) + v % 4;
-                    if (row < p.M && col < p.N) c[static_cast<int64_t>(row) * p.c_rs + col] = narrow_result<T>(acc[i][j][v]);   // (never with column groups: their N is whole pieces)
-                }
         }
     }
 }
