@@ -39,6 +39,24 @@ struct Operand {
 };
 
 
+typedef unsigned int uint4_any __attribute__((ext_vector_type(4), aligned(2)));
+// The piece of 16 bytes that starts at element `first` of a run of `extent` elements at `run`, which may lie at any
+// address: one load when the whole piece lies inside the run, else element by element, with zero for what lies past the end.
+template <class T>
+__device__ inline uint4v piece_of_run(const T* run, uint32_t first, uint32_t extent) {
+    constexpr uint32_t E = 16 / sizeof(T);
+    using U = std::conditional_t<sizeof(T) == 2, uint16_t, uint32_t>;
+    const U* from = reinterpret_cast<const U*>(run) + first;
+    if (first + E <= extent) return *reinterpret_cast<const uint4_any*>(from);
+    U piece[E];
+#pragma unroll
+    for (uint32_t e = 0; e < E; ++e) piece[e] = first + e < extent ? from[e] : U(0);
+    uint4v out;
+    __builtin_memcpy(&out, piece, 16);
+    return out;
+}
+
+
 // ---- global -> registers -> LDS, operand contiguous along K -------------------
 // Rows past the operand's end read a clamped (valid) address: they only feed
 // rows/columns of C that are never stored.  K past the end must contribute
@@ -73,7 +91,6 @@ struct KMajorLoader {
             const U* from = reinterpret_cast<const U*>(base + static_cast<int64_t>(srow) * op.row_stride);
             if (k_left >= static_cast<uint32_t>(kChunkOf<T>)) {
                 // the whole chunk lies inside K: one 16-byte load at whatever address that is (the hardware splits what it must)
-                typedef unsigned int uint4_any __attribute__((ext_vector_type(4), aligned(2)));
                 regs[i] = *reinterpret_cast<const uint4_any*>(from);
             } else {
                 U piece[kChunkOf<T>];
@@ -96,7 +113,8 @@ struct KMajorLoader {
 };
 
 // ---- fp32 operand contiguous along its row index: E x E micro-blocks (E elements per 16 bytes), transposed ----
-template <class T, int ROWS, int THREADS>
+// ALIGNED = false: as for the loader above, with the operand's rows in the place of K.
+template <class T, int ROWS, int THREADS, bool ALIGNED = true>
 struct RowMajorLoader {
     static constexpr int E = kChunkOf<T>;
     using U = std::conditional_t<sizeof(T) == 2, uint16_t, uint32_t>;
@@ -118,7 +136,9 @@ struct RowMajorLoader {
         const uint32_t row = row0 + rb * E;
         const uint32_t srow = (rb < ROWS / E && row < op.rows) ? row : 0;
         const uint32_t k = kfirst + kk;
-        regs[i][kk] = *reinterpret_cast<const uint4v*>(static_cast<const T*>(op.base) + static_cast<int64_t>(k < K_ ? k : 0) * op.k_stride + srow);
+        const T* run = static_cast<const T*>(op.base) + static_cast<int64_t>(k < K_ ? k : 0) * op.k_stride;
+        if constexpr (ALIGNED) regs[i][kk] = *reinterpret_cast<const uint4v*>(run + srow);
+        else regs[i][kk] = piece_of_run<T>(run, srow, op.rows);
     }
     template <bool MASK>
     __device__ inline void commit_one(int idx, T* tile) const {
@@ -150,7 +170,8 @@ struct RowMajorLoader {
 // of the four pointers with q = i / 4 - that is, pointed at k-row e and rows 4q..4q+3, it returns to lane i four
 // consecutive k of row i.  Two such reads make the 8 k of a lane's MFMA fragment.  The 64 bytes added to the pitch put
 // the four k-rows that 32 lanes read together on different banks.
-template <class T, int ROWS, int THREADS>
+// ALIGNED = false: as for the loaders above.
+template <class T, int ROWS, int THREADS, bool ALIGNED = true>
 struct AsIsLoader {
     static constexpr int PITCH = ROWS + 32;
     static constexpr int CHUNKS = ROWS / 8;                    // 16-byte chunks per k-row
@@ -161,7 +182,9 @@ struct AsIsLoader {
     __device__ inline void begin_fetch(const Operand&, uint32_t k0, uint32_t K) { k0_ = k0; K_ = K; }
     __device__ inline void fetch_one(int i, const Operand& op, uint32_t row0) {
         const uint32_t id = threadIdx.x + THREADS * i, k = k0_ + id / CHUNKS, row = row0 + (id % CHUNKS) * 8;
-        regs[i] = *reinterpret_cast<const uint4v*>(static_cast<const T*>(op.base) + static_cast<int64_t>(k < K_ ? k : 0) * op.k_stride + (row < op.rows ? row : 0));
+        const T* run = static_cast<const T*>(op.base) + static_cast<int64_t>(k < K_ ? k : 0) * op.k_stride;
+        if constexpr (ALIGNED) regs[i] = *reinterpret_cast<const uint4v*>(run + (row < op.rows ? row : 0));
+        else regs[i] = piece_of_run<T>(run, row < op.rows ? row : 0, op.rows);
     }
     template <bool MASK>
     __device__ inline void commit_one(int i, T* tile) const {
@@ -192,7 +215,7 @@ template <class T, int ROWS, bool K_MAJOR> constexpr uint32_t kTileElements = kA
 
 template <class T, int ROWS, int THREADS, bool K_MAJOR, bool ALIGNED = true>
 using Loader = std::conditional_t<K_MAJOR, KMajorLoader<T, ROWS, THREADS, ALIGNED>,
-                                  std::conditional_t<sizeof(T) == 2, AsIsLoader<T, ROWS, THREADS>, RowMajorLoader<T, ROWS, THREADS>>>;
+                                  std::conditional_t<sizeof(T) == 2, AsIsLoader<T, ROWS, THREADS, ALIGNED>, RowMajorLoader<T, ROWS, THREADS, ALIGNED>>>;
 
 // WAVES_N: wavefronts along N (2 -> 256 threads, one wavefront per SIMD; 4 -> 512 threads, two per SIMD, so that
 // one wavefront's waits are covered by the other's MFMAs); always two wavefronts along M.
@@ -611,11 +634,17 @@ int run16(const GemmProblem& p, const void* a, const void* b, void* c, hipStream
     for (int d = 0; d < p.batch_rank; ++d) aligned = aligned && mult8(p.a_bs[d]) && mult8(p.b_bs[d]);
     if (p.batches > 65535) return TANNIC_UNSUPPORTED_DTYPE;
     if (!aligned) {
-        // Both operands K-contiguous (a linear layer whose width or row pitch is odd): the tiles are gathered element by
-        // element and the product stays on the matrix cores.  Other layouts take the scalar kernel.
-        if (!(ak && bk) || p.row_bias) return TANNIC_UNSUPPORTED_DTYPE;
-        if (p.M > 64) return launch16<T, 128, 128, 2, true, true, false, false>(p, a, b, c, stream);
-        return launch16<T, 64, 128, 2, true, true, false, false>(p, a, b, c, stream);
+        // An extent, a row pitch or an address that is odd: the loaders fetch their 16-byte pieces at whatever address they
+        // lie (only the piece that straddles the end of a row is gathered element by element) and the product stays on the
+        // matrix cores.
+        if (p.row_bias) return TANNIC_UNSUPPORTED_DTYPE;
+        if (ak && bk) {
+            if (p.M > 64) return launch16<T, 128, 128, 2, true, true, false, false>(p, a, b, c, stream);
+            return launch16<T, 64, 128, 2, true, true, false, false>(p, a, b, c, stream);
+        }
+        if (ak) return launch16<T, 128, 128, 2, true, false, false, false>(p, a, b, c, stream);
+        if (bk) return launch16<T, 128, 128, 2, false, true, false, false>(p, a, b, c, stream);
+        return launch16<T, 128, 128, 2, false, false, false, false>(p, a, b, c, stream);
     }
     // Tile height by M (a tile taller than M multiplies padding).  Large tiles when they give (nearly) every compute unit one.  Tile width: 256 unless a narrower one needs less time
     // for its rounds over the 256 compute units (2048 x 14336: 448 tiles 256 wide are two rounds, the second three

@@ -59,6 +59,15 @@ LAYOUTS = {
     "nt_odd_k": ((130, 75), (190, 75), [], [("transpose", (-1, -2))]),
     "nt_odd_pitch_and_start": ((130, 77), (190, 79), [("index", (slice(None), slice(1, 73)))], [("index", (slice(None), slice(3, 75))), ("transpose", (-1, -2))]),
     "nt_odd_k_few_rows_batched": ((3, 40, 203), (3, 150, 203), [], [("transpose", (-1, -2))]),
+    # the same for operands contiguous along M / N: odd extents, odd pitches, views that start at odd columns, fewer rows than
+    # a 16-byte piece holds, odd batch strides, and tiles on every side of a 128 x 128 grid
+    "nn_odd_extents": ((131, 75), (75, 197), [], []),
+    "nn_odd_pitch_and_start": ((131, 75), (75, 203), [], [("index", (slice(None), slice(3, 200)))]),
+    "tn_odd_pitch_and_start": ((77, 141), (77, 203), [("index", (slice(None), slice(1, 132))), ("transpose", (-1, -2))], [("index", (slice(None), slice(3, 200)))]),
+    "tt_odd_extents": ((75, 131), (197, 75), [("transpose", (-1, -2))], [("transpose", (-1, -2))]),
+    "tn_three_rows": ((200, 3), (200, 5), [("transpose", (-1, -2))], []),
+    "nn_odd_batched": ((3, 41, 203), (3, 203, 151), [], []),
+    "tn_odd_tiles": ((70, 259), (70, 385), [("transpose", (-1, -2))], []),
     # both operands K-contiguous, whole K steps, 200 large tiles: the tiles filled by direct global -> LDS loads
     # (rows past the end of both operands; one, two and three K steps)
     "nt_direct_one_step": ((50, 264, 64), (50, 264, 64), [], [("transpose", (-1, -2))]),
