@@ -193,7 +193,15 @@ template <class... Ts> inline bool have_storage(const Ts*... t) {
 // q = n / d for n < 2^31 with one multiply-high, one add and one shift.
 struct FastDiv {
     uint32_t d, magic, shift;
-    FastDiv() : d(1), magic(1), shift(0) {}
+    __host__ __device__ FastDiv() : d(1), magic(1), shift(0) {}
+    // the divisor 2^31: every n below it has quotient 0 and remainder n
+    __host__ __device__ static FastDiv beyond_all() {
+        FastDiv f;
+        f.d = 1u << 31;
+        f.magic = 1;
+        f.shift = 31;
+        return f;
+    }
     // (a divisor of 0 only comes from an empty index space, where nothing is ever divided: it is taken as 1)
     explicit FastDiv(uint32_t divisor) : d(divisor ? divisor : 1) {
         for (shift = 0; shift < 32; ++shift)

@@ -42,11 +42,12 @@ __global__ __launch_bounds__(256) void conv_subsample4_kernel(const T* x, T* out
     *reinterpret_cast<Quad*>(out + static_cast<int64_t>(row) * p.WO + quad * 4) = bits;
 }
 
-// Pixel counts that are not a multiple of 16 bytes (14 x 14, 7 x 7 ...): the product wants its rows of pixels to start at
-// multiples of 16 bytes, so the sampled pixels of every (image, channel) go to rows of `pitch` elements (the count rounded
-// up; the rest zeros), channel by channel with the images side by side, so that ONE product O x C . C x (N * pitch) does the
-// whole batch on whole tiles (a product per image would have 200 or 56 columns); the product stores its columns image by
-// image (GemmProblem::c_group), straight into y.
+// Pixel counts that are not a multiple of 16 bytes (14 x 14, 7 x 7 ...): ONE product O x C . C x (N * pitch), pitch the
+// count rounded up to 16 bytes, does the whole batch on whole tiles (a product per image would have 200 or 56 columns) and
+// stores its columns image by image (GemmProblem::c_group), straight into y.  Without a stride it also reads the images
+// where they lie (GemmProblem::b_group_stride).  With one, or when a channel's pixels are not one run of memory, the
+// sampled pixels of every (image, channel) first go to rows of `pitch` elements (the rest zeros), channel by channel with
+// the images side by side:
 // out[(c * N + n) * pitch + pix] = x[n][c][oh * stride_h][ow * stride_w], pix = oh * WO + ow; 16 bytes per thread.
 template <class T, bool PLANE>
 __global__ __launch_bounds__(256) void conv_repitch_kernel(const T* x, T* out, ConvProblem p, uint32_t pixels, uint32_t pitch, FastDiv div_groups, FastDiv div_c,
@@ -120,10 +121,34 @@ int run_pointwise(const ConvProblem& p, int dtype, const void* x, const void* w,
         const uint32_t pitch = static_cast<uint32_t>((pixels + E - 1) / E * E), groups = pitch / E;
         const uint64_t in_rows = static_cast<uint64_t>(p.N) * p.C, out_rows = static_cast<uint64_t>(p.N) * p.O;
         if (in_rows * groups >= (1ull << 31) || out_rows * groups >= (1ull << 31) || static_cast<uint64_t>(p.N) * pitch >= (1ull << 31)) return TANNIC_UNSUPPORTED_DTYPE;
+        const bool plane = dense && p.xs[3] == 1 && p.xs[2] == static_cast<int64_t>(p.W) && reinterpret_cast<uintptr_t>(x) % sizeof(T) == 0;
+        const uint64_t columns = static_cast<uint64_t>(p.N) * pitch;
+        // one product O x C . C x (N * pitch) for the whole batch; the columns of image n go to y[n], rows p.ys[1] apart
+        g.N = static_cast<uint32_t>(columns);
+        g.batch_rank = 0;
+        g.batches = 1;
+        g.batch_extent[0] = 1;
+        g.b_bs[0] = g.c_bs[0] = 0;
+        g.c_rs = p.ys[1];
+        g.c_group = pitch;
+        g.c_group_live = static_cast<uint32_t>(pixels);
+        g.c_group_stride = p.ys[0];
+        g.c_group_div = FastDiv(pitch);
+        if (plane && p.C <= 256) {
+            // The pixels of a channel are one run of memory and there are few channels: the product reads the images where
+            // they lie, its loaders taking 16-byte pieces at whatever address they start.  (Those loads are slower than
+            // aligned ones and the kernel that knows them walks all of K in one block; batch 32, fp16: 256 -> 1024 over
+            // 14 x 14 16.6 against 18.4 us through re-pitched rows, but 1024 -> 256 28 against 22 us, 2048 -> 512 over
+            // 7 x 7 53 against 26 us.)
+            g.b_rs = p.xs[1];
+            g.b_group_stride = p.xs[0];
+            const int direct = product<T>(g, dtype, w, x, y, stream);
+            if (direct != TANNIC_UNSUPPORTED_DTYPE) return direct;
+            g.b_group_stride = 0;
+        }
         T* dense_x = nullptr;
         if (scratch_acquire(reinterpret_cast<void**>(&dense_x), in_rows * pitch * sizeof(T), stream) != TANNIC_SUCCESS) return TANNIC_ERROR;
         const uint32_t total_in = static_cast<uint32_t>(in_rows * groups);
-        const bool plane = dense && p.xs[3] == 1 && p.xs[2] == static_cast<int64_t>(p.W) && reinterpret_cast<uintptr_t>(x) % sizeof(T) == 0;
         if (plane)
             hipLaunchKernelGGL((conv_repitch_kernel<T, true>), dim3((total_in + 255) / 256), dim3(256), 0, stream, static_cast<const T*>(x), dense_x, p,
                                static_cast<uint32_t>(pixels), pitch, FastDiv(groups), FastDiv(p.C), FastDiv(p.WO), total_in);
@@ -132,19 +157,7 @@ int run_pointwise(const ConvProblem& p, int dtype, const void* x, const void* w,
                                static_cast<uint32_t>(pixels), pitch, FastDiv(groups), FastDiv(p.C), FastDiv(p.WO), total_in);
         int status = launch_status("conv_repitch_kernel");
         if (status == TANNIC_SUCCESS) {
-            const uint64_t columns = static_cast<uint64_t>(p.N) * pitch;
-            g.N = static_cast<uint32_t>(columns);
             g.b_rs = static_cast<int64_t>(columns);
-            g.batch_rank = 0;
-            g.batches = 1;
-            g.batch_extent[0] = 1;
-            g.b_bs[0] = g.c_bs[0] = 0;
-            // the columns of image n go to y[n]: rows p.ys[1] apart, images p.ys[0]
-            g.c_rs = p.ys[1];
-            g.c_group = pitch;
-            g.c_group_live = static_cast<uint32_t>(pixels);
-            g.c_group_stride = p.ys[0];
-            g.c_group_div = FastDiv(pitch);
             status = product<T>(g, dtype, w, dense_x, y, stream);
             if (status == TANNIC_UNSUPPORTED_DTYPE) {
                 set_error_text("conv2d: internal: the 1x1 product refused a problem its caller had checked");

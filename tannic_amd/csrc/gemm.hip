@@ -66,7 +66,7 @@ int describe_gemm(const tannic_tensor_t* a, const tannic_tensor_t* b, const tann
     p.c_rs = c->strides.sizes[c->rank - 2];
     p.row_bias = nullptr;
     p.c_group = p.c_group_live = 0;
-    p.c_group_stride = 0;
+    p.c_group_stride = p.b_group_stride = 0;
     p.c_group_div = FastDiv(1);
     p.batch_rank = c->rank - 2;
     p.batches = 1;

@@ -28,6 +28,10 @@ struct GemmProblem {
     uint32_t c_group, c_group_live;
     int64_t c_group_stride;
     FastDiv c_group_div;
+    // optional, with c_group and B contiguous along n (b_cs == 1): B's columns lie in the same groups, element (k, j) of
+    // group g at B + g * b_group_stride + k * b_rs + j for j < c_group_live, at any alignment; the other columns of a group
+    // read as zero (0: off).  (The same convolution reading its images where they lie.)
+    int64_t b_group_stride;
 };
 
 // Where the piece of E elements that starts at column `col` (a multiple of E) of row `row` goes, and how many of its elements exist.

@@ -36,6 +36,12 @@ struct Operand {
     const void* base;
     int64_t row_stride, k_stride;
     uint32_t rows;  // M for A, N for B
+    // Rows in groups that lie apart (only the loaders for rows that are contiguous in memory, in their mode for any
+    // alignment, look at this): row r is element r % group of group r / group, which exists when it is below group_live,
+    // and a group starts group_stride elements after the one before.  Plain rows: one group that holds them all.
+    FastDiv group;
+    uint32_t group_live;
+    int64_t group_stride;
 };
 
 
@@ -137,8 +143,13 @@ struct RowMajorLoader {
         const uint32_t srow = (rb < ROWS / E && row < op.rows) ? row : 0;
         const uint32_t k = kfirst + kk;
         const T* run = static_cast<const T*>(op.base) + static_cast<int64_t>(k < K_ ? k : 0) * op.k_stride;
-        if constexpr (ALIGNED) regs[i][kk] = *reinterpret_cast<const uint4v*>(run + srow);
-        else regs[i][kk] = piece_of_run<T>(run, srow, op.rows);
+        if constexpr (ALIGNED) {
+            regs[i][kk] = *reinterpret_cast<const uint4v*>(run + srow);
+        } else {
+            uint32_t g, j;
+            op.group.divmod(srow, g, j);
+            regs[i][kk] = piece_of_run<T>(run + static_cast<int64_t>(g) * op.group_stride, j, op.group_live);
+        }
     }
     template <bool MASK>
     __device__ inline void commit_one(int idx, T* tile) const {
@@ -183,8 +194,13 @@ struct AsIsLoader {
     __device__ inline void fetch_one(int i, const Operand& op, uint32_t row0) {
         const uint32_t id = threadIdx.x + THREADS * i, k = k0_ + id / CHUNKS, row = row0 + (id % CHUNKS) * 8;
         const T* run = static_cast<const T*>(op.base) + static_cast<int64_t>(k < K_ ? k : 0) * op.k_stride;
-        if constexpr (ALIGNED) regs[i] = *reinterpret_cast<const uint4v*>(run + (row < op.rows ? row : 0));
-        else regs[i] = piece_of_run<T>(run, row < op.rows ? row : 0, op.rows);
+        if constexpr (ALIGNED) {
+            regs[i] = *reinterpret_cast<const uint4v*>(run + (row < op.rows ? row : 0));
+        } else {
+            uint32_t g, j;
+            op.group.divmod(row < op.rows ? row : 0, g, j);
+            regs[i] = piece_of_run<T>(run + static_cast<int64_t>(g) * op.group_stride, j, op.group_live);
+        }
     }
     template <bool MASK>
     __device__ inline void commit_one(int i, T* tile) const {
@@ -241,8 +257,11 @@ __global__ __launch_bounds__(128 * WAVES_N) void gemm16_kernel(const T* A, const
     // this block's range of K: all of it, or its share
     const uint32_t k_first = SPLIT ? split * sk.k_chunk : 0;
     const uint32_t K = SPLIT ? (p.K - k_first < sk.k_chunk ? p.K - k_first : sk.k_chunk) : p.K;
-    const Operand opA{A + oa + static_cast<int64_t>(k_first) * p.a_cs, p.a_rs, p.a_cs, p.M};
-    const Operand opB{B + ob + static_cast<int64_t>(k_first) * p.b_rs, p.b_cs, p.b_rs, p.N};   // rows of B's operand are the columns n
+    const FastDiv one_group = FastDiv::beyond_all();
+    const Operand opA{A + oa + static_cast<int64_t>(k_first) * p.a_cs, p.a_rs, p.a_cs, p.M, one_group, p.M, 0};
+    // rows of B's operand are the columns n
+    const Operand opB{B + ob + static_cast<int64_t>(k_first) * p.b_rs, p.b_cs, p.b_rs, p.N, p.b_group_stride ? p.c_group_div : one_group,
+                      p.b_group_stride ? p.c_group_live : p.N, p.b_group_stride};
     const uint32_t m0 = tm * BM, n0 = tn * BN;
 
     const int wave = threadIdx.x / 64, lane = threadIdx.x % 64;
@@ -633,6 +652,13 @@ int run16(const GemmProblem& p, const void* a, const void* b, void* c, hipStream
     aligned = aligned && mult8(ak ? p.a_rs : p.a_cs) && mult8(bk ? p.b_cs : p.b_rs) && mult8(ak ? p.K : p.M) && mult8(bk ? p.K : p.N);
     for (int d = 0; d < p.batch_rank; ++d) aligned = aligned && mult8(p.a_bs[d]) && mult8(p.b_bs[d]);
     if (p.batches > 65535) return TANNIC_UNSUPPORTED_DTYPE;
+    if (p.b_group_stride) {
+        // B's columns in groups: the loaders for any alignment know about them; A is a parameter matrix, K-contiguous
+        if (!p.c_group || bk || !ak || p.batches != 1) return TANNIC_UNSUPPORTED_DTYPE;
+        const uint64_t tiles128 = static_cast<uint64_t>((p.M + 127) / 128) * ((p.N + 127) / 128);
+        if (p.M > 64 && tiles128 >= 200) return launch16<T, 128, 128, 2, true, false, false, false>(p, a, b, c, stream);
+        return launch16<T, 64, 128, 2, true, false, false, false>(p, a, b, c, stream);
+    }
     if (!aligned) {
         // An extent, a row pitch or an address that is odd: the loaders fetch their 16-byte pieces at whatever address they
         // lie (only the piece that straddles the end of a row is gathered element by element) and the product stays on the

@@ -90,6 +90,13 @@ CASES = {
     "k1_s2_14_to_7": ((2, 128, 14, 14), (72, 128, 1, 1), (2, 2), (0, 0)),
     "k1_5x9": ((2, 64, 5, 9), (24, 64, 1, 1), (1, 1), (0, 0)),
     "k1_s2x1_to_5x11": ((1, 64, 9, 11), (16, 64, 1, 1), (2, 1), (0, 0)),
+    # ... and, without a stride, reads the images where they lie: one pixel, fewer pixels than a piece holds, a group that
+    # straddles tiles of 128 columns (200 per image), many output channels, one output channel, a short K
+    "k1_one_pixel": ((9, 64, 1, 1), (24, 64, 1, 1), (1, 1), (0, 0)),
+    "k1_3x1": ((4, 128, 3, 1), (200, 128, 1, 1), (1, 1), (0, 0)),
+    "k1_14x14_many_images": ((7, 64, 14, 14), (136, 64, 1, 1), (1, 1), (0, 0)),
+    "k1_7x7_one_channel_out": ((5, 72, 7, 7), (1, 72, 1, 1), (1, 1), (0, 0)),
+    "k1_13x13_c8": ((3, 8, 13, 13), (520, 8, 1, 1), (1, 1), (0, 0)),
     # few output pixels per image under a long K: the whole batch unfolded side by side, one product
     "unfolded_k3_7x7": ((5, 128, 7, 7), (40, 128, 3, 3), (1, 1), (1, 1)),
     "unfolded_k3_s2_14_to_7": ((6, 64, 14, 14), (48, 64, 3, 3), (2, 2), (1, 1)),
@@ -160,6 +167,19 @@ def test_channel_slice_of_a_larger_signal(device, dtype):
         want = ops.convolve2d(hx[:, 3:35], hw, None, 1, 1).numpy()
         got = ops.convolve2d(dx[:, 3:35], dw, None, 1, 1).numpy()
         support.assert_close(got, want, 2e-3 if dtype is ta.float16 else 2.0 ** -7, 1e-3, f"channel slice, width {width}")
+
+
+@pytest.mark.parametrize("dtype", [ta.float16, ta.bfloat16, ta.float32], ids=str)
+def test_pointwise_over_a_channel_slice_with_odd_pixel_counts(device, dtype):
+    """A 1x1 kernel over channels 5..68 of a [3, 80, 7, 7] signal with a bias: every plane starts at an odd multiple of 49
+    elements and an image is 80 planes long, so no row of the product starts at a multiple of 16 bytes."""
+    hx, dx = support.both(support.values_for(dtype, SEED, 8, (3, 80, 7, 7), -2, 2), dtype, device)
+    hw, dw = support.both(support.values_for(dtype, SEED, 9, (40, 64, 1, 1), -0.2, 0.2), dtype, device)
+    hb, db = support.both(support.values_for(dtype, SEED, 10, (40,), -1, 1), dtype, device)
+    want = ops.convolve2d(hx[:, 5:69], hw, hb, 1, 0).numpy()
+    got = ops.convolve2d(dx[:, 5:69], dw, db, 1, 0).numpy()
+    if dtype is ta.float32: support.assert_close(got, want, 1e-5, 64 * 2.0 ** -24 * 4, "pointwise over a channel slice")
+    else: support.assert_close(got, want, 2e-3 if dtype is ta.float16 else 2.0 ** -7, 1e-3, "pointwise over a channel slice")
 
 
 def test_status_codes(device):
