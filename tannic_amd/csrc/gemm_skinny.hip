@@ -1,4 +1,4 @@
-// Matrix product with very few rows (M <= 32), 16-bit types: y = x * W^T as the
+// Matrix product with very few rows (M <= 32; up to 64 over a small W), 16-bit types: y = x * W^T as the
 // decoding step of a transformer runs it.  The work is reading W once; there is
 // nothing to reuse, so nothing goes through LDS on the way in.
 //
@@ -261,7 +261,7 @@ static int launch_stream(const GemmProblem& p, const void* a, const void* b, voi
 
 template <class T>
 int run_skinny(const GemmProblem& p, const void* a, const void* b, void* c, hipStream_t stream) {
-    if (p.M == 0 || p.M > 32 || p.N == 0 || p.K == 0 || p.batches == 0 || p.batches > 65535 || p.row_bias || p.c_group) return TANNIC_UNSUPPORTED_DTYPE;
+    if (p.M == 0 || p.M > 64 || p.N == 0 || p.K == 0 || p.batches == 0 || p.batches > 65535 || p.row_bias || p.c_group) return TANNIC_UNSUPPORTED_DTYPE;
     // both operands K-contiguous; 16-byte chunks along K
     if (p.a_cs != 1 || p.b_rs != 1) return TANNIC_UNSUPPORTED_DTYPE;
     auto mult8 = [](int64_t v) { return v % 8 == 0; };
@@ -274,8 +274,16 @@ int run_skinny(const GemmProblem& p, const void* a, const void* b, void* c, hipS
         // two column blocks per wavefront (half as many workgroups, x read half as often) while every compute unit still gets one
         const bool two = static_cast<uint64_t>((p.N + 31) / 32) * p.batches >= 400;
         if (p.M <= 16) return two ? launch_stream<T, 1, 2>(p, a, b, c, stream) : launch_stream<T, 1, 1>(p, a, b, c, stream);
-        return two ? launch_stream<T, 2, 2>(p, a, b, c, stream) : launch_stream<T, 2, 1>(p, a, b, c, stream);
+        if (p.M <= 32) return two ? launch_stream<T, 2, 2>(p, a, b, c, stream) : launch_stream<T, 2, 1>(p, a, b, c, stream);
+        // Up to 64 rows: every wavefront still brings its own windows of x, three or four 16-row blocks next to one of W, so
+        // x comes out of the L2s N / 16 times.  That beats the tiles that share K while W is small (bf16, 64 rows, N x K =
+        // 4096 x 4096: 10.0 against 14.1 us; 1024 x 4096: 7.5 against 12.1) and loses to them beyond (14336 x 4096: 33 against
+        // 24 us).
+        if (static_cast<uint64_t>(p.N) * p.K * p.batches > (20u << 20)) return TANNIC_UNSUPPORTED_DTYPE;
+        if (p.M <= 48) return launch_stream<T, 3, 1>(p, a, b, c, stream);
+        return launch_stream<T, 4, 1>(p, a, b, c, stream);
     }
+    if (p.M > 32) return TANNIC_UNSUPPORTED_DTYPE;
     // K is split evenly over the wavefronts, in whole steps of 32
     const uint32_t steps = (p.K + 31) / 32, per_wave = (steps + kSkinnyWaves - 1) / kSkinnyWaves;
     const uint32_t k_per_wave = per_wave * 32;
