@@ -86,6 +86,8 @@ struct GemmWorkspace {
 int gemm_skinny_16bit(const GemmProblem& p, int dtype, const void* a, const void* b, void* c, hipStream_t stream);
 int gemm_mfma_16bit(const GemmProblem& p, int dtype, const void* a, const void* b, void* c, hipStream_t stream, const GemmWorkspace* workspace = nullptr);
 int gemm_mfma_f32(const GemmProblem& p, const float* a, const float* b, float* c, hipStream_t stream, const GemmWorkspace* workspace = nullptr);
+// fp32 products of a few hundred rows and columns (32 x 32 tiles whose wavefronts split K; gemm_small.hip)
+int gemm_small_f32(const GemmProblem& p, const float* a, const float* b, float* c, hipStream_t stream);
 // bm x bn tiles (256 x 256, 256 x 128, 128 x 128) filled by direct global -> LDS loads (gemm_dtl.hip); T is f16 or bf16
 template <class T> int gemm16_dtl(const GemmProblem& p, int bm, int bn, const void* a, const void* b, void* c, hipStream_t stream);
 // the 128 x 128 (bm = 128) or 64 x 128 (bm = 64) tiles with K shared between `splits` workgroups per tile (k_chunk elements each, a multiple of 64): fp32

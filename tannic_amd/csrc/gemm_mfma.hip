@@ -754,6 +754,10 @@ int gemm_mfma_16bit(const GemmProblem& p, int dtype, const void* a, const void* 
     return TANNIC_UNSUPPORTED_DTYPE;
 }
 
-int gemm_mfma_f32(const GemmProblem& p, const float* a, const float* b, float* c, hipStream_t stream, const GemmWorkspace* workspace) { return run16<float>(p, a, b, c, stream, workspace); }
+int gemm_mfma_f32(const GemmProblem& p, const float* a, const float* b, float* c, hipStream_t stream, const GemmWorkspace* workspace) {
+    const int small = gemm_small_f32(p, a, b, c, stream);
+    if (small != TANNIC_UNSUPPORTED_DTYPE) return small;
+    return run16<float>(p, a, b, c, stream, workspace);
+}
 
 }  // namespace th
