@@ -482,6 +482,8 @@ def secondary(b, only):
         work.append(gemm_entry(b, ta.int8, 4096, 4096, 4096, 20))
         work.append(gemm_entry(b, ta.float32, 512, 512, 512, 20))
         work.append(gemm_entry(b, ta.float32, 4096, 4096, 4096, 5))
+        work.append(gemm_entry(b, ta.float32, 16, 4096, 4096, 20))       # the reference's default type through a linear layer, few rows
+        work.append(gemm_entry(b, ta.bfloat16, 64, 4096, 4096, 20))
     if only in (None, "gemm-ceiling"):
         work += gemm_ceiling_entries(b)
     if only in (None, "conv"):

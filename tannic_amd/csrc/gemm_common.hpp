@@ -84,6 +84,7 @@ struct GemmWorkspace {
 // MFMA paths; each returns TANNIC_UNSUPPORTED_DTYPE when the problem does not
 // meet its layout/alignment conditions so that the caller can fall back.
 int gemm_skinny_16bit(const GemmProblem& p, int dtype, const void* a, const void* b, void* c, hipStream_t stream);
+int gemm_skinny_f32(const GemmProblem& p, const float* a, const float* b, float* c, hipStream_t stream);
 int gemm_mfma_16bit(const GemmProblem& p, int dtype, const void* a, const void* b, void* c, hipStream_t stream, const GemmWorkspace* workspace = nullptr);
 int gemm_mfma_f32(const GemmProblem& p, const float* a, const float* b, float* c, hipStream_t stream, const GemmWorkspace* workspace = nullptr);
 // fp32 products of a few hundred rows and columns (32 x 32 tiles whose wavefronts split K; gemm_small.hip)

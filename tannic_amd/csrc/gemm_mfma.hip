@@ -755,6 +755,9 @@ int gemm_mfma_16bit(const GemmProblem& p, int dtype, const void* a, const void* 
 }
 
 int gemm_mfma_f32(const GemmProblem& p, const float* a, const float* b, float* c, hipStream_t stream, const GemmWorkspace* workspace) {
+    // a handful of rows: stream the other operand once
+    const int skinny = gemm_skinny_f32(p, a, b, c, stream);
+    if (skinny != TANNIC_UNSUPPORTED_DTYPE) return skinny;
     const int small = gemm_small_f32(p, a, b, c, stream);
     if (small != TANNIC_UNSUPPORTED_DTYPE) return small;
     return run16<float>(p, a, b, c, stream, workspace);

@@ -33,6 +33,16 @@ template <class T> __device__ inline float4y skinny_mfma(uint4y a, uint4y b, flo
     }
 }
 
+// fp32: element e of both 16-byte fragments is one k of the lane's four: four v_mfma_f32_16x16x4f32
+template <> __device__ inline float4y skinny_mfma<float>(uint4y a, uint4y b, float4y c) {
+    float x[4], y[4];
+    __builtin_memcpy(x, &a, 16);
+    __builtin_memcpy(y, &b, 16);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) c = __builtin_amdgcn_mfma_f32_16x16x4f32(x[e], y[e], c, 0, 0, 0);
+    return c;
+}
+
 constexpr int kSkinnyWaves = 8;
 constexpr int kSkinnyUnroll = 8;   // K steps of 32 whose loads are issued together
 
@@ -172,7 +182,7 @@ __global__ __launch_bounds__(64 * kStreamWaves) void gemm_skinny_stream_kernel(c
         for (int j = 0; j < LOADS; ++j)
             __builtin_amdgcn_raw_ptr_buffer_load_lds(j / 2 < NB ? rsrc_w : rsrc_x, (skinny_lds_void)(ring + stage * STAGE_BYTES + j * 1024), 16, voff[j], k_bytes, 0, 0);
     };
-    const uint32_t all = p.K / 64;
+    const uint32_t all = p.K / kBKof<T>;   // windows of 128 bytes per row: 64 elements of 16 bits, 32 of fp32
     const uint32_t first = wave * windows_per_wave;
     const uint32_t count = first >= all ? 0 : (all - first < windows_per_wave ? all - first : windows_per_wave);
 
@@ -197,9 +207,9 @@ __global__ __launch_bounds__(64 * kStreamWaves) void gemm_skinny_stream_kernel(c
 #pragma unroll
         for (int half = 0; half < 2; ++half) {
 #pragma unroll
-            for (int nb = 0; nb < NB; ++nb) fw[half][nb] = *reinterpret_cast<const uint4y*>(at + nb * 1024 + tile_offset<T>(r, half * 4 + kc));
+            for (int nb = 0; nb < NB; ++nb) fw[half][nb] = *reinterpret_cast<const uint4y*>(at + nb * (2048 / sizeof(T)) + tile_offset<T>(r, half * 4 + kc));
 #pragma unroll
-            for (int mb = 0; mb < MB; ++mb) fx[half][mb] = *reinterpret_cast<const uint4y*>(at + (NB + mb) * 1024 + tile_offset<T>(r, half * 4 + kc));
+            for (int mb = 0; mb < MB; ++mb) fx[half][mb] = *reinterpret_cast<const uint4y*>(at + (NB + mb) * (2048 / sizeof(T)) + tile_offset<T>(r, half * 4 + kc));
         }
 #pragma unroll
         for (int half = 0; half < 2; ++half)
@@ -220,7 +230,7 @@ __global__ __launch_bounds__(64 * kStreamWaves) void gemm_skinny_stream_kernel(c
     __syncthreads();
     // accumulator: lane -> row of x (m) lane % 16; value v -> column n0 + 4 * (lane / 16) + v; wavefront t adds up tile t, t + 4, ..
     T* cb = c + oc;
-    const bool vector_ok = p.c_rs % 4 == 0 && p.N % 4 == 0 && reinterpret_cast<uintptr_t>(cb) % 8 == 0;
+    const bool vector_ok = p.c_rs % 4 == 0 && p.N % 4 == 0 && reinterpret_cast<uintptr_t>(cb) % (4 * sizeof(T)) == 0;
     for (int t = wave; t < MB * NB; t += kStreamWaves) {
         const int mb = t / NB, nb = t % NB;
         float4y sum = partial[t * 64 + lane];
@@ -234,9 +244,10 @@ __global__ __launch_bounds__(64 * kStreamWaves) void gemm_skinny_stream_kernel(c
         T* dst = cb + static_cast<int64_t>(m) * p.c_rs + col;
         if (vector_ok) {
             if (col < p.N) {
-                uint2 bits;
-                __builtin_memcpy(&bits, out, 8);
-                *reinterpret_cast<uint2*>(dst) = bits;
+                using Quad = std::conditional_t<sizeof(T) == 2, uint2, uint4>;
+                Quad bits;
+                __builtin_memcpy(&bits, out, sizeof(Quad));
+                *reinterpret_cast<Quad*>(dst) = bits;
             }
         } else {
 #pragma unroll
@@ -253,7 +264,7 @@ static int launch_stream(const GemmProblem& p, const void* a, const void* b, voi
     constexpr size_t lds = kStreamWaves * kStreamBytesPerWave;
     static std::atomic<uint64_t> configured{0};
     if (int rc = raise_lds_limit(reinterpret_cast<const void*>(kernel), lds, configured)) return rc;
-    const uint32_t windows = p.K / 64, per_wave = (windows + kStreamWaves - 1) / kStreamWaves;
+    const uint32_t windows = p.K / kBKof<T>, per_wave = (windows + kStreamWaves - 1) / kStreamWaves;
     hipLaunchKernelGGL(kernel, dim3((p.N + 16 * NB - 1) / (16 * NB), p.batches), dim3(64 * kStreamWaves), lds, stream, static_cast<const T*>(a), static_cast<const T*>(b),
                        static_cast<T*>(c), p, per_wave);
     return launch_status("gemm_skinny_stream_kernel");
@@ -264,46 +275,57 @@ int run_skinny(const GemmProblem& p, const void* a, const void* b, void* c, hipS
     if (p.M == 0 || p.M > 64 || p.N == 0 || p.K == 0 || p.batches == 0 || p.batches > 65535 || p.row_bias || p.c_group) return TANNIC_UNSUPPORTED_DTYPE;
     // both operands K-contiguous; 16-byte chunks along K
     if (p.a_cs != 1 || p.b_rs != 1) return TANNIC_UNSUPPORTED_DTYPE;
-    auto mult8 = [](int64_t v) { return v % 8 == 0; };
+    auto mult8 = [](int64_t v) { return v % kChunkOf<T> == 0; };   // whole 16-byte chunks
     if (!mult8(p.K) || !mult8(p.a_rs) || !mult8(p.b_cs)) return TANNIC_UNSUPPORTED_DTYPE;
     if (reinterpret_cast<uintptr_t>(a) % 16 || reinterpret_cast<uintptr_t>(b) % 16) return TANNIC_UNSUPPORTED_DTYPE;
     for (int d = 0; d < p.batch_rank; ++d)
         if (!mult8(p.a_bs[d]) || !mult8(p.b_bs[d])) return TANNIC_UNSUPPORTED_DTYPE;
     // whole windows of 64 and rows that do not overlap: the streaming kernel (offsets inside a block are 32-bit byte counts)
-    if (p.K % 64 == 0 && p.a_rs >= static_cast<int64_t>(p.K) && p.b_cs >= static_cast<int64_t>(p.K) && p.a_rs < (1 << 22) && p.b_cs < (1 << 22)) {
+    if (p.K % kBKof<T> == 0 && p.a_rs >= static_cast<int64_t>(p.K) && p.b_cs >= static_cast<int64_t>(p.K) && p.a_rs < (1 << 22) && p.b_cs < (1 << 22)) {
         // two column blocks per wavefront (half as many workgroups, x read half as often) while every compute unit still gets one
         const bool two = static_cast<uint64_t>((p.N + 31) / 32) * p.batches >= 400;
         if (p.M <= 16) return two ? launch_stream<T, 1, 2>(p, a, b, c, stream) : launch_stream<T, 1, 1>(p, a, b, c, stream);
         if (p.M <= 32) return two ? launch_stream<T, 2, 2>(p, a, b, c, stream) : launch_stream<T, 2, 1>(p, a, b, c, stream);
-        // Up to 64 rows: every wavefront still brings its own windows of x, three or four 16-row blocks next to one of W, so
-        // x comes out of the L2s N / 16 times.  That beats the tiles that share K while W is small (bf16, 64 rows, N x K =
-        // 4096 x 4096: 10.0 against 14.1 us; 1024 x 4096: 7.5 against 12.1) and loses to them beyond (14336 x 4096: 33 against
-        // 24 us).
-        if (static_cast<uint64_t>(p.N) * p.K * p.batches > (20u << 20)) return TANNIC_UNSUPPORTED_DTYPE;
-        if (p.M <= 48) return launch_stream<T, 3, 1>(p, a, b, c, stream);
-        return launch_stream<T, 4, 1>(p, a, b, c, stream);
+        // (fp32 stops here: with more row blocks its MFMAs, a sixteenth as fast, take longer than W takes to arrive)
+        if constexpr (sizeof(T) == 4) {
+            return TANNIC_UNSUPPORTED_DTYPE;
+        } else {
+            // Up to 64 rows: every wavefront still brings its own windows of x, three or four 16-row blocks next to one of W, so
+            // x comes out of the L2s N / 16 times.  That beats the tiles that share K while W is small (bf16, 64 rows, N x K =
+            // 4096 x 4096: 10.0 against 14.1 us; 1024 x 4096: 7.5 against 12.1) and loses to them beyond (14336 x 4096: 33 against
+            // 24 us).
+            if (static_cast<uint64_t>(p.N) * p.K * p.batches > (20u << 20)) return TANNIC_UNSUPPORTED_DTYPE;
+            if (p.M <= 48) return launch_stream<T, 3, 1>(p, a, b, c, stream);
+            return launch_stream<T, 4, 1>(p, a, b, c, stream);
+        }
     }
-    if (p.M > 32) return TANNIC_UNSUPPORTED_DTYPE;
-    // K is split evenly over the wavefronts, in whole steps of 32
-    const uint32_t steps = (p.K + 31) / 32, per_wave = (steps + kSkinnyWaves - 1) / kSkinnyWaves;
-    const uint32_t k_per_wave = per_wave * 32;
-    // A single row costs almost nothing to load next to W; with more rows, two column blocks per wavefront halve
-    // what x costs, as long as there are still blocks for every compute unit.
-    const bool pairs = p.M > 4 && static_cast<uint64_t>((p.N + 31) / 32) * p.batches >= 224;
-    const uint32_t blocks = pairs ? (p.N + 31) / 32 : (p.N + 15) / 16;
-    const dim3 grid(blocks, p.batches), block(64 * kSkinnyWaves);
-    const T* pa = static_cast<const T*>(a);
-    const T* pb = static_cast<const T*>(b);
-    T* pc = static_cast<T*>(c);
-    if (p.M <= 16) {
-        if (pairs) hipLaunchKernelGGL((gemm_skinny_kernel<T, 1, 2>), grid, block, 0, stream, pa, pb, pc, p, k_per_wave);
-        else hipLaunchKernelGGL((gemm_skinny_kernel<T, 1, 1>), grid, block, 0, stream, pa, pb, pc, p, k_per_wave);
+    if constexpr (sizeof(T) == 4) {
+        return TANNIC_UNSUPPORTED_DTYPE;   // the kernel for other K is written for 16-bit fragments
     } else {
-        if (pairs) hipLaunchKernelGGL((gemm_skinny_kernel<T, 2, 2>), grid, block, 0, stream, pa, pb, pc, p, k_per_wave);
-        else hipLaunchKernelGGL((gemm_skinny_kernel<T, 2, 1>), grid, block, 0, stream, pa, pb, pc, p, k_per_wave);
+        if (p.M > 32) return TANNIC_UNSUPPORTED_DTYPE;
+        // K is split evenly over the wavefronts, in whole steps of 32
+        const uint32_t steps = (p.K + 31) / 32, per_wave = (steps + kSkinnyWaves - 1) / kSkinnyWaves;
+        const uint32_t k_per_wave = per_wave * 32;
+        // A single row costs almost nothing to load next to W; with more rows, two column blocks per wavefront halve
+        // what x costs, as long as there are still blocks for every compute unit.
+        const bool pairs = p.M > 4 && static_cast<uint64_t>((p.N + 31) / 32) * p.batches >= 224;
+        const uint32_t blocks = pairs ? (p.N + 31) / 32 : (p.N + 15) / 16;
+        const dim3 grid(blocks, p.batches), block(64 * kSkinnyWaves);
+        const T* pa = static_cast<const T*>(a);
+        const T* pb = static_cast<const T*>(b);
+        T* pc = static_cast<T*>(c);
+        if (p.M <= 16) {
+            if (pairs) hipLaunchKernelGGL((gemm_skinny_kernel<T, 1, 2>), grid, block, 0, stream, pa, pb, pc, p, k_per_wave);
+            else hipLaunchKernelGGL((gemm_skinny_kernel<T, 1, 1>), grid, block, 0, stream, pa, pb, pc, p, k_per_wave);
+        } else {
+            if (pairs) hipLaunchKernelGGL((gemm_skinny_kernel<T, 2, 2>), grid, block, 0, stream, pa, pb, pc, p, k_per_wave);
+            else hipLaunchKernelGGL((gemm_skinny_kernel<T, 2, 1>), grid, block, 0, stream, pa, pb, pc, p, k_per_wave);
+        }
+        return launch_status("gemm_skinny_kernel");
     }
-    return launch_status("gemm_skinny_kernel");
 }
+
+int gemm_skinny_f32(const GemmProblem& p, const float* a, const float* b, float* c, hipStream_t stream) { return run_skinny<float>(p, a, b, c, stream); }
 
 int gemm_skinny_16bit(const GemmProblem& p, int dtype, const void* a, const void* b, void* c, hipStream_t stream) {
     if (dtype == TANNIC_FLOAT16) return run_skinny<f16>(p, a, b, c, stream);
