@@ -118,6 +118,9 @@ static int conv2d_entry(const tannic_tensor_t* x, const tannic_tensor_t* w, cons
     if (status != TANNIC_UNSUPPORTED_DTYPE) return status;
     status = conv2d_unfold(p, x->dtype, x->address, w->address, pb, y->address, s);
     if (status != TANNIC_UNSUPPORTED_DTYPE) return status;
+    // 16-bit shapes none of the above takes: unfolded and multiplied, while the unfolded operand is small
+    status = conv2d_unfold_batch_any(p, x->dtype, x->address, w->address, pb, y->address, s);
+    if (status != TANNIC_UNSUPPORTED_DTYPE) return status;
     status = conv2d_mfma(p, x->dtype, x->address, w->address, pb, y->address, s);
     if (status != TANNIC_UNSUPPORTED_DTYPE) return status;
     switch (x->dtype) {

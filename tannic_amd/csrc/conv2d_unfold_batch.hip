@@ -43,7 +43,9 @@ __global__ __launch_bounds__(256) void conv_unfold_batch_kernel(const T* x, T* c
     *reinterpret_cast<uint4*>(col + static_cast<size_t>(row) * pitch + group * E) = bits;
 }
 
-template <class T>
+// ANY_SIZE: as the last kernel before the general ones, for whatever the specialised kernels have refused, as long as
+// the unfolded operand stays small enough to be worth writing out.
+template <class T, bool ANY_SIZE>
 static int run_unfold_batch(const ConvProblem& p, int dtype, const void* x, const void* w, const void* bias, void* y, hipStream_t stream) {
     if (p.has_bias && p.bs != 1 && p.O > 1) return TANNIC_UNSUPPORTED_DTYPE;   // the product reads its row bias as a dense vector
     if (p.N == 0 || p.O == 0 || p.HO == 0 || p.WO == 0) return TANNIC_SUCCESS;
@@ -51,11 +53,13 @@ static int run_unfold_batch(const ConvProblem& p, int dtype, const void* x, cons
     const uint64_t K = static_cast<uint64_t>(p.C) * p.KH * p.KW, pixels = static_cast<uint64_t>(p.HO) * p.WO;
     // Where this pays: few pixels per image (a tile of the patch kernels would be mostly empty), a long K, and enough
     // columns in all for whole tiles of the product.
-    if (pixels > 100 || K < 512 || K % E != 0 || K >= (1u << 24)) return TANNIC_UNSUPPORTED_DTYPE;
+    // (ANY_SIZE, fp16, us against the general tile kernel: K = 2352 49 / 104, 648 13 / 38, 600 22 / 31, 360 23 / 26, but 216 20 / 15,
+    // 144 33 / 25, 72 25 / 16: with a short K the unfolded operand is as large as the work)
+    if ((ANY_SIZE ? K < 320 : (pixels > 100 || K < 512)) || K % E != 0 || K >= (1u << 24) || pixels >= (1u << 24)) return TANNIC_UNSUPPORTED_DTYPE;
     const uint32_t pitch = static_cast<uint32_t>((pixels + E - 1) / E * E);
     const uint64_t columns = static_cast<uint64_t>(p.N) * pitch;
     if (columns < 256 || columns >= (1ull << 31) || K * p.N * (pitch / E) >= (1ull << 31)) return TANNIC_UNSUPPORTED_DTYPE;
-    if (K * columns * sizeof(T) > (512ull << 20)) return TANNIC_UNSUPPORTED_DTYPE;
+    if (K * columns * sizeof(T) > ((ANY_SIZE ? 128ull : 512ull) << 20)) return TANNIC_UNSUPPORTED_DTYPE;
     // the kernel tensor as a K-contiguous O x K matrix, the result as pixel-contiguous rows
     if (p.ws[3] != 1 || p.ws[2] != static_cast<int64_t>(p.KW) || p.ws[1] != static_cast<int64_t>(p.KH) * p.KW || p.ws[0] != static_cast<int64_t>(K) ||
         reinterpret_cast<uintptr_t>(w) % 16 != 0)
@@ -102,9 +106,16 @@ static int run_unfold_batch(const ConvProblem& p, int dtype, const void* x, cons
 
 int conv2d_unfold_batch(const ConvProblem& p, int dtype, const void* x, const void* w, const void* bias, void* y, hipStream_t stream) {
     if (p.KH == 1 && p.KW == 1) return TANNIC_UNSUPPORTED_DTYPE;   // conv2d_pointwise.hip: no unfolding needed
-    if (dtype == TANNIC_FLOAT16) return run_unfold_batch<f16>(p, dtype, x, w, bias, y, stream);
-    if (dtype == TANNIC_BFLOAT16) return run_unfold_batch<bf16>(p, dtype, x, w, bias, y, stream);
-    if (dtype == TANNIC_FLOAT32) return run_unfold_batch<float>(p, dtype, x, w, bias, y, stream);
+    if (dtype == TANNIC_FLOAT16) return run_unfold_batch<f16, false>(p, dtype, x, w, bias, y, stream);
+    if (dtype == TANNIC_BFLOAT16) return run_unfold_batch<bf16, false>(p, dtype, x, w, bias, y, stream);
+    if (dtype == TANNIC_FLOAT32) return run_unfold_batch<float, false>(p, dtype, x, w, bias, y, stream);
+    return TANNIC_UNSUPPORTED_DTYPE;
+}
+
+int conv2d_unfold_batch_any(const ConvProblem& p, int dtype, const void* x, const void* w, const void* bias, void* y, hipStream_t stream) {
+    if (p.KH == 1 && p.KW == 1) return TANNIC_UNSUPPORTED_DTYPE;
+    if (dtype == TANNIC_FLOAT16) return run_unfold_batch<f16, true>(p, dtype, x, w, bias, y, stream);
+    if (dtype == TANNIC_BFLOAT16) return run_unfold_batch<bf16, true>(p, dtype, x, w, bias, y, stream);
     return TANNIC_UNSUPPORTED_DTYPE;
 }
 

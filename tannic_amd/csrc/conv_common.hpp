@@ -29,6 +29,7 @@ int conv2d_gather32(const ConvProblem& p, int dtype, const void* x, const void* 
 int conv2d_unfold(const ConvProblem& p, int dtype, const void* x, const void* w, const void* bias, void* y, hipStream_t stream);
 // few output pixels per image under many channels (fp16, bf16, fp32): the whole batch unfolded side by side, one product
 int conv2d_unfold_batch(const ConvProblem& p, int dtype, const void* x, const void* w, const void* bias, void* y, hipStream_t stream);
+int conv2d_unfold_batch_any(const ConvProblem& p, int dtype, const void* x, const void* w, const void* bias, void* y, hipStream_t stream);
 int conv2d_mfma(const ConvProblem& p, int dtype, const void* x, const void* w, const void* bias, void* y, hipStream_t stream);
 
 }  // namespace th

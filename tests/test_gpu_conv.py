@@ -102,6 +102,10 @@ CASES = {
     "unfolded_k3_s2_14_to_7": ((6, 64, 14, 14), (48, 64, 3, 3), (2, 2), (1, 1)),
     "unfolded_k5_9x9": ((8, 32, 9, 9), (16, 32, 5, 5), (1, 1), (2, 2)),
     "unfolded_k3x2_100_pixels": ((3, 96, 10, 11), (24, 96, 3, 2), (1, 1), (1, 0)),
+    # ... and as the last resort before the general tiles, for channel counts that no patch kernel takes (K >= 320)
+    "unfolded_any_k7_48ch": ((2, 48, 20, 20), (48, 48, 7, 7), (1, 1), (3, 3)),
+    "unfolded_any_k3_72ch": ((4, 72, 17, 17), (100, 72, 3, 3), (1, 1), (1, 1)),
+    "unfolded_any_k3_40ch_s2": ((3, 40, 21, 19), (24, 40, 3, 3), (2, 2), (1, 1)),
 }
 
 
