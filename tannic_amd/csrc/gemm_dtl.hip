@@ -311,10 +311,20 @@ __global__ __launch_bounds__(256, BLOCKS_PER_CU) void gemm16_dtl_kernel(const T*
     constexpr int PIECES = WN / 8, LANES_PER_ROW = PIECES <= 4 ? 4 : PIECES <= 8 ? 8 : 16, ROWS_PER_PASS = 64 / LANES_PER_ROW;
     static_assert(PIECES <= 16, "a wavefront's block is at most 128 columns wide");
     const uint32_t piece = lane % LANES_PER_ROW, col = n0 + wn + piece * 8;
-    if (p.c_group) {
-        // columns in groups (an image each): the lane's piece belongs to one group, at one place in it, for every row
+    const bool aligned_rows = (p.c_rs | p.N) % 8 == 0 && reinterpret_cast<uintptr_t>(c) % 16 == 0;
+    if (p.c_group || !aligned_rows) {
+        // Columns in groups (an image each): the lane's piece belongs to one group, at one place in it, for every row.
+        // Plain rows that do not start at multiples of 16 bytes, or end inside a piece, are stored the same way.
         uint32_t live = 0;
-        T* first = piece < PIECES && col < p.N ? grouped_piece(c, p, 0, col, 8, live) : c;
+        T* first = c;
+        if (piece < PIECES && col < p.N) {
+            if (p.c_group) {
+                first = grouped_piece(c, p, 0, col, 8, live);
+            } else {
+                first = c + col;
+                live = p.N - col < 8 ? p.N - col : 8;
+            }
+        }
 #pragma unroll
         for (int r0 = 0; r0 < WM; r0 += ROWS_PER_PASS) {
             const uint32_t r = r0 + lane / LANES_PER_ROW, row = m0 + wm + r;
@@ -433,9 +443,10 @@ int gemm16_dtl(const GemmProblem& p, int bm, int bn, const void* a, const void* 
     if (!operands_fit<T>(p, bm, bn, a_t, b_t)) return TANNIC_UNSUPPORTED_DTYPE;
     constexpr int quad = 16 / sizeof(typename DtlTypes<T>::Out);   // results per 16-byte store
     if (p.c_group && (sizeof(T) != 2 || p.N % 8 != 0)) return TANNIC_UNSUPPORTED_DTYPE;   // column groups: 16-bit results, whole pieces of eight
-    if (!p.c_group && (p.N % quad != 0 || p.c_rs % quad != 0 || reinterpret_cast<uintptr_t>(c) % 16 != 0)) return TANNIC_UNSUPPORTED_DTYPE;
+    // (16-bit results may lie anywhere: the kernel looks at the alignment of its own rows; int32 results are stored as quads)
+    if (sizeof(T) != 2 && (p.N % quad != 0 || p.c_rs % quad != 0 || reinterpret_cast<uintptr_t>(c) % 16 != 0)) return TANNIC_UNSUPPORTED_DTYPE;
     for (int d = 0; d < p.batch_rank; ++d)
-        if (p.c_bs[d] % quad != 0) return TANNIC_UNSUPPORTED_DTYPE;
+        if (sizeof(T) != 2 && p.c_bs[d] % quad != 0) return TANNIC_UNSUPPORTED_DTYPE;
     if constexpr (sizeof(T) == 2) {
         if (a_t || b_t) return gemm16_dtl_krows<T>(p, bm, bn, a_t, b_t, SplitK{0, 0, nullptr}, a, b, c, stream);
     }

@@ -687,13 +687,19 @@ int run16(const GemmProblem& p, const void* a, const void* b, void* c, hipStream
         const double cost = static_cast<double>((tiles + 255) / 256) * w * (1.0 + (256 - w) * kNarrowTilePenalty);
         if (cost < least) { least = cost; width = w; }
     }
+    // Not when the last (or only) column of large tiles would be mostly empty (attention's P . V has 64 or 128 columns: fp16
+    // [200, 200] . [200, 64] x 384 takes 31 us on 256 x 256 tiles and 17-19 us on the smaller ones, fp32 140 against 60), and
+    // for fp32 only under a long K: its matrix pipe, not the operand traffic, sets the pace, so what counts is how little
+    // of a tile is padding and how many blocks overlap their starts and ends ([2048, 128] . [128, 2048] x 32: 437 us on
+    // 256 x 256 tiles, 383 on 128 x 128; 4096^3: 1094 against 1105).
+    const bool large_ok = static_cast<double>(p.N) >= 0.75 * (((p.N + 255) / 256) * 256.0) && (sizeof(T) == 2 || p.K >= 1024);
     if constexpr (sizeof(T) == 2) {
-        if (p.M > 192 && width && width != 256) {
+        if (large_ok && p.M > 192 && width && width != 256) {
             const int rc = gemm16_dtl<T>(p, 256, width, a, b, c, stream);
             if (rc != TANNIC_UNSUPPORTED_DTYPE) return rc;
         }
     }
-    if (p.M > 192 && tiles_m * ((p.N + 255) / 256) * p.batches >= 200) {
+    if (large_ok && p.M > 192 && tiles_m * ((p.N + 255) / 256) * p.batches >= 200) {
         if constexpr (sizeof(T) == 2) {
             const int rc = gemm16_dtl<T>(p, 256, 256, a, b, c, stream);
             if (rc != TANNIC_UNSUPPORTED_DTYPE) return rc;
@@ -709,8 +715,14 @@ int run16(const GemmProblem& p, const void* a, const void* b, void* c, hipStream
     double best_cost = 1e30;
     int best_bm = tall ? 128 : 64;
     uint32_t best_splits = 1;
-    for (int bm : {256, 128, 64}) {
+    // (fp32: equal costs go to the 128-row tile, which is tried first)
+    const int heights[3] = {sizeof(T) == 4 ? 128 : 256, sizeof(T) == 4 ? 256 : 128, 64};
+    // Under a short K a block's start and end count: about 2 us for the 128- and 256-row tiles and 0.7 us for the 64-row
+    // one, per round of blocks (fp16, K = 64, [192, 64] . [64, 192] x 384: 23 us on 128 x 128 tiles, 15 us on 64 x 128).
+    const bool short_k = steps_all <= 4 && sizeof(T) == 2;
+    for (int bm : heights) {
         if ((bm == 128 && !tall) || (bm == 256 && p.M <= 192)) continue;
+        const double block_fixed = short_k ? (bm == 64 ? 0.7 : 2.0) : 0.0;
         const uint64_t tiles = static_cast<uint64_t>((p.M + bm - 1) / bm) * ((p.N + 127) / 128) * p.batches;
         for (uint32_t splits : {1u, 2u, 4u, 8u, 16u}) {
             if (splits > 1 && (bm == 256 || splits > p.K / (sizeof(T) == 4 ? 64 : 256))) break;
@@ -725,7 +737,7 @@ int run16(const GemmProblem& p, const void* a, const void* b, void* c, hipStream
             // fp32: the matrix pipe, sixteen times slower than for the 16-bit types, sets the pace of a step
             // (2 * bm * 128 * 64 flops at 157.3 TFLOP/s over 256 compute units)
             if constexpr (sizeof(T) == 4) step_us = std::max(step_us, 2.0 * bm * 128 * 64 / (157.3e6 / 256));
-            double cost = rounds * (steps_all / splits) * step_us + 5.0;
+            double cost = rounds * ((steps_all / splits) * step_us + block_fixed) + 5.0;
             if (splits > 1) cost += 4.0 + (splits + 0.5) * static_cast<double>(p.M) * p.N * p.batches * 4.0 / 5.0e6;
             if (cost < best_cost) { best_cost = cost; best_bm = bm; best_splits = splits; }
         }

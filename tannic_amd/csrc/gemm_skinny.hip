@@ -294,7 +294,9 @@ int run_skinny(const GemmProblem& p, const void* a, const void* b, void* c, hipS
             // x comes out of the L2s N / 16 times.  That beats the tiles that share K while W is small (bf16, 64 rows, N x K =
             // 4096 x 4096: 10.0 against 14.1 us; 1024 x 4096: 7.5 against 12.1) and loses to them beyond (14336 x 4096: 33 against
             // 24 us).
-            if (static_cast<uint64_t>(p.N) * p.K * p.batches > (20u << 20)) return TANNIC_UNSUPPORTED_DTYPE;
+            // (One product at a time: the many small products of an attention head - 64 x 64 x 64, a thousand of them - have one
+            // window of K for four wavefronts and take 28 us here against 8 on tiles.)
+            if (p.batches != 1 || p.K < 256 || static_cast<uint64_t>(p.N) * p.K > (20u << 20)) return TANNIC_UNSUPPORTED_DTYPE;
             if (p.M <= 48) return launch_stream<T, 3, 1>(p, a, b, c, stream);
             return launch_stream<T, 4, 1>(p, a, b, c, stream);
         }

@@ -47,10 +47,13 @@ LAYOUTS = {
     "stream_20_rows_one_window": ((20, 64), (48, 64), [], [("transpose", (-1, -2))]),
     "stream_32_rows_many_columns": ((32, 128), (12840, 128), [], [("transpose", (-1, -2))]),
     "stream_5_rows_many_columns": ((5, 192), (12816, 192), [], [("transpose", (-1, -2))]),
-    # 33 .. 64 rows over a small W: three and four row blocks per wavefront
-    "stream_40_rows": ((40, 192), (100, 192), [], [("transpose", (-1, -2))]),
+    # 33 .. 64 rows over a small W (one product, K >= 256): three and four row blocks per wavefront; batches of such
+    # products and shorter K stay on tiles
+    "stream_40_rows": ((40, 320), (100, 320), [], [("transpose", (-1, -2))]),
     "stream_64_rows_ragged_columns": ((64, 256), (90, 256), [], [("transpose", (-1, -2))]),
-    "stream_33_rows_batched": ((2, 33, 128), (2, 50, 128), [], [("transpose", (-1, -2))]),
+    "stream_33_rows": ((33, 256), (50, 256), [], [("transpose", (-1, -2))]),
+    "tiles_33_rows_batched": ((2, 33, 128), (2, 50, 128), [], [("transpose", (-1, -2))]),
+    "tiles_64_rows_many_small_batches": ((40, 64, 64), (40, 64, 64), [], [("transpose", (-1, -2))]),
     "stream_49_rows_long_k": ((49, 2048), (24, 2048), [], [("transpose", (-1, -2))]),
     "stream_batched_views": ((3, 9, 320), (3, 70, 320), [("index", (Ellipsis, slice(0, 256)))], [("index", (Ellipsis, slice(64, 320))), ("transpose", (-1, -2))]),
     "split_k_nt": ((128, 1096), (136, 1096), [], [("transpose", (-1, -2))]),
