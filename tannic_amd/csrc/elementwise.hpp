@@ -238,6 +238,77 @@ __global__ __launch_bounds__(kBlock) void elementwise_kernel(F f, Plan p) {
     }
 }
 
+// Rows whose length is not a multiple of the vector (softmax over 197 columns: x - max, x / sum) when every operand is
+// either contiguous over the whole index space or constant along the row: the kernel above would go element by element,
+// but the contiguous operands do not care where a row ends.  A thread owns VEC consecutive elements of the flat index
+// space (the last thread of all a shorter tail); the row-constant operand is looked up for the row of the thread's first
+// element and, when the vector runs over the row's end, for the next row (rows are at least VEC long: two rows at most).
+struct FlatPlan {
+    Plan p;                 // the collapsed plan; p.row_div divides by the row length
+    uint64_t elements;      // all of them
+    uint32_t rows;          // product of the outer extents
+    bool full[2];           // source o is contiguous over everything (else constant along the row)
+};
+
+template <class T>
+__device__ inline int64_t outer_offset(const Plan& p, int o, uint32_t row) {
+    int64_t off = 0;
+    for (int d = p.rank - 2; d >= 0; --d) {
+        uint32_t q, c;
+        p.div[d].divmod(row, q, c);
+        row = q;
+        off += static_cast<int64_t>(c) * p.stride[o][d];
+    }
+    return off;
+}
+
+template <class T, int VEC>
+__device__ inline Pack<T, VEC> flat_source(const FlatPlan& fp, int o, const T* base, uint64_t first, uint32_t row, uint32_t col, uint32_t live) {
+    Pack<T, VEC> r;
+    if (fp.full[o]) {
+        if (live == VEC) return load_pack<T, VEC>(base + first);
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) r.v[i] = static_cast<uint32_t>(i) < live ? base[first + i] : T{};
+        return r;
+    }
+    const uint32_t length = fp.p.extent[fp.p.rank - 1];
+    const T here = base[outer_offset<T>(fp.p, o, row)];
+    const bool runs_over = col + VEC > length && row + 1 < fp.rows;
+    const T next = runs_over ? base[outer_offset<T>(fp.p, o, row + 1)] : here;
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) r.v[i] = col + i < length ? here : next;
+    return r;
+}
+
+template <class F, int VEC>
+__global__ __launch_bounds__(kBlock) void elementwise_flat_kernel(F f, FlatPlan fp, uint32_t vectors) {
+    using S0 = typename F::S0;
+    using S1 = typename F::S1;
+    using D = typename F::D;
+    const uint32_t v = blockIdx.x * kBlock + threadIdx.x;
+    if (v >= vectors) return;
+    const uint64_t first = static_cast<uint64_t>(v) * VEC;
+    const uint32_t live = fp.elements - first < VEC ? static_cast<uint32_t>(fp.elements - first) : VEC;
+    uint32_t row = 0, col = 0;
+    if (fp.p.rank > 1) fp.p.row_div.divmod(static_cast<uint32_t>(first), row, col);   // fewer than 2^31 elements (the launch checks)
+    const Pack<S0, VEC> a = flat_source<S0, VEC>(fp, 0, f.a, first, row, col, live);
+    Pack<S1, VEC> b;
+    if constexpr (F::sources == 2) b = flat_source<S1, VEC>(fp, 1, f.b, first, row, col, live);
+    Pack<D, VEC> r;
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) {
+        if constexpr (F::sources == 2) r.v[i] = f(a.v[i], b.v[i]);
+        else r.v[i] = f(a.v[i], S1{});
+    }
+    if (live == VEC) {
+        store_pack<D, VEC>(f.out + first, r);
+    } else {
+#pragma unroll
+        for (int i = 0; i < VEC; ++i)
+            if (static_cast<uint32_t>(i) < live) f.out[first + i] = r.v[i];
+    }
+}
+
 template <class A, class B>
 constexpr size_t max_size() { return sizeof(A) > sizeof(B) ? sizeof(A) : sizeof(B); }
 
@@ -270,6 +341,44 @@ int launch_elementwise(F f, Plan p, hipStream_t stream) {
     bool vec = VEC > 1 && p.extent[last] % VEC == 0 && vector_ok(p, 0, f.a, VEC, false) &&
                vector_ok(p, 2, f.out, VEC, true);
     if (F::sources == 2) vec = vec && vector_ok(p, 1, f.b, VEC, false);
+    if constexpr (VEC > 1) {
+        if (!vec) {
+            // contiguous operands next to row-constant ones, a row length the vector does not divide: vectors over the flat index
+            FlatPlan fp;
+            fp.elements = rows * p.extent[last];
+            auto contiguous = [&](int o) {
+                int64_t expect = 1;
+                for (int d = last; d >= 0; --d) {
+                    if (p.stride[o][d] != expect) return false;
+                    expect *= p.extent[d];
+                }
+                return true;
+            };
+            auto aligned_to = [](const void* ptr, size_t bytes) { return reinterpret_cast<uintptr_t>(ptr) % bytes == 0; };
+            bool flat = fp.elements > 0 && fp.elements < (1ull << 31) && contiguous(2) && aligned_to(f.out, sizeof(D) * VEC);
+            bool any_constant = false;
+            fp.full[0] = fp.full[1] = true;
+            if (flat) {
+                fp.full[0] = contiguous(0);
+                flat = fp.full[0] ? aligned_to(f.a, sizeof(S0) * VEC) : p.stride[0][last] == 0;
+                any_constant = !fp.full[0];
+            }
+            if (flat && F::sources == 2) {
+                fp.full[1] = contiguous(1);
+                flat = fp.full[1] ? aligned_to(f.b, sizeof(S1) * VEC) : p.stride[1][last] == 0;
+                any_constant = any_constant || !fp.full[1];
+            }
+            if (flat && any_constant && (p.rank < 2 || p.extent[last] < static_cast<uint32_t>(VEC))) flat = false;
+            if (flat) {
+                fp.rows = static_cast<uint32_t>(rows);
+                p.row_div = FastDiv(p.extent[last]);
+                fp.p = p;
+                const uint32_t vectors = static_cast<uint32_t>((fp.elements + VEC - 1) / VEC);
+                hipLaunchKernelGGL((elementwise_flat_kernel<F, VEC>), dim3((vectors + kBlock - 1) / kBlock), dim3(kBlock), 0, stream, f, fp, vectors);
+                return launch_status("elementwise_flat_kernel");
+            }
+        }
+    }
     p.row_vectors = vec ? p.extent[last] / VEC : p.extent[last];
     p.row_div = FastDiv(p.row_vectors);
     if (rows * p.row_vectors >= (1ull << 31)) {

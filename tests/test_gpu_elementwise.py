@@ -42,6 +42,14 @@ LAYOUTS = {
     "expanded": ((1, 96), (50, 96), [("expand", (50, 96))], []),
     "sliced_misaligned": ((64, 130), (64, 128), [("index", (slice(None), slice(1, 129)))], []),
     "singleton": ((1, 1), (1,), [], []),
+    # rows whose length no vector divides next to an operand that is constant along the row (softmax's x - max): vectors
+    # over the flat index that run over row ends; the constant operand with its own outer strides; rows shorter than a
+    # vector; an odd number of elements in all; the constant operand first
+    "odd_rows_column": ((37, 197), (37, 1), [], []),
+    "odd_rows_column_outer_broadcast": ((3, 5, 21, 19), (3, 1, 21, 1), [], []),
+    "short_odd_rows_column": ((50, 5), (50, 1), [], []),
+    "odd_count_column": ((9, 31), (9, 1), [], []),
+    "column_first_odd_rows": ((23, 1), (23, 45), [], []),
     "rank8": ((2, 1, 2, 3, 1, 2, 2, 3), (1, 3, 2, 1, 2, 2, 1, 3), [], []),
 }
 PAIRS = ([(d, d) for d in INTS + FLOATS + [ta.complex64, ta.complex128]] +
