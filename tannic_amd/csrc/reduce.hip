@@ -181,7 +181,11 @@ __device__ inline void emit(typename Op::A acc, uint32_t count, typename Op::Out
 
 // ---- rows: inner == 1 ----------------------------------------------------------
 // WAVES waves cooperate on one row; a block of 256 threads holds 4 / WAVES rows.
-template <class Op, int VEC, int WAVES>
+// RAGGED: rows that do not start at multiples of 16 bytes or whose length no vector divides (a softmax over 197 columns).
+// The aligned middle of a row is read as vectors all the same; the up to VEC - 1 elements before it and after it are
+// taken one per lane by the row's first wavefront, before and after its share of the middle, so that a lane still meets
+// its elements in increasing index order.
+template <class Op, int VEC, int WAVES, bool RAGGED = false>
 __global__ __launch_bounds__(kThreads) void reduce_rows_kernel(const typename Op::S* src, typename Op::Out* dst, uint32_t rows, uint32_t R) {
     using A = typename Op::A;
     using T = typename Op::S;
@@ -194,10 +198,17 @@ __global__ __launch_bounds__(kThreads) void reduce_rows_kernel(const typename Op
     if (row < rows) {
         const T* p = src + static_cast<size_t>(row) * R;
         constexpr uint32_t STRIDE = kWave * WAVES * VEC;
-        uint32_t r = (part * kWave + lane) * VEC;
+        uint32_t head = 0, end = R;   // [head, end): whole aligned vectors
+        if constexpr (RAGGED) {
+            head = static_cast<uint32_t>((VEC - (reinterpret_cast<uintptr_t>(p) / sizeof(T)) % VEC) % VEC);
+            if (head > R) head = R;
+            end = head + (R - head) / VEC * VEC;
+            if (part == 0 && static_cast<uint32_t>(lane) < head) acc = Op::step(acc, p[lane], lane);
+        }
+        uint32_t r = head + (part * kWave + lane) * VEC;
         // two independent accumulators keep two 16-byte loads in flight per lane
         A acc2 = Op::init();
-        for (; r + STRIDE + VEC <= R; r += 2 * STRIDE) {
+        for (; r + STRIDE + VEC <= end; r += 2 * STRIDE) {
             const Vec<T, VEC> x = load_vec<T, VEC>(p + r);
             const Vec<T, VEC> y = load_vec<T, VEC>(p + r + STRIDE);
 #pragma unroll
@@ -205,10 +216,13 @@ __global__ __launch_bounds__(kThreads) void reduce_rows_kernel(const typename Op
 #pragma unroll
             for (int i = 0; i < VEC; ++i) acc2 = Op::step(acc2, y.v[i], r + STRIDE + i);
         }
-        for (; r + VEC <= R; r += STRIDE) {
+        for (; r + VEC <= end; r += STRIDE) {
             const Vec<T, VEC> x = load_vec<T, VEC>(p + r);
 #pragma unroll
             for (int i = 0; i < VEC; ++i) acc = Op::step(acc, x.v[i], r + i);
+        }
+        if constexpr (RAGGED) {
+            if (part == 0 && end + lane < R) acc = Op::step(acc, p[end + lane], end + lane);
         }
         acc = Op::combine(acc, acc2);
     }
@@ -406,6 +420,39 @@ __global__ __launch_bounds__(kThreads) void reduce_columns_kernel(const typename
     }
 }
 
+// A few very long rows (the index of the largest of 128 256 logits, one row per sequence): a row is shared by `gridDim.x`
+// blocks, each folding a range of its aligned vectors (the first block also the elements before and after them), and
+// reduce_finish_kernel folds the blocks' results.
+template <class Op, int VEC>
+__global__ __launch_bounds__(kThreads) void reduce_rows_split_kernel(const typename Op::S* src, typename Op::A* partial, uint32_t rows, uint32_t R,
+                                                                      uint32_t vectors_per_split) {
+    using A = typename Op::A;
+    using T = typename Op::S;
+    const uint32_t row = blockIdx.y, split = blockIdx.x, tid = threadIdx.x;
+    const T* p = src + static_cast<size_t>(row) * R;
+    uint32_t head = static_cast<uint32_t>((VEC - (reinterpret_cast<uintptr_t>(p) / sizeof(T)) % VEC) % VEC);
+    if (head > R) head = R;
+    const uint32_t vectors = (R - head) / VEC, end = head + vectors * VEC;
+    const uint32_t v0 = split * vectors_per_split, v1 = v0 + vectors_per_split < vectors ? v0 + vectors_per_split : vectors;
+    __shared__ A shared[kThreads / kWave];
+    A acc = Op::init();
+    if (split == 0 && tid < head) acc = Op::step(acc, p[tid], tid);
+    for (uint32_t v = v0 + tid; v < v1; v += kThreads) {
+        const Vec<T, VEC> x = load_vec<T, VEC>(p + head + static_cast<size_t>(v) * VEC);
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) acc = Op::step(acc, x.v[i], head + v * VEC + i);
+    }
+    if (split == 0 && end + tid < R) acc = Op::step(acc, p[end + tid], end + tid);
+    acc = wave_reduce<Op>(acc);
+    if (tid % kWave == 0) shared[tid / kWave] = acc;
+    __syncthreads();
+    if (tid == 0) {
+        A total = shared[0];
+        for (int w = 1; w < kThreads / kWave; ++w) total = Op::combine(total, shared[w]);
+        partial[static_cast<size_t>(split) * rows + row] = total;
+    }
+}
+
 // Second pass of the split-R column reduction: folds `splits` partials per slot.
 template <class Op>
 __global__ __launch_bounds__(kThreads) void reduce_finish_kernel(const typename Op::A* partial, typename Op::Out* dst, const typename Op::S* src,
@@ -498,14 +545,39 @@ int run_reduce(const tannic_tensor_t* src, tannic_tensor_t* dst, hipStream_t str
             // rows that fit the registers of one wavefront (four 16-byte pieces per lane)
             if (vec && R <= 8 * kWave * 4 && rows >= 1024) return ArgRows16<Op>::run(ps, pd, rows, static_cast<uint32_t>(R), stream);
         }
+        // a handful of very long rows: several blocks per row and a second pass over their results
+        if (VEC > 1 && rows <= 64 && R >= 16384 && reinterpret_cast<uintptr_t>(ps) % sizeof(T) == 0) {
+            uint32_t splits = static_cast<uint32_t>(R / 4096);
+            if (splits > 64) splits = 64;
+            while (splits > 2 && static_cast<size_t>(splits) * rows > 512) splits /= 2;
+            const uint32_t vectors_per_split = (static_cast<uint32_t>(R / VEC) + splits - 1) / splits;
+            A* partial = nullptr;
+            if (scratch_acquire(reinterpret_cast<void**>(&partial), sizeof(A) * splits * rows, stream) != TANNIC_SUCCESS) return TANNIC_ERROR;
+            hipLaunchKernelGGL((reduce_rows_split_kernel<Op, VEC>), dim3(splits, rows), dim3(kThreads), 0, stream, ps, partial, rows, static_cast<uint32_t>(R),
+                               vectors_per_split);
+            int status = launch_status("reduce_rows_split_kernel");
+            if (status == TANNIC_SUCCESS) {
+                hipLaunchKernelGGL((reduce_finish_kernel<Op>), dim3((rows + kThreads - 1) / kThreads), dim3(kThreads), 0, stream, partial, pd, ps, splits, rows,
+                                   static_cast<uint32_t>(R), 1u);
+                status = launch_status("reduce_finish_kernel");
+            }
+            scratch_release(partial, stream);
+            return status;
+        }
         // few long rows: a whole block per row
         const bool wide = rows < 2048 && R >= 8192;
         const uint32_t grid = wide ? rows : (rows + 3) / 4;
         auto launch = [&](auto kernel) {
             hipLaunchKernelGGL(kernel, dim3(grid), dim3(kThreads), 0, stream, ps, pd, rows, static_cast<uint32_t>(R));
         };
+        // Rows of any start and length still read their aligned middle as vectors when they are long (fp16 sums, us against
+        // element by element: rows of 4097 7.1 / 11.3, of 1025 14.4 / 17.4; of 511 36 / 37, of 197 18.5 / 13.3 - a short row
+        // has too few vectors for a wavefront's lanes, and its two ends wait one after the other).
+        const bool ragged = VEC > 1 && !vec && R >= 1024 && reinterpret_cast<uintptr_t>(ps) % sizeof(T) == 0;
         if (vec && wide) launch(reduce_rows_kernel<Op, VEC, 4>);
         else if (vec) launch(reduce_rows_kernel<Op, VEC, 1>);
+        else if (ragged && wide) launch(reduce_rows_kernel<Op, VEC, 4, true>);
+        else if (ragged) launch(reduce_rows_kernel<Op, VEC, 1, true>);
         else if (wide) launch(reduce_rows_kernel<Op, 1, 4>);
         else launch(reduce_rows_kernel<Op, 1, 1>);
         return launch_status("reduce_rows_kernel");

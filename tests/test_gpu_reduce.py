@@ -24,6 +24,15 @@ SHAPES = {
     "rows_vector": ((512, 1024), 1),
     "rows_odd": ((77, 1001), 1),
     "rows_block_wide": ((3, 40000), 1),
+    # rows that start anywhere / whose length no vector divides: the aligned middle as vectors, its ends one element per lane
+    "rows_odd_1025": ((70, 1025), 1),
+    "rows_odd_2051": ((9, 2051), 1),
+    "rows_odd_block_wide": ((3, 8195), 1),
+    # a handful of very long rows: several blocks per row (vocabulary logits); odd and even lengths, one and many rows
+    "rows_split_one_odd": ((1, 50257), 1),
+    "rows_split_sixteen_odd": ((16, 50257), 1),
+    "rows_split_even": ((5, 32768), 1),
+    "rows_split_long": ((2, 300003), 1),
     "one_row": ((9000,), 0),
     "columns_wide": ((4, 300, 1024), 1),
     "columns_split": ((2, 4096, 256), 1),
