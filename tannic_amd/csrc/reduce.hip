@@ -460,7 +460,24 @@ __global__ __launch_bounds__(kThreads) void reduce_finish_kernel(const typename 
     const uint32_t slot = blockIdx.x * kThreads + threadIdx.x;
     if (slot >= slots) return;
     typename Op::A total = partial[slot];
-    for (uint32_t s = 1; s < splits; ++s) total = Op::combine(total, partial[static_cast<size_t>(s) * slots + slot]);
+    // sixteen partial results are fetched before they are folded (in split order): one after the other, each waiting for
+    // its own load, 64 of them took 16 us
+    uint32_t s = 1;
+    for (; s + 16 <= splits; s += 16) {
+        typename Op::A part[16];
+#pragma unroll
+        for (int k = 0; k < 16; ++k) part[k] = partial[static_cast<size_t>(s + k) * slots + slot];
+#pragma unroll
+        for (int k = 0; k < 16; ++k) total = Op::combine(total, part[k]);
+    }
+    if (s < splits) {
+        typename Op::A part[16];
+#pragma unroll
+        for (int k = 0; k < 16; ++k) part[k] = partial[static_cast<size_t>(s + k < splits ? s + k : s) * slots + slot];
+#pragma unroll
+        for (int k = 0; k < 16; ++k)
+            if (s + k < splits) total = Op::combine(total, part[k]);
+    }
     const uint32_t outer = slot / inner, col = slot % inner;
     emit<Op>(total, R, dst, slot, src, static_cast<size_t>(outer) * R * inner + col, inner);
 }
@@ -609,7 +626,10 @@ int run_reduce(const tannic_tensor_t* src, tannic_tensor_t* dst, hipStream_t str
     const uint32_t gx = (column_groups + TX - 1) / TX;
     uint32_t splits = 1;
     const size_t base_blocks = static_cast<size_t>(gx) * outer;
-    while (base_blocks * splits < 512 && R / (static_cast<size_t>(TY) * splits * 2) >= 16 && splits < 64) splits *= 2;
+    // (down to eight rows per thread: the partial results are then still a sixteenth of the source at most, and a matrix
+    // summed over its rows - one slice, a few thousand columns - gets its two blocks per compute unit: [4097, 4096] fp16
+    // 27 us with 256 blocks)
+    while (base_blocks * splits < 512 && R / (static_cast<size_t>(TY) * splits * 2) >= 4 && splits < 64) splits *= 2;
     A* partial = nullptr;
     if (splits > 1) {
         if (scratch_acquire(reinterpret_cast<void**>(&partial), sizeof(A) * splits * slots, stream) != TANNIC_SUCCESS) return TANNIC_ERROR;
