@@ -406,6 +406,93 @@ int launch_elementwise(F f, Plan p, hipStream_t stream) {
     return launch_status("elementwise_kernel");
 }
 
+// ---- copies that transpose -------------------------------------------------------------------------------------------
+// A copy whose source is contiguous along another dimension than the destination's last one (a transposed matrix made
+// contiguous, [B, S, H, D] read as [B, D, S, H] ...): element by element, either the loads or the stores of a wavefront
+// are a line apart each.  Here a block moves a 64 x 64 tile of those two dimensions through LDS: it reads rows along the
+// source's contiguous dimension and writes rows along the destination's, both as whole lines.  The other dimensions are
+// decoded from the block number.
+struct TransposePlan {
+    int outer;                         // dimensions besides the two of the tile
+    FastDiv div[TANNIC_DIMENSIONS];    // their extents, innermost last
+    int64_t src_stride[TANNIC_DIMENSIONS], dst_stride[TANNIC_DIMENSIONS];
+    uint32_t extent_c, extent_l;       // the source's contiguous dimension, the destination's last one
+    int64_t src_stride_l, dst_stride_c;
+    uint32_t tiles_c, tiles_l;
+};
+
+template <class U>
+__global__ __launch_bounds__(256) void transposed_copy_kernel(const U* src, U* dst, TransposePlan q) {
+    constexpr int TILE = 64;
+    __shared__ U tile[TILE][TILE + 1];
+    uint32_t rest = blockIdx.x;
+    const uint32_t tc = rest % q.tiles_c;
+    rest /= q.tiles_c;
+    const uint32_t tl = rest % q.tiles_l;
+    rest /= q.tiles_l;
+    int64_t from = 0, to = 0;
+    for (int d = q.outer - 1; d >= 0; --d) {
+        uint32_t next, c;
+        q.div[d].divmod(rest, next, c);
+        rest = next;
+        from += static_cast<int64_t>(c) * q.src_stride[d];
+        to += static_cast<int64_t>(c) * q.dst_stride[d];
+    }
+    const uint32_t c0 = tc * TILE, l0 = tl * TILE, tx = threadIdx.x % TILE, ty = threadIdx.x / TILE;
+#pragma unroll 4
+    for (int i = 0; i < TILE; i += 4) {
+        const uint32_t c = c0 + tx, l = l0 + ty + i;
+        if (c < q.extent_c && l < q.extent_l) tile[ty + i][tx] = src[from + c + static_cast<int64_t>(l) * q.src_stride_l];
+    }
+    __syncthreads();
+#pragma unroll 4
+    for (int i = 0; i < TILE; i += 4) {
+        const uint32_t l = l0 + tx, c = c0 + ty + i;
+        if (c < q.extent_c && l < q.extent_l) dst[to + l + static_cast<int64_t>(c) * q.dst_stride_c] = tile[tx][ty + i];
+    }
+}
+
+// Runs the copy described by `p` (operand 0 the source, operand 2 the destination) through the tiles above when it is one
+// of those; TANNIC_UNSUPPORTED_DTYPE otherwise.  U: an unsigned type (or 16-byte struct) of the element's size.
+template <class U>
+inline int transposed_copy(const Plan& p, const void* src, void* dst, hipStream_t stream) {
+    const int last = p.rank - 1;
+    if (p.rank < 2 || p.stride[2][last] != 1 || p.stride[0][last] == 1 || p.stride[0][last] == 0) return TANNIC_UNSUPPORTED_DTYPE;
+    int c = -1;
+    for (int d = last - 1; d >= 0; --d)
+        if (p.stride[0][d] == 1) { c = d; break; }
+    if (c < 0 || p.extent[c] < 16 || p.extent[last] < 16) return TANNIC_UNSUPPORTED_DTYPE;
+    TransposePlan q{};
+    uint64_t blocks = 1;
+    for (int d = 0; d < last; ++d) {
+        if (d == c) continue;
+        q.div[q.outer] = p.div[d];
+        q.src_stride[q.outer] = p.stride[0][d];
+        q.dst_stride[q.outer] = p.stride[2][d];
+        ++q.outer;
+        blocks *= p.extent[d];
+    }
+    q.extent_c = p.extent[c];
+    q.extent_l = p.extent[last];
+    q.src_stride_l = p.stride[0][last];
+    q.dst_stride_c = p.stride[2][c];
+    q.tiles_c = (q.extent_c + 63) / 64;
+    q.tiles_l = (q.extent_l + 63) / 64;
+    blocks *= static_cast<uint64_t>(q.tiles_c) * q.tiles_l;
+    if (blocks == 0) return TANNIC_SUCCESS;
+    if (blocks >= (1ull << 31)) return TANNIC_UNSUPPORTED_DTYPE;
+    hipLaunchKernelGGL((transposed_copy_kernel<U>), dim3(static_cast<uint32_t>(blocks)), dim3(256), 0, stream, static_cast<const U*>(src), static_cast<U*>(dst), q);
+    return launch_status("transposed_copy_kernel");
+}
+
+template <int BYTES> struct BitsOf;
+template <> struct BitsOf<1> { using type = uint8_t; };
+template <> struct BitsOf<2> { using type = uint16_t; };
+template <> struct BitsOf<4> { using type = uint32_t; };
+template <> struct BitsOf<8> { using type = uint64_t; };
+struct alignas(16) SixteenBytes { uint64_t lo, hi; };
+template <> struct BitsOf<16> { using type = SixteenBytes; };
+
 // Strides of `t` right-aligned on a destination of `rank` dims with `extent`;
 // size-1 dims (and missing leading dims) get stride 0
 // (src/cpu/ops-binary.cpp:89-95).

@@ -79,6 +79,8 @@ int run_cpy(const tannic_tensor_t* src, tannic_tensor_t* dst, hipStream_t stream
         set_error_text("elementwise: tensors of 2^31 elements or more are not supported");
         return TANNIC_ERROR;
     }
+    const int tiled = transposed_copy<typename BitsOf<sizeof(T)>::type>(plan, src->address, dst->address, stream);
+    if (tiled != TANNIC_UNSUPPORTED_DTYPE) return tiled;
     CopyF<T> f{static_cast<const T*>(src->address), nullptr, static_cast<T*>(dst->address)};
     return launch_elementwise(f, plan, stream);
 }

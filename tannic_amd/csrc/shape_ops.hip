@@ -115,17 +115,35 @@ template <class U>
 __global__ __launch_bounds__(256) void concat_kernel(const U* a, const U* b, U* dst, ConcatPlan q) {
     const uint32_t idx = blockIdx.x * 256 + threadIdx.x;
     if (idx >= q.total) return;
-    uint32_t rest = idx, coord[8];
+    // both sources' offsets are formed on the way through the dimensions (no coordinate array: one indexed by the axis
+    // would live in scratch memory)
+    uint32_t rest = idx;
+    int64_t off_a = 0, off_b = 0;
+    bool second = false;
     for (int d = q.rank - 1; d >= 0; --d) {
-        uint32_t next;
-        q.div[d].divmod(rest, next, coord[d]);
+        uint32_t next, c;
+        q.div[d].divmod(rest, next, c);
         rest = next;
+        uint32_t cb = c;
+        if (d == q.axis) {
+            second = c >= q.first_extent;
+            cb = c - q.first_extent;
+        }
+        off_a += static_cast<int64_t>(c) * q.stride_a[d];
+        off_b += static_cast<int64_t>(cb) * q.stride_b[d];
     }
-    const bool second = coord[q.axis] >= q.first_extent;
-    if (second) coord[q.axis] -= q.first_extent;
-    int64_t off = 0;
-    for (int d = 0; d < q.rank; ++d) off += static_cast<int64_t>(coord[d]) * (second ? q.stride_b[d] : q.stride_a[d]);
-    dst[idx] = second ? b[off] : a[off];
+    dst[idx] = second ? b[off_b] : a[off_a];
+}
+
+// Both sources contiguous, and what each contributes to a row of the result (its extent along the axis times everything
+// behind the axis) a whole number of 16-byte pieces: the result is, outer index by outer index, a run of `a` followed by a
+// run of `b` (appending to a key / value cache).  A thread moves one piece.
+__global__ __launch_bounds__(256) void concat_runs_kernel(const uint4* a, const uint4* b, uint4* dst, uint32_t run_a, uint32_t run_b, FastDiv row, uint32_t total) {
+    const uint32_t idx = blockIdx.x * 256 + threadIdx.x;
+    if (idx >= total) return;
+    uint32_t outer, at;
+    row.divmod(idx, outer, at);
+    dst[idx] = at < run_a ? a[static_cast<size_t>(outer) * run_a + at] : b[static_cast<size_t>(outer) * run_b + (at - run_a)];
 }
 
 int run_concat(const tannic_tensor_t* a, const tannic_tensor_t* b, tannic_tensor_t* dst, int axis, hipStream_t stream) {
@@ -164,6 +182,20 @@ int run_concat(const tannic_tensor_t* a, const tannic_tensor_t* b, tannic_tensor
     q.axis = axis;
     q.total = static_cast<uint32_t>(total);
     q.first_extent = static_cast<uint32_t>(a->shape.sizes[axis]);
+    {
+        size_t behind = 1;
+        for (int d = axis + 1; d < rank; ++d) behind *= a->shape.sizes[d];
+        const size_t bytes_a = a->shape.sizes[axis] * behind * esize, bytes_b = b->shape.sizes[axis] * behind * esize;
+        auto at16 = [](const void* ptr) { return reinterpret_cast<uintptr_t>(ptr) % 16 == 0; };
+        if (a->layout == TANNIC_CONTIGUOUS && b->layout == TANNIC_CONTIGUOUS && bytes_a % 16 == 0 && bytes_b % 16 == 0 && at16(a->address) && at16(b->address) &&
+            at16(dst->address)) {
+            const uint32_t run_a = static_cast<uint32_t>(bytes_a / 16), run_b = static_cast<uint32_t>(bytes_b / 16);
+            const uint32_t pieces = static_cast<uint32_t>(total * esize / 16);
+            hipLaunchKernelGGL(concat_runs_kernel, dim3((pieces + 255) / 256), dim3(256), 0, stream, static_cast<const uint4*>(a->address),
+                               static_cast<const uint4*>(b->address), static_cast<uint4*>(dst->address), run_a, run_b, FastDiv(run_a + run_b), pieces);
+            return launch_status("concat_runs_kernel");
+        }
+    }
     const dim3 grid((q.total + 255) / 256);
     switch (esize) {
         case 1: hipLaunchKernelGGL((concat_kernel<uint8_t>), grid, dim3(256), 0, stream, static_cast<const uint8_t*>(a->address), static_cast<const uint8_t*>(b->address), static_cast<uint8_t*>(dst->address), q); break;

@@ -103,6 +103,11 @@ int run_unary(const tannic_tensor_t* src, tannic_tensor_t* dst, hipStream_t stre
         set_error_text("elementwise: tensors of 2^31 elements or more are not supported");
         return TANNIC_ERROR;
     }
+    if constexpr (K == U_CPY) {
+        // a source that is contiguous along another dimension than the last: tiles through LDS
+        const int tiled = transposed_copy<typename BitsOf<sizeof(T)>::type>(plan, src->address, dst->address, stream);
+        if (tiled != TANNIC_UNSUPPORTED_DTYPE) return tiled;
+    }
     // operand 1 is unused: give it the source's strides so that it never blocks merging
     UnaryF<T, K> f{static_cast<const T*>(src->address), nullptr, static_cast<T*>(dst->address), eps};
     return launch_elementwise(f, plan, stream);

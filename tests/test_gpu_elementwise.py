@@ -150,6 +150,31 @@ def test_neg_repack_abs_other_types(device, dtype):
             support.assert_bit_exact(getattr(ops, op)(dv).storage(), getattr(ops, op)(hv).storage(), f"{op} {dtype}")
 
 
+TRANSPOSING_COPIES = {
+    "matrix": ((130, 70), [("transpose", (0, 1))]),
+    "matrix_ragged_tiles": ((65, 193), [("transpose", (0, 1))]),
+    "batched_matrices": ((5, 40, 72), [("transpose", (1, 2))]),
+    "heads_to_front_of_columns": ((2, 33, 4, 20), [("permute", (0, 3, 1, 2))]),
+    "nchw_as_nhwc": ((3, 17, 9, 21), [("permute", (0, 2, 3, 1))]),
+    "first_axis_last": ((40, 3, 50), [("permute", (1, 2, 0))]),
+    "column_slice_of_a_transposed_matrix": ((90, 64), [("transpose", (0, 1)), ("index", (slice(3, 60), slice(5, 88)))]),
+}
+
+
+@pytest.mark.parametrize("name", list(TRANSPOSING_COPIES))
+@pytest.mark.parametrize("dtype", [ta.int8, ta.float16, ta.float32, ta.float64, ta.complex128], ids=str)
+def test_repack_of_views_that_are_contiguous_along_another_dimension(device, dtype, name):
+    """Copies whose source runs contiguously along another dimension than the result's last one move 64 x 64 tiles
+    through LDS: tiles that end inside the matrix, batches before and between the two dimensions, views that start
+    inside the storage, every element size."""
+    shape, spec = TRANSPOSING_COPIES[name]
+    h, d = pair_of(dtype, 12, shape, device, -100, 100)
+    hv, dv = support.apply_view(h, spec), support.apply_view(d, spec)
+    want, got = ops.repack(hv), ops.repack(dv)
+    assert got.shape == want.shape
+    support.assert_bit_exact(got.storage(), want.storage(), f"repack {name} {dtype}")
+
+
 @pytest.mark.parametrize("view", ["contiguous", "transposed", "singleton"])
 @pytest.mark.parametrize("dtype", INTS + FLOATS, ids=str)
 def test_scale(device, dtype, view):
