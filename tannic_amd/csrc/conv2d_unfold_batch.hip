@@ -59,7 +59,7 @@ static int run_unfold_batch(const ConvProblem& p, int dtype, const void* x, cons
     const uint32_t pitch = static_cast<uint32_t>((pixels + E - 1) / E * E);
     const uint64_t columns = static_cast<uint64_t>(p.N) * pitch;
     if (columns < 256 || columns >= (1ull << 31) || K * p.N * (pitch / E) >= (1ull << 31)) return TANNIC_UNSUPPORTED_DTYPE;
-    if (K * columns * sizeof(T) > ((ANY_SIZE ? 128ull : 512ull) << 20)) return TANNIC_UNSUPPORTED_DTYPE;
+    if (K * columns * sizeof(T) > ((ANY_SIZE ? 256ull : 512ull) << 20)) return TANNIC_UNSUPPORTED_DTYPE;
     // the kernel tensor as a K-contiguous O x K matrix, the result as pixel-contiguous rows
     if (p.ws[3] != 1 || p.ws[2] != static_cast<int64_t>(p.KW) || p.ws[1] != static_cast<int64_t>(p.KH) * p.KW || p.ws[0] != static_cast<int64_t>(K) ||
         reinterpret_cast<uintptr_t>(w) % 16 != 0)

@@ -663,7 +663,6 @@ int run16(const GemmProblem& p, const void* a, const void* b, void* c, hipStream
         // An extent, a row pitch or an address that is odd: the loaders fetch their 16-byte pieces at whatever address they
         // lie (only the piece that straddles the end of a row is gathered element by element) and the product stays on the
         // matrix cores.
-        if (p.row_bias) return TANNIC_UNSUPPORTED_DTYPE;
         if (ak && bk) {
             if (p.M > 64) return launch16<T, 128, 128, 2, true, true, false, false>(p, a, b, c, stream);
             return launch16<T, 64, 128, 2, true, true, false, false>(p, a, b, c, stream);

@@ -97,6 +97,10 @@ CASES = {
     "k1_14x14_many_images": ((7, 64, 14, 14), (136, 64, 1, 1), (1, 1), (0, 0)),
     "k1_7x7_one_channel_out": ((5, 72, 7, 7), (1, 72, 1, 1), (1, 1), (0, 0)),
     "k1_13x13_c8": ((3, 8, 13, 13), (520, 8, 1, 1), (1, 1), (0, 0)),
+    # channel counts that are not a multiple of 16 bytes over aligned pixel counts: the product per image with rows of weights
+    # that start anywhere
+    "k1_c100_28x28": ((3, 100, 28, 28), (200, 100, 1, 1), (1, 1), (0, 0)),
+    "k1_c7_8x8": ((5, 7, 8, 8), (33, 7, 1, 1), (1, 1), (0, 0)),
     # few output pixels per image under a long K: the whole batch unfolded side by side, one product
     "unfolded_k3_7x7": ((5, 128, 7, 7), (40, 128, 3, 3), (1, 1), (1, 1)),
     "unfolded_k3_s2_14_to_7": ((6, 64, 14, 14), (48, 64, 3, 3), (2, 2), (1, 1)),
