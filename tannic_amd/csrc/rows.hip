@@ -163,6 +163,45 @@ __global__ __launch_bounds__(kRowBlock) void softmax_kernel(const T* x, const T*
     }
 }
 
+// Rows of up to 64 * NE elements whose length or start no 16-byte access fits (attention over 197 or 1025 positions): a
+// wavefront per row, a lane holding elements lane, lane + 64, ...: one read of the row, single-element accesses that a
+// wavefront still makes as whole lines.
+template <class T, int NE, bool MASK>
+__global__ __launch_bounds__(kRowBlock) void softmax_wave_kernel(const T* x, const T* mask, T* y, uint32_t rows, uint32_t L, FastDiv q, float scale) {
+    using A = RowAcc<T>;
+    const uint32_t lane = threadIdx.x % 64, row = blockIdx.x * (kRowBlock / 64) + threadIdx.x / 64;
+    if (row >= rows) return;   // whole wavefronts; nothing below synchronises across them
+    const size_t base = static_cast<size_t>(row) * L;
+    uint32_t mrow = 0, quotient = 0;
+    if (MASK) q.divmod(row, quotient, mrow);
+    A s[NE];
+    A top = -INFINITY;
+#pragma unroll
+    for (int e = 0; e < NE; ++e) {
+        const uint32_t i = lane + 64 * e;
+        s[e] = -INFINITY;
+        if (i < L) {
+            s[e] = static_cast<A>(widen(x[base + i])) * static_cast<A>(scale);
+            if (MASK) s[e] += static_cast<A>(widen(mask[static_cast<size_t>(mrow) * L + i]));
+        }
+        top = MaxOp::combine(top, s[e]);
+    }
+    top = wave_reduce<MaxOp>(top);
+    A sum = 0;
+#pragma unroll
+    for (int e = 0; e < NE; ++e) {
+        s[e] = lane + 64 * e < L ? fast_exp(s[e] - top, is_16bit<T>::value) : A(0);
+        sum += s[e];
+    }
+    sum = wave_reduce<AddOp>(sum);
+    const A inv = A(1) / sum;
+#pragma unroll
+    for (int e = 0; e < NE; ++e)
+        if (lane + 64 * e < L) y[base + lane + 64 * e] = narrow<T>(s[e] * inv);
+}
+
+// any length, any alignment: one block per row, the row read three times (from cache after the first), four elements of a
+// thread on their way at a time
 template <class T, bool MASK>
 __global__ __launch_bounds__(kRowBlock) void softmax_any_kernel(const T* x, const T* mask, T* y, uint32_t L, FastDiv q, float scale) {
     using A = RowAcc<T>;
@@ -176,14 +215,35 @@ __global__ __launch_bounds__(kRowBlock) void softmax_any_kernel(const T* x, cons
         if (MASK) a += static_cast<A>(widen(mk[i]));
         return a;
     };
+    // four values at i, i + 256, ... (-inf past the end of the row)
+    auto four = [&](uint32_t i, A (&v)[4]) {
+#pragma unroll
+        for (int u = 0; u < 4; ++u) v[u] = i + u * kRowBlock < L ? value(i + u * kRowBlock) : static_cast<A>(-INFINITY);
+    };
     A top = -INFINITY;
-    for (uint32_t i = threadIdx.x; i < L; i += kRowBlock) top = MaxOp::combine(top, value(i));
+    for (uint32_t i = threadIdx.x; i < L; i += 4 * kRowBlock) {
+        A v[4];
+        four(i, v);
+#pragma unroll
+        for (int u = 0; u < 4; ++u) top = MaxOp::combine(top, v[u]);
+    }
     top = group_reduce<MaxOp, kRowBlock>(top, lds);
     A sum = 0;
-    for (uint32_t i = threadIdx.x; i < L; i += kRowBlock) sum += fast_exp(value(i) - top, is_16bit<T>::value);
+    for (uint32_t i = threadIdx.x; i < L; i += 4 * kRowBlock) {
+        A v[4];
+        four(i, v);
+#pragma unroll
+        for (int u = 0; u < 4; ++u) sum += i + u * kRowBlock < L ? fast_exp(v[u] - top, is_16bit<T>::value) : A(0);
+    }
     sum = group_reduce<AddOp, kRowBlock>(sum, lds);
     const A inv = A(1) / sum;
-    for (uint32_t i = threadIdx.x; i < L; i += kRowBlock) y[base + i] = narrow<T>(fast_exp(value(i) - top, is_16bit<T>::value) * inv);
+    for (uint32_t i = threadIdx.x; i < L; i += 4 * kRowBlock) {
+        A v[4];
+        four(i, v);
+#pragma unroll
+        for (int u = 0; u < 4; ++u)
+            if (i + u * kRowBlock < L) y[base + i + u * kRowBlock] = narrow<T>(fast_exp(v[u] - top, is_16bit<T>::value) * inv);
+    }
 }
 
 // ---- rotary embedding -----------------------------------------------------------------
@@ -354,6 +414,19 @@ int run_softmax(const tannic_tensor_t* x, const tannic_tensor_t* mask, tannic_te
     if (L % VEC == 0 && aligned16(px) && aligned16(pm) && aligned16(py) && row_shape(L / VEC, rows, group, nch)) {
         if (group == 64) return pick_softmax<T, 64>(nch, px, pm, py, rows, L, Q, scale, stream);
         return pick_softmax<T, kRowBlock>(nch, px, pm, py, rows, L, Q, scale, stream);
+    }
+    if (L <= 64 * 32 && rows >= 256) {
+        // short rows that the vector kernel cannot take: a wavefront per row
+        const dim3 grid((rows + kRowBlock / 64 - 1) / (kRowBlock / 64));
+        auto launch = [&](auto with_mask, auto without) {
+            if (pm) hipLaunchKernelGGL(with_mask, grid, dim3(kRowBlock), 0, stream, px, pm, py, rows, L, FastDiv(Q), scale);
+            else hipLaunchKernelGGL(without, grid, dim3(kRowBlock), 0, stream, px, pm, py, rows, L, FastDiv(1), scale);
+        };
+        if (L <= 64 * 4) launch(softmax_wave_kernel<T, 4, true>, softmax_wave_kernel<T, 4, false>);
+        else if (L <= 64 * 8) launch(softmax_wave_kernel<T, 8, true>, softmax_wave_kernel<T, 8, false>);
+        else if (L <= 64 * 16) launch(softmax_wave_kernel<T, 16, true>, softmax_wave_kernel<T, 16, false>);
+        else launch(softmax_wave_kernel<T, 32, true>, softmax_wave_kernel<T, 32, false>);
+        return launch_status("softmax_wave_kernel");
     }
     if (pm) hipLaunchKernelGGL((softmax_any_kernel<T, true>), dim3(rows), dim3(kRowBlock), 0, stream, px, pm, py, L, FastDiv(Q), scale);
     else hipLaunchKernelGGL((softmax_any_kernel<T, false>), dim3(rows), dim3(kRowBlock), 0, stream, px, pm, py, L, FastDiv(1), scale);

@@ -226,7 +226,9 @@ def causal(n, dtype):
     return np.where(np.tril(np.ones((n, n), dtype=bool)), 0.0, -np.inf).astype(np.float32)
 
 
-SOFTMAX_SHAPES = [(4, 64), (3, 40, 512), (2, 4, 128, 128), (1300, 200), (5, 4096), (3, 37), (2, 1028), (2, 70000)]
+# the last five: rows no 16-byte access fits, a wavefront per row (4, 8, 16 and 32 elements per lane), and too few of them for that
+SOFTMAX_SHAPES = [(4, 64), (3, 40, 512), (2, 4, 128, 128), (1300, 200), (5, 4096), (3, 37), (2, 1028), (2, 70000),
+                  (300, 197), (2, 130, 511), (260, 1025), (257, 2047), (100, 197)]
 
 
 @pytest.mark.parametrize("shape", SOFTMAX_SHAPES, ids=str)
@@ -243,7 +245,7 @@ def test_softmax(device, dtype, shape):
     np.testing.assert_allclose(f64(got).sum(axis=-1), 1.0, rtol=0, atol=shape[-1] * ROUNDING[dtype])
 
 
-@pytest.mark.parametrize("n", [16, 128, 512, 100])
+@pytest.mark.parametrize("n", [16, 128, 512, 100, 197])
 @pytest.mark.parametrize("dtype", [ta.float16, ta.bfloat16, ta.float32], ids=str)
 def test_softmax_causal_mask(device, dtype, n):
     x = values(dtype, 19, (2, 3, n, n), -8.0, 8.0)
