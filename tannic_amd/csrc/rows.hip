@@ -246,6 +246,76 @@ __global__ __launch_bounds__(kRowBlock) void softmax_any_kernel(const T* x, cons
     }
 }
 
+// A few very long rows (the probabilities of a vocabulary's logits, one row per sequence): one block per row leaves the
+// chip idle and walks the row three times.  Here a row is shared by gridDim.x blocks.  The first kernel leaves, per block,
+// the largest value of its range and the sum of exp(value - that); the second combines a row's pairs (every block for
+// itself: they are few) into the row's maximum and sum and writes its range.
+template <class T, bool MASK>
+__global__ __launch_bounds__(kRowBlock) void softmax_shared_rows_first_kernel(const T* x, const T* mask, RowAcc<T>* partial, uint32_t L, FastDiv q, float scale,
+                                                                              uint32_t per_block) {
+    using A = RowAcc<T>;
+    __shared__ A lds[4];
+    const uint32_t row = blockIdx.y, first = blockIdx.x * per_block, end = first + per_block < L ? first + per_block : L;
+    const size_t base = static_cast<size_t>(row) * L;
+    uint32_t mrow = 0, quotient = 0;
+    if (MASK) q.divmod(row, quotient, mrow);
+    const T* mk = MASK ? mask + static_cast<size_t>(mrow) * L : nullptr;
+    auto value = [&](uint32_t i) {
+        A a = static_cast<A>(widen(x[base + i])) * static_cast<A>(scale);
+        if (MASK) a += static_cast<A>(widen(mk[i]));
+        return a;
+    };
+    A top = -INFINITY;
+    for (uint32_t i = first + threadIdx.x; i < end; i += 4 * kRowBlock) {
+        A v[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) v[u] = i + u * kRowBlock < end ? value(i + u * kRowBlock) : static_cast<A>(-INFINITY);
+#pragma unroll
+        for (int u = 0; u < 4; ++u) top = MaxOp::combine(top, v[u]);
+    }
+    top = group_reduce<MaxOp, kRowBlock>(top, lds);
+    A sum = 0;
+    for (uint32_t i = first + threadIdx.x; i < end; i += 4 * kRowBlock) {
+        A v[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) v[u] = i + u * kRowBlock < end ? value(i + u * kRowBlock) : static_cast<A>(-INFINITY);
+#pragma unroll
+        for (int u = 0; u < 4; ++u) sum += i + u * kRowBlock < end ? fast_exp(v[u] - top, is_16bit<T>::value) : A(0);
+    }
+    sum = group_reduce<AddOp, kRowBlock>(sum, lds);
+    if (threadIdx.x == 0) {
+        A* out = partial + (static_cast<size_t>(row) * gridDim.x + blockIdx.x) * 2;
+        out[0] = top;
+        out[1] = top == static_cast<A>(-INFINITY) ? A(0) : sum;   // a range of -inf only: nothing to add (its own sum is NaN)
+    }
+}
+
+template <class T, bool MASK>
+__global__ __launch_bounds__(kRowBlock) void softmax_shared_rows_second_kernel(const T* x, const T* mask, T* y, const RowAcc<T>* partial, uint32_t L, FastDiv q,
+                                                                               float scale, uint32_t per_block) {
+    using A = RowAcc<T>;
+    const uint32_t row = blockIdx.y, first = blockIdx.x * per_block, end = first + per_block < L ? first + per_block : L;
+    const size_t base = static_cast<size_t>(row) * L;
+    // the row's maximum and sum from its blocks' pairs (at most 64 of them: a lane each, every wavefront for itself)
+    const uint32_t lane = threadIdx.x % 64;
+    const A* pairs = partial + static_cast<size_t>(row) * gridDim.x * 2;
+    const A my_top = lane < gridDim.x ? pairs[2 * lane] : static_cast<A>(-INFINITY);
+    const A my_sum = lane < gridDim.x ? pairs[2 * lane + 1] : A(0);
+    const A top = wave_reduce<MaxOp>(my_top);
+    // a block whose range held nothing above -inf contributes nothing; a row of -inf only has the sum 0 and, from
+    // exp(-inf - -inf) below, NaN everywhere, as the definition has it
+    const A sum = wave_reduce<AddOp>(my_top == static_cast<A>(-INFINITY) ? A(0) : my_sum * fast_exp(my_top - top, false));
+    const A inv = A(1) / sum;
+    uint32_t mrow = 0, quotient = 0;
+    if (MASK) q.divmod(row, quotient, mrow);
+    const T* mk = MASK ? mask + static_cast<size_t>(mrow) * L : nullptr;
+    for (uint32_t i = first + threadIdx.x; i < end; i += kRowBlock) {
+        A a = static_cast<A>(widen(x[base + i])) * static_cast<A>(scale);
+        if (MASK) a += static_cast<A>(widen(mk[i]));
+        y[base + i] = narrow<T>(fast_exp(a - top, is_16bit<T>::value) * inv);
+    }
+}
+
 // ---- rotary embedding -----------------------------------------------------------------
 struct RopeMap {
     int outer;                              // dims in front of the last one
@@ -414,6 +484,26 @@ int run_softmax(const tannic_tensor_t* x, const tannic_tensor_t* mask, tannic_te
     if (L % VEC == 0 && aligned16(px) && aligned16(pm) && aligned16(py) && row_shape(L / VEC, rows, group, nch)) {
         if (group == 64) return pick_softmax<T, 64>(nch, px, pm, py, rows, L, Q, scale, stream);
         return pick_softmax<T, kRowBlock>(nch, px, pm, py, rows, L, Q, scale, stream);
+    }
+    if (rows <= 64 && L >= 16384) {
+        // a handful of very long rows: up to 64 blocks per row, two kernels
+        uint32_t splits = L / 4096;
+        if (splits > 64) splits = 64;
+        while (splits > 2 && splits * rows > 1024) splits /= 2;
+        const uint32_t per_block = (L + splits - 1) / splits;
+        RowAcc<T>* partial = nullptr;
+        if (scratch_acquire(reinterpret_cast<void**>(&partial), sizeof(RowAcc<T>) * 2 * splits * rows, stream) != TANNIC_SUCCESS) return TANNIC_ERROR;
+        const dim3 grid(splits, rows);
+        if (pm) hipLaunchKernelGGL((softmax_shared_rows_first_kernel<T, true>), grid, dim3(kRowBlock), 0, stream, px, pm, partial, L, FastDiv(Q), scale, per_block);
+        else hipLaunchKernelGGL((softmax_shared_rows_first_kernel<T, false>), grid, dim3(kRowBlock), 0, stream, px, pm, partial, L, FastDiv(1), scale, per_block);
+        int status = launch_status("softmax_shared_rows_first_kernel");
+        if (status == TANNIC_SUCCESS) {
+            if (pm) hipLaunchKernelGGL((softmax_shared_rows_second_kernel<T, true>), grid, dim3(kRowBlock), 0, stream, px, pm, py, partial, L, FastDiv(Q), scale, per_block);
+            else hipLaunchKernelGGL((softmax_shared_rows_second_kernel<T, false>), grid, dim3(kRowBlock), 0, stream, px, pm, py, partial, L, FastDiv(1), scale, per_block);
+            status = launch_status("softmax_shared_rows_second_kernel");
+        }
+        scratch_release(partial, stream);
+        return status;
     }
     if (L <= 64 * 32 && rows >= 256) {
         // short rows that the vector kernel cannot take: a wavefront per row

@@ -228,7 +228,9 @@ def causal(n, dtype):
 
 # the last five: rows no 16-byte access fits, a wavefront per row (4, 8, 16 and 32 elements per lane), and too few of them for that
 SOFTMAX_SHAPES = [(4, 64), (3, 40, 512), (2, 4, 128, 128), (1300, 200), (5, 4096), (3, 37), (2, 1028), (2, 70000),
-                  (300, 197), (2, 130, 511), (260, 1025), (257, 2047), (100, 197)]
+                  (300, 197), (2, 130, 511), (260, 1025), (257, 2047), (100, 197),
+                  # a handful of very long rows shared by several blocks: odd and even lengths, one and many rows
+                  (1, 50257), (16, 50257), (3, 32768), (64, 16385)]
 
 
 @pytest.mark.parametrize("shape", SOFTMAX_SHAPES, ids=str)
@@ -276,6 +278,22 @@ def test_softmax_fully_masked_row_is_nan(device):
     got = ops.softmax(ta.tensor(x, ta.float32, device), ta.tensor(m, ta.float32, device)).numpy()
     np.testing.assert_array_equal(got[0], np.float32(1.0 / 64))
     assert np.isnan(got[1]).all()
+
+
+def test_softmax_over_long_rows_with_masked_ranges(device):
+    """Rows shared by several blocks: a block whose whole range is masked adds nothing, a row masked everywhere is NaN, and
+    the other entries are what the definition gives."""
+    length = 40000
+    x = values(ta.float32, 23, (3, length), -4.0, 4.0)
+    m = np.zeros((3, length), dtype=np.float32)
+    m[0, :20000] = -np.inf      # the first blocks of row 0 see -inf only
+    m[1, 12345:] = -np.inf
+    m[2] = -np.inf
+    got = ops.softmax(ta.tensor(x, ta.float32, device), ta.tensor(m, ta.float32, device)).numpy().astype(np.float64)
+    want = softmax_definition(x[:2], m[:2], 1.0)
+    np.testing.assert_allclose(got[:2], want, rtol=2e-5, atol=1e-12)
+    assert (got[0, :20000] == 0.0).all() and (got[1, 12345:] == 0.0).all()
+    assert np.isnan(got[2]).all()
 
 
 @pytest.mark.parametrize("dtype", [ta.float16, ta.bfloat16], ids=str)
