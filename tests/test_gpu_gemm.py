@@ -128,11 +128,12 @@ def test_integer_gemm_bit_exact(device, pair, layout):
 
 
 @pytest.mark.parametrize("shape", [((300, 256), (520, 256)), ((16, 300, 128), (16, 520, 128)), ((50, 264, 128), (50, 264, 128)), ((2, 3, 70, 384), (136, 384)),
-                                   ((4096, 512), (1024, 512))], ids=lambda s: "x".join(map(str, s[0])) + "." + "x".join(map(str, s[1])) + "T")
+                                   ((4096, 512), (1024, 512)), ((1, 512), (1024, 512)), ((16, 256), (130, 256)), ((3, 5, 128), (3, 70, 128))],
+                         ids=lambda s: "x".join(map(str, s[0])) + "." + "x".join(map(str, s[1])) + "T")
 def test_int8_gemm_on_matrix_cores_is_bit_exact(device, shape):
     """int8 x int8 -> int32 with both operands K-contiguous and K a multiple of 128: the tiled kernels on
     v_mfma_i32_16x16x64_i8 in each tile size (128 x 128, 256 x 128, 256 x 256; ragged rows and columns, batches, a
-    broadcast second operand).  Integer sums are exact, so the checker's sequential loop and numpy agree bit for bit."""
+    broadcast second operand; one, five and sixteen rows in a 128-row tile).  Integer sums are exact, so the checker's sequential loop and numpy agree bit for bit."""
     sa, sb = shape
     a = support.integers(SEED, 31, sa, -128, 128).astype(np.int8)
     b = support.integers(SEED, 32, sb, -128, 128).astype(np.int8)
