@@ -211,15 +211,24 @@ int gemm_entry(const tannic_tensor_t* a, const tannic_tensor_t* b, tannic_tensor
                 GemmProblem p;
                 status = describe_gemm(a, b, dst, p);
                 if (status != TANNIC_SUCCESS) return;
-                if constexpr (std::is_same_v<A, B> && is_16bit<A>::value) {
-                    status = gemm_mfma_16bit(p, a->dtype, a->address, b->address, dst->address, s, workspace);
-                    if (status != TANNIC_UNSUPPORTED_DTYPE) return;
-                } else if constexpr (std::is_same_v<A, int8_t> && std::is_same_v<B, int8_t>) {
-                    status = gemm_mfma_int8(p, a->address, b->address, dst->address, s);
-                    if (status != TANNIC_UNSUPPORTED_DTYPE) return;
-                } else if constexpr (std::is_same_v<A, float> && std::is_same_v<B, float>) {
-                    status = gemm_mfma_f32(p, static_cast<const float*>(a->address), static_cast<const float*>(b->address),
-                                           static_cast<float*>(dst->address), s, workspace);
+                constexpr bool tiled = std::is_same_v<A, B> && (is_16bit<A>::value || std::is_same_v<A, int8_t> || std::is_same_v<A, float>);
+                if constexpr (tiled) {
+                    // operands that do not lie as the tiled kernels want them are copied first when that pays (never on the
+                    // path that must not allocate)
+                    GemmProblem q;
+                    const void *pa = a->address, *pb = b->address;
+                    void* held[2] = {nullptr, nullptr};
+                    const int repacked = gemm_repack(p, sizeof(A), a->address, b->address, s, workspace == nullptr, q, pa, pb, held);
+                    if (repacked == TANNIC_ERROR) {
+                        status = TANNIC_ERROR;
+                        return;
+                    }
+                    const GemmProblem& use = repacked == TANNIC_SUCCESS ? q : p;
+                    if constexpr (is_16bit<A>::value) status = gemm_mfma_16bit(use, a->dtype, pa, pb, dst->address, s, workspace);
+                    else if constexpr (std::is_same_v<A, int8_t>) status = gemm_mfma_int8(use, pa, pb, dst->address, s);
+                    else status = gemm_mfma_f32(use, static_cast<const float*>(pa), static_cast<const float*>(pb), static_cast<float*>(dst->address), s, workspace);
+                    for (void* h : held)
+                        if (h) scratch_release(h, s);
                     if (status != TANNIC_UNSUPPORTED_DTYPE) return;
                 }
                 status = run_generic<A, B, D>(p, a->address, b->address, dst->address, s);

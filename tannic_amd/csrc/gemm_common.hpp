@@ -87,6 +87,10 @@ int gemm_skinny_16bit(const GemmProblem& p, int dtype, const void* a, const void
 int gemm_skinny_f32(const GemmProblem& p, const float* a, const float* b, float* c, hipStream_t stream);
 int gemm_mfma_16bit(const GemmProblem& p, int dtype, const void* a, const void* b, void* c, hipStream_t stream, const GemmWorkspace* workspace = nullptr);
 int gemm_mfma_f32(const GemmProblem& p, const float* a, const float* b, float* c, hipStream_t stream, const GemmWorkspace* workspace = nullptr);
+// Operands that do not lie as the tiled kernels want them, copied into dense K-contiguous rows (gemm_repack.hip).  SUCCESS:
+// multiply q, a2, b2 instead and release held[0..1] (each may be null) afterwards; UNSUPPORTED: nothing was done.
+int gemm_repack(const GemmProblem& p, size_t esize, const void* a, const void* b, hipStream_t stream, bool may_copy, GemmProblem& q, const void*& a2, const void*& b2,
+                void* held[2]);
 // fp32 products of a few hundred rows and columns (32 x 32 tiles whose wavefronts split K; gemm_small.hip)
 int gemm_small_f32(const GemmProblem& p, const float* a, const float* b, float* c, hipStream_t stream);
 // bm x bn tiles (256 x 256, 256 x 128, 128 x 128) filled by direct global -> LDS loads (gemm_dtl.hip); T is f16 or bf16

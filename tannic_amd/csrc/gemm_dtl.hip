@@ -279,15 +279,29 @@ __global__ __launch_bounds__(256, BLOCKS_PER_CU) void gemm16_dtl_kernel(const T*
         }
         return;
     } else if constexpr (ES == 1) {
-        // int32 results: a lane's four consecutive columns are 16 bytes already
+        // int32 results: a lane's four consecutive columns are 16 bytes already (rows that start anywhere, or end inside
+        // them, go through the store for any alignment)
         int32_t* c32 = C + oc;
+        const bool quads = (p.c_rs | p.N) % 4 == 0 && reinterpret_cast<uintptr_t>(c32) % 16 == 0;
+        if (quads) {
 #pragma unroll
-        for (int i = 0; i < TM; ++i) {
-            const uint32_t row = m0 + wm + i * 16 + lane % 16;
+            for (int i = 0; i < TM; ++i) {
+                const uint32_t row = m0 + wm + i * 16 + lane % 16;
 #pragma unroll
-            for (int j = 0; j < TN; ++j) {
-                const uint32_t col = n0 + wn + j * 16 + 4 * (lane / 16);
-                if (row < p.M && col < p.N) *reinterpret_cast<int4v*>(c32 + static_cast<int64_t>(row) * p.c_rs + col) = acc[i][j];
+                for (int j = 0; j < TN; ++j) {
+                    const uint32_t col = n0 + wn + j * 16 + 4 * (lane / 16);
+                    if (row < p.M && col < p.N) *reinterpret_cast<int4v*>(c32 + static_cast<int64_t>(row) * p.c_rs + col) = acc[i][j];
+                }
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < TM; ++i) {
+                const uint32_t row = m0 + wm + i * 16 + lane % 16;
+#pragma unroll
+                for (int j = 0; j < TN; ++j) {
+                    const uint32_t col = n0 + wn + j * 16 + 4 * (lane / 16);
+                    if (row < p.M && col < p.N) store_piece_anywhere<int32_t>(c32 + static_cast<int64_t>(row) * p.c_rs + col, &acc[i][j], p.N - col < 4 ? p.N - col : 4);
+                }
             }
         }
         return;
@@ -441,12 +455,9 @@ template <class T>
 int gemm16_dtl(const GemmProblem& p, int bm, int bn, const void* a, const void* b, void* c, hipStream_t stream) {
     bool a_t, b_t;
     if (!operands_fit<T>(p, bm, bn, a_t, b_t)) return TANNIC_UNSUPPORTED_DTYPE;
-    constexpr int quad = 16 / sizeof(typename DtlTypes<T>::Out);   // results per 16-byte store
     if (p.c_group && (sizeof(T) != 2 || p.N % 8 != 0)) return TANNIC_UNSUPPORTED_DTYPE;   // column groups: 16-bit results, whole pieces of eight
-    // (16-bit results may lie anywhere: the kernel looks at the alignment of its own rows; int32 results are stored as quads)
-    if (sizeof(T) != 2 && (p.N % quad != 0 || p.c_rs % quad != 0 || reinterpret_cast<uintptr_t>(c) % 16 != 0)) return TANNIC_UNSUPPORTED_DTYPE;
-    for (int d = 0; d < p.batch_rank; ++d)
-        if (sizeof(T) != 2 && p.c_bs[d] % quad != 0) return TANNIC_UNSUPPORTED_DTYPE;
+    // (results may lie anywhere: the kernel looks at the alignment of its own rows)
+    if (reinterpret_cast<uintptr_t>(c) % sizeof(typename DtlTypes<T>::Out) != 0) return TANNIC_UNSUPPORTED_DTYPE;
     if constexpr (sizeof(T) == 2) {
         if (a_t || b_t) return gemm16_dtl_krows<T>(p, bm, bn, a_t, b_t, SplitK{0, 0, nullptr}, a, b, c, stream);
     }

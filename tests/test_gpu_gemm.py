@@ -128,12 +128,14 @@ def test_integer_gemm_bit_exact(device, pair, layout):
 
 
 @pytest.mark.parametrize("shape", [((300, 256), (520, 256)), ((16, 300, 128), (16, 520, 128)), ((50, 264, 128), (50, 264, 128)), ((2, 3, 70, 384), (136, 384)),
-                                   ((4096, 512), (1024, 512)), ((1, 512), (1024, 512)), ((16, 256), (130, 256)), ((3, 5, 128), (3, 70, 128))],
+                                   ((4096, 512), (1024, 512)), ((1, 512), (1024, 512)), ((16, 256), (130, 256)), ((3, 5, 128), (3, 70, 128)),
+                                   ((130, 384), (1001, 384)), ((70, 200), (333, 200)), ((300, 1000), (77, 1000))],
                          ids=lambda s: "x".join(map(str, s[0])) + "." + "x".join(map(str, s[1])) + "T")
 def test_int8_gemm_on_matrix_cores_is_bit_exact(device, shape):
     """int8 x int8 -> int32 with both operands K-contiguous and K a multiple of 128: the tiled kernels on
     v_mfma_i32_16x16x64_i8 in each tile size (128 x 128, 256 x 128, 256 x 256; ragged rows and columns, batches, a
-    broadcast second operand; one, five and sixteen rows in a 128-row tile).  Integer sums are exact, so the checker's sequential loop and numpy agree bit for bit."""
+    broadcast second operand; one, five and sixteen rows in a 128-row tile; a number of columns no quad divides; K that is
+    not a multiple of 128, which goes through zero-padded copies of both operands).  Integer sums are exact, so the checker's sequential loop and numpy agree bit for bit."""
     sa, sb = shape
     a = support.integers(SEED, 31, sa, -128, 128).astype(np.int8)
     b = support.integers(SEED, 32, sb, -128, 128).astype(np.int8)
@@ -144,6 +146,45 @@ def test_int8_gemm_on_matrix_cores_is_bit_exact(device, shape):
     support.assert_bit_exact(got.storage(), want, f"int8 gemm {sa} x {sb}^T against numpy")
     if int(np.prod(sa)) * sb[-2] < 40_000_000:
         support.assert_bit_exact(got.storage(), ops.matmul(ha, hb.transpose()).storage(), f"int8 gemm {sa} x {sb}^T against the checker")
+
+
+@pytest.mark.parametrize("layout", ["nn", "tn", "tt"])
+def test_int8_gemm_in_other_layouts_is_bit_exact(device, layout):
+    """int8 operands that are not contiguous along K (and a K of 300) are copied into K-contiguous rows, zero-padded to
+    whole steps, and multiplied on the matrix cores."""
+    m, n, k = 200, 170, 300
+    a = support.integers(SEED, 33, (k, m) if layout[0] == "t" else (m, k), -128, 128).astype(np.int8)
+    b = support.integers(SEED, 34, (n, k) if layout[1] == "t" else (k, n), -128, 128).astype(np.int8)
+    (ha, da), (hb, db) = support.both(a, ta.int8, device), support.both(b, ta.int8, device)
+    view = lambda t, transposed: t.transpose() if transposed else t
+    got = ops.matmul(view(da, layout[0] == "t"), view(db, layout[1] == "t"))
+    want = ops.matmul(view(ha, layout[0] == "t"), view(hb, layout[1] == "t"))
+    assert got.dtype is ta.int32 and got.shape == (m, n)
+    support.assert_bit_exact(got.storage(), want.storage(), f"int8 gemm {layout}")
+
+
+REPACKED = {
+    # large enough to be worth a copy: a second operand whose rows start at odd addresses, an odd K (zeros added to both), a
+    # first operand stored transposed with an odd number of rows, and a single row of a transposed first operand
+    "nn_odd_columns": ((300, 1032), (1032, 1001), [], []),
+    "nn_odd_k": ((260, 1001), (1001, 1040), [], []),
+    "tn_odd_rows": ((1032, 301), (1032, 1000), [("transpose", (-1, -2))], []),
+    "nt_odd_k_few_rows": ((8, 2049), (1500, 2049), [], [("transpose", (-1, -2))]),
+    "tn_single_row": ((4096, 1), (4096, 520), [("transpose", (-1, -2))], []),
+}
+
+
+@pytest.mark.parametrize("name", list(REPACKED))
+@pytest.mark.parametrize("dtype", [ta.float16, ta.bfloat16, ta.float32], ids=str)
+def test_products_whose_operands_are_copied_into_aligned_rows(device, dtype, name):
+    sa, sb, va, vb = REPACKED[name]
+    ha, da = support.both(support.values_for(dtype, SEED, 41, sa, -1, 1), dtype, device)
+    hb, db = support.both(support.values_for(dtype, SEED, 42, sb, -1, 1), dtype, device)
+    want = ops.matmul(support.apply_view(ha, va), support.apply_view(hb, vb)).numpy()
+    got = ops.matmul(support.apply_view(da, va), support.apply_view(db, vb)).numpy()
+    k = support.apply_view(ha, va).shape[-1]
+    if dtype is ta.float32: support.assert_close(got, want, 1e-5, k * 2.0 ** -24, f"gemm {dtype} {name}")
+    else: support.assert_close(got, want, 2e-3 if dtype is ta.float16 else 2.0 ** -7, 1e-3, f"gemm {dtype} {name}")
 
 
 @pytest.mark.parametrize("pair", [(ta.int32, ta.float32), (ta.float64, ta.float32), (ta.float16, ta.float32), (ta.float32, ta.bfloat16)],
