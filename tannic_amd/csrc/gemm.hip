@@ -174,9 +174,58 @@ __global__ __launch_bounds__(256) void gemm_generic_kernel(const A* a, const B* 
         }
 }
 
+// A handful of rows over a long K, both operands contiguous along K (a linear layer on a few tokens, in float64, an integer
+// type or a mixed pair): the kernel above would give each 64 x 64 tile to one block that walks all of K.  Here a
+// wavefront owns four columns of the result and ROWS rows; its lanes stride over K (whole lines of B's rows, A's rows from
+// the caches) and the 4 * ROWS sums meet in a butterfly at the end.  Integer sums are exact in any order; floating sums
+// are a tree instead of the CPU path's sequence, within rounding of it.
+template <class A, class B, class D, int ROWS>
+__global__ __launch_bounds__(256) void gemm_generic_few_rows_kernel(const A* a, const B* b, D* c, GemmProblem p) {
+    using Acc = std::conditional_t<is_16bit<D>::value, float, D>;
+    int64_t oa, ob, oc;
+    batch_offsets(p, blockIdx.z, oa, ob, oc);
+    a += oa;
+    b += ob;
+    c += oc;
+    const uint32_t lane = threadIdx.x % 64, n0 = (blockIdx.x * 4 + threadIdx.x / 64) * 4, m0 = blockIdx.y * ROWS;
+    if (n0 >= p.N) return;   // whole wavefronts; nothing below synchronises across them
+    Acc acc[ROWS][4] = {};
+    for (uint32_t k = lane; k < p.K; k += 64) {
+        Acc y[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) y[j] = static_cast<Acc>(widen(b[static_cast<int64_t>(n0 + j < p.N ? n0 + j : n0) * p.b_cs + k]));
+#pragma unroll
+        for (int i = 0; i < ROWS; ++i) {
+            const Acc x = static_cast<Acc>(widen(a[static_cast<int64_t>(m0 + i < p.M ? m0 + i : m0) * p.a_rs + k]));
+#pragma unroll
+            for (int j = 0; j < 4; ++j) acc[i][j] += x * y[j];
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < ROWS; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            Acc v = acc[i][j];
+#pragma unroll
+            for (int step = 32; step >= 1; step >>= 1) v += __shfl_xor(v, step, 64);
+            if (lane == 0 && m0 + i < p.M && n0 + j < p.N) c[static_cast<int64_t>(m0 + i) * p.c_rs + n0 + j] = narrow<D>(v);
+        }
+}
+
 template <class A, class B, class D>
 int run_generic(const GemmProblem& p, const void* a, const void* b, void* c, hipStream_t stream) {
     if (p.M == 0 || p.N == 0 || p.batches == 0) return TANNIC_SUCCESS;
+    if (p.M <= 16 && p.a_cs == 1 && p.b_rs == 1 && p.K >= 256 && p.batches <= 65535) {
+        const dim3 grid((p.N + 15) / 16, (p.M + 7) / 8, p.batches);
+        if (p.M <= 4) {
+            hipLaunchKernelGGL((gemm_generic_few_rows_kernel<A, B, D, 4>), dim3(grid.x, (p.M + 3) / 4, p.batches), dim3(256), 0, stream, static_cast<const A*>(a),
+                               static_cast<const B*>(b), static_cast<D*>(c), p);
+        } else {
+            hipLaunchKernelGGL((gemm_generic_few_rows_kernel<A, B, D, 8>), grid, dim3(256), 0, stream, static_cast<const A*>(a), static_cast<const B*>(b),
+                               static_cast<D*>(c), p);
+        }
+        return launch_status("gemm_generic_few_rows_kernel");
+    }
     const uint32_t gx = (p.N + 63) / 64, gy = (p.M + 63) / 64;
     if (gy > 65535 || p.batches > 65535) {
         set_error_text("gemm: generic kernel grid limit exceeded");

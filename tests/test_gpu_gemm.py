@@ -118,7 +118,8 @@ def test_16bit_gemm_fp32_accumulate(device, dtype, layout):
     support.assert_close(got.numpy(), want.numpy(), rtol, 1e-3, f"gemm {dtype} {layout}")
 
 
-@pytest.mark.parametrize("layout", ["nn", "nt_mid", "tn_mid", "batched", "batch_broadcast", "rank4_rank2_nt"])
+@pytest.mark.parametrize("layout", ["nn", "nt_mid", "tn_mid", "batched", "batch_broadcast", "rank4_rank2_nt",
+                                    "single_row", "sixteen_rows", "stream_16_rows_ragged_columns", "stream_batched_views"])
 @pytest.mark.parametrize("pair", [(ta.int8, ta.int8), (ta.int16, ta.int32), (ta.int32, ta.int32), (ta.int64, ta.int8)], ids=lambda p: f"{p[0]}-{p[1]}")
 def test_integer_gemm_bit_exact(device, pair, layout):
     host, dev, _ = operands(pair, layout, device, -100, 100)
