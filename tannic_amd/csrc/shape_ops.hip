@@ -242,6 +242,35 @@ __global__ __launch_bounds__(256) void triangular_kernel(const U* src, U* dst, u
     dst[static_cast<int64_t>(i) * ds0 + static_cast<int64_t>(j) * ds1] = keep ? src[static_cast<int64_t>(i) * ss0 + static_cast<int64_t>(j) * ss1] : U(0);
 }
 
+// Rows contiguous and 16-byte friendly in both tensors: a thread writes one 16-byte piece, and reads it only when some of it
+// is kept (the zeroed half of the matrix is not read at all).
+template <class U, bool UPPER>
+__global__ __launch_bounds__(256) void triangular_pieces_kernel(const U* src, U* dst, uint32_t pieces_per_row, uint32_t total, int64_t ss0, int64_t ds0, int k, FastDiv div_pieces) {
+    constexpr uint32_t E = 16 / sizeof(U);
+    const uint32_t idx = blockIdx.x * 256 + threadIdx.x;
+    if (idx >= total) return;
+    uint32_t i, piece;
+    div_pieces.divmod(idx, i, piece);
+    const uint32_t j0 = piece * E;
+    const uint64_t edge = static_cast<uint64_t>(i) + static_cast<uint64_t>(static_cast<int64_t>(k));   // as in the kernel above
+    bool keep[E], any = false;
+#pragma unroll
+    for (uint32_t e = 0; e < E; ++e) {
+        keep[e] = UPPER ? static_cast<uint64_t>(j0 + e) >= edge : static_cast<uint64_t>(j0 + e) <= edge;
+        any = any || keep[e];
+    }
+    U v[E];
+    if (any) {
+        const uint4 bits = *reinterpret_cast<const uint4*>(src + static_cast<int64_t>(i) * ss0 + j0);
+        __builtin_memcpy(v, &bits, 16);
+    }
+#pragma unroll
+    for (uint32_t e = 0; e < E; ++e) v[e] = (any && keep[e]) ? v[e] : U(0);
+    uint4 out;
+    __builtin_memcpy(&out, v, 16);
+    *reinterpret_cast<uint4*>(dst + static_cast<int64_t>(i) * ds0 + j0) = out;
+}
+
 template <bool UPPER>
 int run_triangular(const tannic_tensor_t* src, tannic_tensor_t* dst, int k, hipStream_t stream) {
     size_t esize;
@@ -267,6 +296,17 @@ int run_triangular(const tannic_tensor_t* src, tannic_tensor_t* dst, int k, hipS
     const int64_t ss0 = src->strides.sizes[0], ss1 = src->strides.sizes[1], ds0 = dst->strides.sizes[0], ds1 = dst->strides.sizes[1];
     const FastDiv dc(static_cast<uint32_t>(cols));
     const uint32_t r = static_cast<uint32_t>(rows), c = static_cast<uint32_t>(cols);
+    const uint64_t per = 16 / esize;
+    if (ss1 == 1 && ds1 == 1 && cols % per == 0 && ss0 % static_cast<int64_t>(per) == 0 && ds0 % static_cast<int64_t>(per) == 0 &&
+        reinterpret_cast<uintptr_t>(src->address) % 16 == 0 && reinterpret_cast<uintptr_t>(dst->address) % 16 == 0) {
+        const uint32_t pieces = static_cast<uint32_t>(cols / per), total = r * pieces;
+        const dim3 pgrid((total + 255) / 256);
+        const FastDiv dp(pieces);
+        if (esize == 2) hipLaunchKernelGGL((triangular_pieces_kernel<uint16_t, UPPER>), pgrid, dim3(256), 0, stream, static_cast<const uint16_t*>(src->address), static_cast<uint16_t*>(dst->address), pieces, total, ss0, ds0, k, dp);
+        else if (esize == 4) hipLaunchKernelGGL((triangular_pieces_kernel<uint32_t, UPPER>), pgrid, dim3(256), 0, stream, static_cast<const uint32_t*>(src->address), static_cast<uint32_t*>(dst->address), pieces, total, ss0, ds0, k, dp);
+        else hipLaunchKernelGGL((triangular_pieces_kernel<uint64_t, UPPER>), pgrid, dim3(256), 0, stream, static_cast<const uint64_t*>(src->address), static_cast<uint64_t*>(dst->address), pieces, total, ss0, ds0, k, dp);
+        return launch_status("triangular_pieces_kernel");
+    }
     if (esize == 2) hipLaunchKernelGGL((triangular_kernel<uint16_t, UPPER>), grid, dim3(256), 0, stream, static_cast<const uint16_t*>(src->address), static_cast<uint16_t*>(dst->address), r, c, ss0, ss1, ds0, ds1, k, dc);
     else if (esize == 4) hipLaunchKernelGGL((triangular_kernel<uint32_t, UPPER>), grid, dim3(256), 0, stream, static_cast<const uint32_t*>(src->address), static_cast<uint32_t*>(dst->address), r, c, ss0, ss1, ds0, ds1, k, dc);
     else hipLaunchKernelGGL((triangular_kernel<uint64_t, UPPER>), grid, dim3(256), 0, stream, static_cast<const uint64_t*>(src->address), static_cast<uint64_t*>(dst->address), r, c, ss0, ss1, ds0, ds1, k, dc);

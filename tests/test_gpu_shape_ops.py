@@ -59,6 +59,18 @@ def test_triangular_bit_exact(device, dtype, op, view, k):
     support.assert_bit_exact(got.storage(), want.storage(), f"{op} {dtype} {view} k={k}")
 
 
+@pytest.mark.parametrize("k", [0, 1, 5, -1, -7, 40, -40])
+@pytest.mark.parametrize("op", ["triu", "tril"])
+@pytest.mark.parametrize("dtype", [ta.int64, ta.float16, ta.float32], ids=str)
+def test_triangular_of_rows_in_16_byte_pieces(device, dtype, op, k):
+    """Rows of 32 columns (whole 16-byte pieces, some wholly kept, some wholly zeroed, some cut by the diagonal), from a
+    plain matrix and from rows 3.. of a taller one."""
+    hx, dx = support.both(support.values_for(dtype, SEED, 3, (37, 32), -4, 4), dtype, device)
+    for first in (0, 3):
+        want, got = getattr(ops, op)(hx[first:], k), getattr(ops, op)(dx[first:], k)
+        support.assert_bit_exact(got.storage(), want.storage(), f"{op} {dtype} rows from {first} k={k}")
+
+
 def test_causal_mask_shape(device):
     n = 512
     hx, dx = support.both(np.ones((n, n), dtype=np.float32), ta.float32, device)
