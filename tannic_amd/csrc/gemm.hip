@@ -260,14 +260,36 @@ int gemm_entry(const tannic_tensor_t* a, const tannic_tensor_t* b, tannic_tensor
                 GemmProblem p;
                 status = describe_gemm(a, b, dst, p);
                 if (status != TANNIC_SUCCESS) return;
+                const void *first = a->address, *second = b->address;
+                if constexpr (std::is_same_v<A, B>) {
+                    // A matrix times a column, y = A . v: the same numbers are v^T . A^T, one row times a matrix whose "rows of
+                    // W" are A's rows - the shape the kernels for few rows stream (a column of results lies in memory like a row).
+                    if (p.N == 1 && p.M > 1 && p.c_rs == 1) {
+                        GemmProblem t = p;
+                        t.M = 1;
+                        t.N = p.M;
+                        t.a_rs = p.b_cs;   // a single row: its pitch is never used
+                        t.a_cs = p.b_rs;
+                        t.b_rs = p.a_cs;
+                        t.b_cs = p.a_rs;
+                        t.c_rs = p.M;
+                        for (int d = 0; d < 6; ++d) {
+                            t.a_bs[d] = p.b_bs[d];
+                            t.b_bs[d] = p.a_bs[d];
+                        }
+                        p = t;
+                        first = b->address;
+                        second = a->address;
+                    }
+                }
                 constexpr bool tiled = std::is_same_v<A, B> && (is_16bit<A>::value || std::is_same_v<A, int8_t> || std::is_same_v<A, float>);
                 if constexpr (tiled) {
                     // operands that do not lie as the tiled kernels want them are copied first when that pays (never on the
                     // path that must not allocate)
                     GemmProblem q;
-                    const void *pa = a->address, *pb = b->address;
+                    const void *pa = first, *pb = second;
                     void* held[2] = {nullptr, nullptr};
-                    const int repacked = gemm_repack(p, sizeof(A), a->address, b->address, s, workspace == nullptr, q, pa, pb, held);
+                    const int repacked = gemm_repack(p, sizeof(A), first, second, s, workspace == nullptr, q, pa, pb, held);
                     if (repacked == TANNIC_ERROR) {
                         status = TANNIC_ERROR;
                         return;
@@ -280,7 +302,7 @@ int gemm_entry(const tannic_tensor_t* a, const tannic_tensor_t* b, tannic_tensor
                         if (h) scratch_release(h, s);
                     if (status != TANNIC_UNSUPPORTED_DTYPE) return;
                 }
-                status = run_generic<A, B, D>(p, a->address, b->address, dst->address, s);
+                status = run_generic<A, B, D>(p, first, second, dst->address, s);
             }
         });
     });

@@ -37,6 +37,10 @@ LAYOUTS = {
     "sixteen_rows": ((16, 256), (96, 256), [], [("transpose", (-1, -2))]),
     "single_column": ((64, 96), (1, 96), [], [("transpose", (-1, -2))]),
     "k_one": ((9, 1), (1, 11), [], []),
+    # a matrix times a column (run as one row times the transposed matrix): plain, the matrix stored transposed, batches
+    "matrix_vector": ((300, 512), (512, 1), [], []),
+    "matrix_vector_transposed_matrix": ((512, 300), (512, 1), [("transpose", (-1, -2))], []),
+    "matrix_vector_batched": ((3, 70, 256), (3, 256, 1), [], []),
     # few rows: ragged K steps and columns, two row blocks, batches; a long K shared between blocks
     "skinny_17_rows_ragged": ((17, 72), (40, 72), [], [("transpose", (-1, -2))]),
     "skinny_batched": ((3, 5, 64), (3, 24, 64), [], [("transpose", (-1, -2))]),
@@ -119,7 +123,8 @@ def test_16bit_gemm_fp32_accumulate(device, dtype, layout):
 
 
 @pytest.mark.parametrize("layout", ["nn", "nt_mid", "tn_mid", "batched", "batch_broadcast", "rank4_rank2_nt",
-                                    "single_row", "sixteen_rows", "stream_16_rows_ragged_columns", "stream_batched_views"])
+                                    "single_row", "sixteen_rows", "stream_16_rows_ragged_columns", "stream_batched_views", "matrix_vector",
+                                    "matrix_vector_batched"])
 @pytest.mark.parametrize("pair", [(ta.int8, ta.int8), (ta.int16, ta.int32), (ta.int32, ta.int32), (ta.int64, ta.int8)], ids=lambda p: f"{p[0]}-{p[1]}")
 def test_integer_gemm_bit_exact(device, pair, layout):
     host, dev, _ = operands(pair, layout, device, -100, 100)
