@@ -282,6 +282,11 @@ int run_skinny(const GemmProblem& p, const void* a, const void* b, void* c, hipS
         if (!mult8(p.a_bs[d]) || !mult8(p.b_bs[d])) return TANNIC_UNSUPPORTED_DTYPE;
     // whole windows of 64 and rows that do not overlap: the streaming kernel (offsets inside a block are 32-bit byte counts)
     if (p.K % kBKof<T> == 0 && p.a_rs >= static_cast<int64_t>(p.K) && p.b_cs >= static_cast<int64_t>(p.K) && p.a_rs < (1 << 22) && p.b_cs < (1 << 22)) {
+        // Many small products under a short K (the scores of attention while decoding: one row against [4096, 128] per head):
+        // a block's four wavefronts share K, two windows here, and a block moves 4 KB - the tiles do better (fp16, 256
+        // heads: 73 against 173 us; 1024 x [512, 64]: 22 against 83; fp32 from 128 heads on: 64 against 95).  A single
+        // product stays (one row against [32000, 256]: 7.5 against 13.7 us).
+        if (sizeof(T) == 2 ? (p.batches >= 8 && p.K <= 512) : (p.batches >= 128 && p.K <= 128)) return TANNIC_UNSUPPORTED_DTYPE;
         // two column blocks per wavefront (half as many workgroups, x read half as often) while every compute unit still gets one
         const bool two = static_cast<uint64_t>((p.N + 31) / 32) * p.batches >= 400;
         if (p.M <= 16) return two ? launch_stream<T, 1, 2>(p, a, b, c, stream) : launch_stream<T, 1, 1>(p, a, b, c, stream);
