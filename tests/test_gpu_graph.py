@@ -124,6 +124,14 @@ def test_every_operator_family_replays(device):
     b = ta.tensor(support.normal(13, 10, (2048, 4096), 0.02), f16, device)
     rho = ta.tensor(support.uniform(13, 11, (40, 30), 0.5, 2.0), f32, device)
     theta = ta.tensor(support.uniform(13, 12, (40, 30), -3.0, 3.0), f32, device)
+    # operands that are copied into aligned rows first (an odd number of columns), a matrix times a column, a handful of
+    # very long rows shared by several blocks, a transposing copy, the unfolded batch of a convolution
+    odd_a = ta.tensor(support.normal(13, 13, (300, 1032), 1.0), f16, device)
+    odd_b = ta.tensor(support.normal(13, 14, (1032, 1001), 0.05), f16, device)
+    column = ta.tensor(support.normal(13, 15, (4096, 1), 0.05), f16, device)
+    logits = ta.tensor(support.normal(13, 16, (4, 50257), 2.0), f32, device)
+    img7 = ta.tensor(support.normal(13, 17, (8, 128, 7, 7), 1.0), f16, device)
+    ker7 = ta.tensor(support.normal(13, 18, (64, 128, 3, 3), 0.05), f16, device)
 
     def everything():
         return [
@@ -135,6 +143,8 @@ def test_every_operator_family_replays(device):
             ops.repeat(img32, 3, 1), ops.concatenate(big, other, 2), ops.triu(rho, 1), ops.outer(bias32, bias32),
             ops.softmax(rows), ops.rms_norm(rows, gain), ops.cast(rows, f32),
             ops.matmul(a, b.transpose()),
+            ops.matmul(odd_a, odd_b), ops.matmul(b, column), ops.argmax(logits, 1), ops.softmax(logits), ops.sum(logits, 1),
+            ops.repack(b.transpose()), ops.convolve2d(img7, ker7, None, 1, 1),
         ]
 
     want = [t.storage() for t in everything()]
