@@ -212,6 +212,15 @@ __global__ __launch_bounds__(256) void gemm_generic_few_rows_kernel(const A* a, 
         }
 }
 
+// c[m * c_rs + n] = t[n * M + m]: the few rows of a transposed result back into the columns they belong to
+template <class U>
+__global__ __launch_bounds__(256) void gemm_columns_from_rows_kernel(const U* t, U* c, uint32_t M, uint32_t N, int64_t c_rs, uint32_t total) {
+    const uint32_t idx = blockIdx.x * 256 + threadIdx.x;
+    if (idx >= total) return;
+    const uint32_t m = idx / N, n = idx % N;
+    c[static_cast<int64_t>(m) * c_rs + n] = t[static_cast<size_t>(n) * M + m];
+}
+
 template <class A, class B, class D>
 int run_generic(const GemmProblem& p, const void* a, const void* b, void* c, hipStream_t stream) {
     if (p.M == 0 || p.N == 0 || p.batches == 0) return TANNIC_SUCCESS;
@@ -283,6 +292,46 @@ int gemm_entry(const tannic_tensor_t* a, const tannic_tensor_t* b, tannic_tensor
                     }
                 }
                 constexpr bool tiled = std::is_same_v<A, B> && (is_16bit<A>::value || std::is_same_v<A, int8_t> || std::is_same_v<A, float>);
+                if constexpr (std::is_same_v<A, B> && (is_16bit<A>::value || std::is_same_v<A, float>)) {
+                    // Many rows times a few columns (a classifier's last layer over a batch): C^T = W . X^T has the few as its
+                    // rows, which the streaming kernel takes - X goes by once - and the small result is turned back.  Only
+                    // where that kernel will take it (whole windows of K, aligned K-contiguous rows) and scratch may be had.
+                    constexpr uint32_t window = 128 / sizeof(A), unit = 16 / sizeof(A);
+                    const bool streams = p.N >= 2 && p.N <= 32 && p.M >= 256 && p.batches == 1 && workspace == nullptr && p.a_cs == 1 && p.b_rs == 1 &&
+                                         p.K % window == 0 && p.a_rs % unit == 0 && p.b_cs % unit == 0 && p.a_rs >= static_cast<int64_t>(p.K) &&
+                                         p.b_cs >= static_cast<int64_t>(p.K) && p.a_rs < (1 << 22) && p.b_cs < (1 << 22) &&
+                                         reinterpret_cast<uintptr_t>(first) % 16 == 0 && reinterpret_cast<uintptr_t>(second) % 16 == 0 &&
+                                         static_cast<uint64_t>(p.M) * p.K >= (1u << 21) &&
+                                         // (16-bit tiles already fill the chip from 16384 rows on, and a short K leaves the streaming
+                                         // kernel's blocks too little each; fp32 tiles pay the matrix pipe for every padded column)
+                                         (sizeof(A) == 2 ? (p.M <= 16384 && p.K >= 1024) : p.K >= 512);
+                    if (streams) {
+                        GemmProblem t = p;
+                        t.M = p.N;
+                        t.N = p.M;
+                        t.a_rs = p.b_cs;
+                        t.a_cs = p.b_rs;
+                        t.b_rs = p.a_cs;
+                        t.b_cs = p.a_rs;
+                        t.c_rs = p.M;
+                        void* turned = nullptr;
+                        if (scratch_acquire(&turned, static_cast<size_t>(p.M) * p.N * sizeof(A), s) != TANNIC_SUCCESS) {
+                            status = TANNIC_ERROR;
+                            return;
+                        }
+                        if constexpr (is_16bit<A>::value) status = gemm_skinny_16bit(t, a->dtype, second, first, turned, s);
+                        else status = gemm_skinny_f32(t, static_cast<const float*>(second), static_cast<const float*>(first), static_cast<float*>(turned), s);
+                        if (status == TANNIC_SUCCESS) {
+                            using U = typename std::conditional<sizeof(A) == 2, uint16_t, uint32_t>::type;
+                            const uint32_t total = p.M * p.N;
+                            hipLaunchKernelGGL((gemm_columns_from_rows_kernel<U>), dim3((total + 255) / 256), dim3(256), 0, s, static_cast<const U*>(turned),
+                                               static_cast<U*>(dst->address), p.M, p.N, p.c_rs, total);
+                            status = launch_status("gemm_columns_from_rows_kernel");
+                        }
+                        scratch_release(turned, s);
+                        if (status != TANNIC_UNSUPPORTED_DTYPE) return;   // (refused after all: on with the product as it is)
+                    }
+                }
                 if constexpr (tiled) {
                     // operands that do not lie as the tiled kernels want them are copied first when that pays (never on the
                     // path that must not allocate)

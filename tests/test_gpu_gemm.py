@@ -41,6 +41,9 @@ LAYOUTS = {
     "matrix_vector": ((300, 512), (512, 1), [], []),
     "matrix_vector_transposed_matrix": ((512, 300), (512, 1), [("transpose", (-1, -2))], []),
     "matrix_vector_batched": ((3, 70, 256), (3, 256, 1), [], []),
+    # many rows times a few columns (run transposed through the streaming kernel and turned back)
+    "few_columns": ((600, 4096), (10, 4096), [], [("transpose", (-1, -2))]),
+    "two_columns_of_a_wider_result": ((700, 4096), (32, 4096), [], [("index", (slice(3, 5), slice(None))), ("transpose", (-1, -2))]),
     # few rows: ragged K steps and columns, two row blocks, batches; a long K shared between blocks
     "skinny_17_rows_ragged": ((17, 72), (40, 72), [], [("transpose", (-1, -2))]),
     "skinny_batched": ((3, 5, 64), (3, 24, 64), [], [("transpose", (-1, -2))]),
