@@ -118,10 +118,15 @@ static int conv2d_entry(const tannic_tensor_t* x, const tannic_tensor_t* w, cons
     if (status != TANNIC_UNSUPPORTED_DTYPE) return status;
     status = conv2d_unfold(p, x->dtype, x->address, w->address, pb, y->address, s);
     if (status != TANNIC_UNSUPPORTED_DTYPE) return status;
-    // 16-bit shapes none of the above takes: unfolded and multiplied, while the unfolded operand is small
+    // 16-bit shapes none of the above takes: unfolded and multiplied, or the general tile kernel.  Large images go to
+    // the tile kernel first: their unfolded operand is hundreds of megabytes under few output channels
+    // (fp16, batch 8, 7x7, us unfolded / tiles: 64 -> 64 over 112 x 112 468 / 303, 24 -> 48 168 / 123, over 56 x 56 110 / 139, 48 / 56).
+    const bool large_images = static_cast<uint64_t>(p.HO) * p.WO > 8192;
+    if (large_images) status = conv2d_mfma(p, x->dtype, x->address, w->address, pb, y->address, s);
+    if (status != TANNIC_UNSUPPORTED_DTYPE) return status;
     status = conv2d_unfold_batch_any(p, x->dtype, x->address, w->address, pb, y->address, s);
     if (status != TANNIC_UNSUPPORTED_DTYPE) return status;
-    status = conv2d_mfma(p, x->dtype, x->address, w->address, pb, y->address, s);
+    if (!large_images) status = conv2d_mfma(p, x->dtype, x->address, w->address, pb, y->address, s);
     if (status != TANNIC_UNSUPPORTED_DTYPE) return status;
     switch (x->dtype) {
         case TANNIC_INT8: return run_direct<int8_t>(p, x->address, w->address, pb, y->address, s);

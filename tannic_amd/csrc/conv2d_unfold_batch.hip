@@ -57,9 +57,19 @@ static int run_unfold_batch(const ConvProblem& p, int dtype, const void* x, cons
     // 144 33 / 25, 72 25 / 16: with a short K the unfolded operand is as large as the work)
     if ((ANY_SIZE ? K < 320 : (pixels > 100 || K < 512)) || K % E != 0 || K >= (1u << 24) || pixels >= (1u << 24)) return TANNIC_UNSUPPORTED_DTYPE;
     const uint32_t pitch = static_cast<uint32_t>((pixels + E - 1) / E * E);
-    const uint64_t columns = static_cast<uint64_t>(p.N) * pitch;
-    if (columns < 256 || columns >= (1ull << 31) || K * p.N * (pitch / E) >= (1ull << 31)) return TANNIC_UNSUPPORTED_DTYPE;
-    if (K * columns * sizeof(T) > ((ANY_SIZE ? 256ull : 512ull) << 20)) return TANNIC_UNSUPPORTED_DTYPE;
+    if (static_cast<uint64_t>(p.N) * pitch < 256) return TANNIC_UNSUPPORTED_DTYPE;
+    // The unfolded operand is kept small: ANY_SIZE takes the images in runs whose unfolded operand stays within the
+    // limit (one image's may reach four times that), one product per run, all through the same buffer.
+    const uint64_t limit = (ANY_SIZE ? 256ull : 512ull) << 20, image_bytes = K * pitch * sizeof(T);
+    uint32_t run = p.N;
+    if (image_bytes * p.N > limit) {
+        if (!ANY_SIZE || image_bytes > 4 * limit) return TANNIC_UNSUPPORTED_DTYPE;
+        run = static_cast<uint32_t>(limit / image_bytes);
+        if (run == 0) run = 1;
+        if (static_cast<uint64_t>(run) * pitch < 256) return TANNIC_UNSUPPORTED_DTYPE;
+    }
+    const uint64_t columns = static_cast<uint64_t>(run) * pitch;
+    if (columns >= (1ull << 31) || K * run * (pitch / E) >= (1ull << 31)) return TANNIC_UNSUPPORTED_DTYPE;
     // the kernel tensor as a K-contiguous O x K matrix, the result as pixel-contiguous rows
     if (p.ws[3] != 1 || p.ws[2] != static_cast<int64_t>(p.KW) || p.ws[1] != static_cast<int64_t>(p.KH) * p.KW || p.ws[0] != static_cast<int64_t>(K) ||
         reinterpret_cast<uintptr_t>(w) % 16 != 0)
@@ -67,18 +77,25 @@ static int run_unfold_batch(const ConvProblem& p, int dtype, const void* x, cons
     if (p.ys[3] != 1 || p.ys[2] != static_cast<int64_t>(p.WO)) return TANNIC_UNSUPPORTED_DTYPE;
     T* col = nullptr;
     if (scratch_acquire(reinterpret_cast<void**>(&col), static_cast<size_t>(K) * columns * sizeof(T), stream) != TANNIC_SUCCESS) return TANNIC_ERROR;
-    const uint32_t groups = pitch / E, total = static_cast<uint32_t>(K * p.N * groups);
-    hipLaunchKernelGGL((conv_unfold_batch_kernel<T>), dim3((total + 255) / 256), dim3(256), 0, stream, static_cast<const T*>(x), col, p, static_cast<uint32_t>(pixels), pitch,
-                       FastDiv(groups), FastDiv(p.N), FastDiv(p.WO), FastDiv(p.KH * p.KW), FastDiv(p.KW), total);
-    int status = launch_status("conv_unfold_batch_kernel");
-    if (status == TANNIC_SUCCESS) {
+    int status = TANNIC_SUCCESS;
+    for (uint32_t n0 = 0; n0 < p.N && status == TANNIC_SUCCESS; n0 += run) {
+        ConvProblem part = p;
+        part.N = p.N - n0 < run ? p.N - n0 : run;
+        const T* x_part = static_cast<const T*>(x) + static_cast<int64_t>(n0) * p.xs[0];
+        T* y_part = static_cast<T*>(y) + static_cast<int64_t>(n0) * p.ys[0];
+        const uint64_t part_columns = static_cast<uint64_t>(part.N) * pitch;
+        const uint32_t groups = pitch / E, total = static_cast<uint32_t>(K * part.N * groups);
+        hipLaunchKernelGGL((conv_unfold_batch_kernel<T>), dim3((total + 255) / 256), dim3(256), 0, stream, x_part, col, part, static_cast<uint32_t>(pixels), pitch,
+                           FastDiv(groups), FastDiv(part.N), FastDiv(p.WO), FastDiv(p.KH * p.KW), FastDiv(p.KW), total);
+        status = launch_status("conv_unfold_batch_kernel");
+        if (status != TANNIC_SUCCESS) break;
         GemmProblem g{};
         g.M = p.O;
-        g.N = static_cast<uint32_t>(columns);
+        g.N = static_cast<uint32_t>(part_columns);
         g.K = static_cast<uint32_t>(K);
         g.a_rs = p.ws[0];
         g.a_cs = 1;
-        g.b_rs = static_cast<int64_t>(columns);
+        g.b_rs = static_cast<int64_t>(part_columns);
         g.b_cs = 1;
         // the columns of image n go to y[n]: rows p.ys[1] apart, images p.ys[0]
         g.c_rs = p.ys[1];
@@ -93,8 +110,8 @@ static int run_unfold_batch(const ConvProblem& p, int dtype, const void* x, cons
             g.a_bs[d] = g.b_bs[d] = g.c_bs[d] = 0;
         }
         g.row_bias = bias;
-        if constexpr (std::is_same_v<T, float>) status = gemm_mfma_f32(g, static_cast<const float*>(w), reinterpret_cast<const float*>(col), static_cast<float*>(y), stream);
-        else status = gemm_mfma_16bit(g, dtype, w, col, y, stream);
+        if constexpr (std::is_same_v<T, float>) status = gemm_mfma_f32(g, static_cast<const float*>(w), reinterpret_cast<const float*>(col), static_cast<float*>(y_part), stream);
+        else status = gemm_mfma_16bit(g, dtype, w, col, y_part, stream);
         if (status == TANNIC_UNSUPPORTED_DTYPE) {
             set_error_text("conv2d: internal: the unfolded product refused a problem its caller had checked");
             status = TANNIC_ERROR;

@@ -110,6 +110,10 @@ CASES = {
     "unfolded_any_k7_48ch": ((2, 48, 20, 20), (48, 48, 7, 7), (1, 1), (3, 3)),
     "unfolded_any_k3_72ch": ((4, 72, 17, 17), (100, 72, 3, 3), (1, 1), (1, 1)),
     "unfolded_any_k3_40ch_s2": ((3, 40, 21, 19), (24, 40, 3, 3), (2, 2), (1, 1)),
+    # ... in runs of images when the whole batch unfolded would be large (13 images and 1; one image at a time), with a
+    # K beyond what the general tiles keep a table of
+    "unfolded_any_runs_of_images": ((14, 128, 40, 40), (4, 128, 7, 7), (1, 1), (3, 3)),
+    "unfolded_any_one_image_a_run": ((2, 256, 112, 112), (2, 256, 7, 7), (1, 1), (3, 3)),
 }
 
 
