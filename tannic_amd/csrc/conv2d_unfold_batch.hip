@@ -125,7 +125,16 @@ int conv2d_unfold_batch(const ConvProblem& p, int dtype, const void* x, const vo
     if (p.KH == 1 && p.KW == 1) return TANNIC_UNSUPPORTED_DTYPE;   // conv2d_pointwise.hip: no unfolding needed
     if (dtype == TANNIC_FLOAT16) return run_unfold_batch<f16, false>(p, dtype, x, w, bias, y, stream);
     if (dtype == TANNIC_BFLOAT16) return run_unfold_batch<bf16, false>(p, dtype, x, w, bias, y, stream);
-    if (dtype == TANNIC_FLOAT32) return run_unfold_batch<float, false>(p, dtype, x, w, bias, y, stream);
+    if (dtype == TANNIC_FLOAT32) {
+        const int status = run_unfold_batch<float, false>(p, dtype, x, w, bias, y, stream);
+        if (status != TANNIC_UNSUPPORTED_DTYPE) return status;
+        // fp32 has no patch kernels, and the gathering tiles (conv2d_gather32.hip) are few when the whole batch has few pixels:
+        // each walks all of K alone, where the product over the unfolded batch shares K between blocks
+        // (batch 8, us gathered / unfolded: 64 -> 64 7x7 over 14 x 14 175 / 34, 256 -> 128 3x3 124 / 38, 64 -> 64 3x3 over
+        // 28 x 28 35 / 27; at batch 32 over 28 x 28, 25088 pixels, 38 / 53 and 186 / 269)
+        if (static_cast<uint64_t>(p.N) * p.HO * p.WO <= 8192) return run_unfold_batch<float, true>(p, dtype, x, w, bias, y, stream);
+        return TANNIC_UNSUPPORTED_DTYPE;
+    }
     return TANNIC_UNSUPPORTED_DTYPE;
 }
 
