@@ -351,6 +351,10 @@ int gemm_entry(const tannic_tensor_t* a, const tannic_tensor_t* b, tannic_tensor
                         if (h) scratch_release(h, s);
                     if (status != TANNIC_UNSUPPORTED_DTYPE) return;
                 }
+                if constexpr (std::is_same_v<A, double> && std::is_same_v<B, double>) {
+                    status = gemm_mfma_f64(p, static_cast<const double*>(first), static_cast<const double*>(second), static_cast<double*>(dst->address), s);
+                    if (status != TANNIC_UNSUPPORTED_DTYPE) return;
+                }
                 status = run_generic<A, B, D>(p, first, second, dst->address, s);
             }
         });

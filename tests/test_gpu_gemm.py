@@ -88,6 +88,18 @@ LAYOUTS = {
     "nt_direct_one_step": ((50, 264, 64), (50, 264, 64), [], [("transpose", (-1, -2))]),
     "nt_direct_two_steps": ((50, 264, 128), (50, 264, 128), [], [("transpose", (-1, -2))]),
     "nt_direct_ragged_rows": ((10, 1000, 192), (10, 1096, 192), [], [("transpose", (-1, -2))]),
+    # enough tiles of 128 x 128 to fill the chip (float64: wavefronts of 4 x 4 MFMA tiles, each walking all of K), a
+    # thousand square (float64: 64 x 64 per workgroup, its wavefronts sharing K; under a K of 100 side by side), every layout
+    "many_tiles_nt": ((2001, 40), (2039, 40), [], [("transpose", (-1, -2))]),
+    "many_tiles_nn": ((2001, 40), (40, 2039), [], []),
+    "many_tiles_tn": ((40, 2001), (40, 2039), [("transpose", (-1, -2))], []),
+    "many_tiles_tt": ((40, 2001), (2039, 40), [("transpose", (-1, -2))], [("transpose", (-1, -2))]),
+    "thousand_square_nt": ((1000, 200), (1010, 200), [], [("transpose", (-1, -2))]),
+    "thousand_square_nn": ((1000, 200), (200, 1010), [], []),
+    "thousand_square_tn": ((200, 1000), (200, 1010), [("transpose", (-1, -2))], []),
+    "thousand_square_tt": ((200, 1000), (1010, 200), [("transpose", (-1, -2))], [("transpose", (-1, -2))]),
+    "thousand_square_short_k_nt": ((1000, 100), (1010, 100), [], [("transpose", (-1, -2))]),
+    "thousand_square_short_k_nn": ((1000, 100), (100, 1010), [], []),
 }
 
 
