@@ -55,9 +55,18 @@ static int run_unfold_batch(const ConvProblem& p, int dtype, const void* x, cons
     // columns in all for whole tiles of the product.
     // (ANY_SIZE, fp16, us against the general tile kernel: K = 2352 49 / 104, 648 13 / 38, 600 22 / 31, 360 23 / 26, but 216 20 / 15,
     // 144 33 / 25, 72 25 / 16: with a short K the unfolded operand is as large as the work)
-    if ((ANY_SIZE ? K < 320 : (pixels > 100 || K < 512)) || K % E != 0 || K >= (1u << 24) || pixels >= (1u << 24)) return TANNIC_UNSUPPORTED_DTYPE;
+    // More pixels per image, but few in the whole batch, leave the patch kernels with a handful of blocks that each walk
+    // all of K, where the product shares K between blocks; signals one row high (conv1d) also fill their patches badly.
+    // (fp16, us patches / unfolded: batch 8 256 -> 256 1x7 over 256 75 / 23, batch 32 512 -> 128 1x3 over 256 76 / 33,
+    // batch 1 512 -> 512 5x5 over 28 x 28 119 / 42, batch 8 256 -> 128 5x5 over 14 x 14 63 / 37; but batch 8 over 28 x 28,
+    // 6272 pixels, 64 / 67 and 139 / 207; with a stride of 2 and 512 channels, batch 32 over 28 x 28, 136 / 80)
+    const uint64_t batch_pixels = p.N * pixels;
+    const bool few = pixels <= 100 ? K >= 512
+                                   : (K >= 768 && (batch_pixels <= 2048 || (p.HO == 1 && batch_pixels <= 8192))) || (K >= 2304 && batch_pixels <= 4096) ||
+                                         (K >= 4608 && batch_pixels <= 8192 && p.stride_h > 1 && p.stride_w > 1);
+    if ((ANY_SIZE ? K < 320 : !few) || K % E != 0 || K >= (1u << 24) || pixels >= (1u << 24)) return TANNIC_UNSUPPORTED_DTYPE;
     const uint32_t pitch = static_cast<uint32_t>((pixels + E - 1) / E * E);
-    if (static_cast<uint64_t>(p.N) * pitch < 256) return TANNIC_UNSUPPORTED_DTYPE;
+    if (static_cast<uint64_t>(p.N) * pitch < (ANY_SIZE ? 16 : 256)) return TANNIC_UNSUPPORTED_DTYPE;
     // The unfolded operand is kept small: ANY_SIZE takes the images in runs whose unfolded operand stays within the
     // limit (one image's may reach four times that), one product per run, all through the same buffer.
     const uint64_t limit = (ANY_SIZE ? 256ull : 512ull) << 20, image_bytes = K * pitch * sizeof(T);
@@ -66,7 +75,6 @@ static int run_unfold_batch(const ConvProblem& p, int dtype, const void* x, cons
         if (!ANY_SIZE || image_bytes > 4 * limit) return TANNIC_UNSUPPORTED_DTYPE;
         run = static_cast<uint32_t>(limit / image_bytes);
         if (run == 0) run = 1;
-        if (static_cast<uint64_t>(run) * pitch < 256) return TANNIC_UNSUPPORTED_DTYPE;
     }
     const uint64_t columns = static_cast<uint64_t>(run) * pitch;
     if (columns >= (1ull << 31) || K * run * (pitch / E) >= (1ull << 31)) return TANNIC_UNSUPPORTED_DTYPE;

@@ -110,6 +110,11 @@ CASES = {
     "unfolded_any_k7_48ch": ((2, 48, 20, 20), (48, 48, 7, 7), (1, 1), (3, 3)),
     "unfolded_any_k3_72ch": ((4, 72, 17, 17), (100, 72, 3, 3), (1, 1), (1, 1)),
     "unfolded_any_k3_40ch_s2": ((3, 40, 21, 19), (24, 40, 3, 3), (2, 2), (1, 1)),
+    # ... more pixels per image but few in the whole batch, signals one row high (conv1d's shape), and one image under a
+    # K beyond the general tiles' table (fewer columns than a tile is wide)
+    "unfolded_few_pixels_in_batch": ((2, 96, 14, 14), (24, 96, 3, 3), (1, 1), (1, 1)),
+    "unfolded_one_row_high": ((4, 128, 1, 200), (40, 128, 1, 7), (1, 2), (0, 3)),
+    "unfolded_any_one_image_long_k": ((1, 160, 12, 12), (8, 160, 7, 7), (1, 1), (3, 3)),
     # ... in runs of images when the whole batch unfolded would be large (13 images and 1; one image at a time), with a
     # K beyond what the general tiles keep a table of
     "unfolded_any_runs_of_images": ((14, 128, 40, 40), (4, 128, 7, 7), (1, 1), (3, 3)),
