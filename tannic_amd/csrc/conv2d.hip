@@ -106,7 +106,7 @@ static int conv2d_entry(const tannic_tensor_t* x, const tannic_tensor_t* w, cons
     if (!pointwise) status = conv2d_stem(p, x->dtype, x->address, w->address, pb, y->address, s);
     if (status != TANNIC_UNSUPPORTED_DTYPE) return status;
     // few pixels per image under many channels: the unfolded batch as one product (before the patch kernels, whose tile would be mostly empty)
-    if (!pointwise) status = conv2d_unfold_batch(p, x->dtype, x->address, w->address, pb, y->address, s);
+    if (!pointwise || x->dtype == TANNIC_FLOAT64) status = conv2d_unfold_batch(p, x->dtype, x->address, w->address, pb, y->address, s);
     if (status != TANNIC_UNSUPPORTED_DTYPE) return status;
     if (!pointwise) status = conv2d_k3(p, x->dtype, x->address, w->address, pb, y->address, s);
     if (status != TANNIC_UNSUPPORTED_DTYPE) return status;

@@ -64,7 +64,11 @@ static int run_unfold_batch(const ConvProblem& p, int dtype, const void* x, cons
     const bool few = pixels <= 100 ? K >= 512
                                    : (K >= 768 && (batch_pixels <= 2048 || (p.HO == 1 && batch_pixels <= 8192))) || (K >= 2304 && batch_pixels <= 4096) ||
                                          (K >= 4608 && batch_pixels <= 8192 && p.stride_h > 1 && p.stride_w > 1);
-    if ((ANY_SIZE ? K < 320 : !few) || K % E != 0 || K >= (1u << 24) || pixels >= (1u << 24)) return TANNIC_UNSUPPORTED_DTYPE;
+    // (float64: the alternative is the scalar kernel, which sixteen output channels sharing an unfolded column already beat;
+    // its product reads single doubles and asks nothing of K or of where the weights lie)
+    constexpr bool f64 = std::is_same_v<T, double>;
+    if (f64 ? (K < 16 || p.O < 16) : ((ANY_SIZE ? K < 320 : !few) || K % E != 0)) return TANNIC_UNSUPPORTED_DTYPE;
+    if (K >= (1u << 24) || pixels >= (1u << 24)) return TANNIC_UNSUPPORTED_DTYPE;
     const uint32_t pitch = static_cast<uint32_t>((pixels + E - 1) / E * E);
     if (static_cast<uint64_t>(p.N) * pitch < (ANY_SIZE ? 16 : 256)) return TANNIC_UNSUPPORTED_DTYPE;
     // The unfolded operand is kept small: ANY_SIZE takes the images in runs whose unfolded operand stays within the
@@ -80,7 +84,7 @@ static int run_unfold_batch(const ConvProblem& p, int dtype, const void* x, cons
     if (columns >= (1ull << 31) || K * run * (pitch / E) >= (1ull << 31)) return TANNIC_UNSUPPORTED_DTYPE;
     // the kernel tensor as a K-contiguous O x K matrix, the result as pixel-contiguous rows
     if (p.ws[3] != 1 || p.ws[2] != static_cast<int64_t>(p.KW) || p.ws[1] != static_cast<int64_t>(p.KH) * p.KW || p.ws[0] != static_cast<int64_t>(K) ||
-        reinterpret_cast<uintptr_t>(w) % 16 != 0)
+        (!f64 && reinterpret_cast<uintptr_t>(w) % 16 != 0))
         return TANNIC_UNSUPPORTED_DTYPE;
     if (p.ys[3] != 1 || p.ys[2] != static_cast<int64_t>(p.WO)) return TANNIC_UNSUPPORTED_DTYPE;
     T* col = nullptr;
@@ -118,7 +122,8 @@ static int run_unfold_batch(const ConvProblem& p, int dtype, const void* x, cons
             g.a_bs[d] = g.b_bs[d] = g.c_bs[d] = 0;
         }
         g.row_bias = bias;
-        if constexpr (std::is_same_v<T, float>) status = gemm_mfma_f32(g, static_cast<const float*>(w), reinterpret_cast<const float*>(col), static_cast<float*>(y_part), stream);
+        if constexpr (f64) status = gemm_mfma_f64(g, static_cast<const double*>(w), reinterpret_cast<const double*>(col), static_cast<double*>(y_part), stream);
+        else if constexpr (std::is_same_v<T, float>) status = gemm_mfma_f32(g, static_cast<const float*>(w), reinterpret_cast<const float*>(col), static_cast<float*>(y_part), stream);
         else status = gemm_mfma_16bit(g, dtype, w, col, y_part, stream);
         if (status == TANNIC_UNSUPPORTED_DTYPE) {
             set_error_text("conv2d: internal: the unfolded product refused a problem its caller had checked");
@@ -130,6 +135,8 @@ static int run_unfold_batch(const ConvProblem& p, int dtype, const void* x, cons
 }
 
 int conv2d_unfold_batch(const ConvProblem& p, int dtype, const void* x, const void* w, const void* bias, void* y, hipStream_t stream) {
+    // float64 has this path and the scalar kernel only (a 1x1 kernel's "unfolding" is a copy of the signal)
+    if (dtype == TANNIC_FLOAT64) return run_unfold_batch<double, true>(p, dtype, x, w, bias, y, stream);
     if (p.KH == 1 && p.KW == 1) return TANNIC_UNSUPPORTED_DTYPE;   // conv2d_pointwise.hip: no unfolding needed
     if (dtype == TANNIC_FLOAT16) return run_unfold_batch<f16, false>(p, dtype, x, w, bias, y, stream);
     if (dtype == TANNIC_BFLOAT16) return run_unfold_batch<bf16, false>(p, dtype, x, w, bias, y, stream);

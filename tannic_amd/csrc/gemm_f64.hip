@@ -98,13 +98,23 @@ __global__ __launch_bounds__(256) void gemm_f64_kernel(const double* A, const do
     }
 
     // (sixteen lanes write sixteen consecutive doubles of a row)
+    // With grouped columns (GemmProblem::c_group) column j of group q goes to C + q * c_group_stride + row * c_rs + j, and
+    // the columns past a group's live ones nowhere; a per-row start value (row_bias) is added to the finished sum.
     auto store_tile = [&](int i, int j, const double4v& sum) {
         const uint32_t col = n0 + 16 * j + r;
         if (col >= p.N) return;
+        int64_t at = oc + col;
+        if (p.c_group) {
+            uint32_t q, within;
+            p.c_group_div.divmod(col, q, within);
+            if (within >= p.c_group_live) return;
+            at = static_cast<int64_t>(q) * p.c_group_stride + within;
+        }
+        const double* bias = static_cast<const double*>(p.row_bias);
 #pragma unroll
         for (int v = 0; v < 4; ++v) {
             const uint32_t row = m0 + 16 * i + 4 * v + g;
-            if (row < p.M) C[oc + static_cast<int64_t>(row) * p.c_rs + col] = sum[v];
+            if (row < p.M) C[at + static_cast<int64_t>(row) * p.c_rs] = bias ? sum[v] + bias[row] : sum[v];
         }
     };
     if constexpr (SPLIT) {
@@ -166,7 +176,7 @@ static int launch_f64(const GemmProblem& p, const double* a, const double* b, do
 }
 
 int gemm_mfma_f64(const GemmProblem& p, const double* a, const double* b, double* c, hipStream_t stream) {
-    if (p.row_bias || p.c_group || p.b_group_stride) return TANNIC_UNSUPPORTED_DTYPE;
+    if (p.b_group_stride || (p.c_group && p.batches != 1)) return TANNIC_UNSUPPORTED_DTYPE;
     // (fewer than 17 rows under a long K stream through the kernels for few rows: they are bound by memory)
     if (p.M < 8 || p.N < 8 || p.K < 16 || p.batches == 0 || p.batches > 65535) return TANNIC_UNSUPPORTED_DTYPE;
     if (p.M <= 16 && p.a_cs == 1 && p.b_rs == 1 && p.K >= 256) return TANNIC_UNSUPPORTED_DTYPE;
