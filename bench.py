@@ -37,7 +37,7 @@ import numpy as np  # noqa: E402
 
 PREHEAT_SECONDS = 0.25
 SECONDARY_PREHEAT_SECONDS = 0.08   # the secondary matrix workloads: as long as it takes the clock to settle
-MFMA_PEAK_TFLOPS = {"f16": 2500.0, "bf16": 2500.0, "f32": 157.3, "i8": 5000.0}   # i8: tera-operations per second
+MFMA_PEAK_TFLOPS = {"f16": 2500.0, "bf16": 2500.0, "f32": 157.3, "f64": 78.6, "i8": 5000.0}   # i8: tera-operations per second
 HBM_PEAK_GBS = 8000.0
 
 
@@ -150,7 +150,7 @@ def gemm_entry(b, dtype, M, N, K, iters, layout="NT"):
     flops = 2.0 * M * N * K
     nbytes = (M * K + N * K) * dtype.itemsize + M * N * y.dtype.itemsize
     tflops, gbs = flops / ms / 1e9, nbytes / ms / 1e6
-    peak = MFMA_PEAK_TFLOPS["f32" if dtype is ta.float32 else "i8" if dtype is ta.int8 else "f16"]
+    peak = MFMA_PEAK_TFLOPS["f64" if dtype is ta.float64 else "f32" if dtype is ta.float32 else "i8" if dtype is ta.int8 else "f16"]
     hbm_bound = flops / nbytes < peak * 1e3 / HBM_PEAK_GBS   # below the ridge of the matrix peak over 8 TB/s
     name = {"NT": f"X[{M},{K}].W[{N},{K}]^T", "NN": f"X[{M},{K}].W[{K},{N}]", "TN": f"X[{K},{M}]^T.W[{K},{N}]"}[layout]
     return {"op": f"gemm {dtype} {name}", "us": round(ms * 1e3, 2), "tflops": round(tflops, 2), "gbs": round(gbs, 1),
@@ -484,6 +484,8 @@ def secondary(b, only):
         work.append(gemm_entry(b, ta.float32, 4096, 4096, 4096, 5))
         work.append(gemm_entry(b, ta.float32, 16, 4096, 4096, 20))       # the reference's default type through a linear layer, few rows
         work.append(gemm_entry(b, ta.bfloat16, 64, 4096, 4096, 20))
+        work.append(gemm_entry(b, ta.float64, 2048, 2048, 2048, 5))
+        work.append(gemm_entry(b, ta.float64, 512, 512, 512, 20))
     if only in (None, "gemm-ceiling"):
         work += gemm_ceiling_entries(b)
     if only in (None, "conv"):
