@@ -21,6 +21,8 @@
 //     b[2,3,K,N] by its row stride;
 //   - operand extents are checked against the destination's (the CPU path
 //     takes M and N from the destination and K from the first operand on trust).
+#include <utility>
+
 #include "gemm_common.hpp"
 
 namespace th {
@@ -251,6 +253,52 @@ using namespace th;
 
 namespace {
 
+// A dense copy of `t` in the element type `dtype`, laid out in the order of t's own strides (a transposed matrix stays
+// transposed: the copy reads and writes along the same dimension).  `out` describes the copy with t's extents.
+// TANNIC_UNSUPPORTED_DTYPE: t is not copied (broadcast or reversed dims, too large).
+int dense_copy_as(const tannic_tensor_t* t, int dtype, tannic_tensor_t& out, void*& held, tannic_stream_t stream) {
+    held = nullptr;
+    const int rank = t->rank;
+    uint64_t elements = 1;
+    int order[TANNIC_DIMENSIONS];
+    for (int d = 0; d < rank; ++d) {
+        if (t->shape.sizes[d] != 1 && t->strides.sizes[d] <= 0) return TANNIC_UNSUPPORTED_DTYPE;
+        elements *= t->shape.sizes[d];
+        order[d] = d;
+    }
+    if (elements == 0 || elements >= (1ull << 31)) return TANNIC_UNSUPPORTED_DTYPE;
+    // dims by stride, largest first; extents of 1 (whose stride is never used) lead
+    auto key = [&](int d) { return t->shape.sizes[d] == 1 ? INT64_MAX : t->strides.sizes[d]; };
+    for (int i = 1; i < rank; ++i)
+        for (int j = i; j > 0 && key(order[j]) > key(order[j - 1]); --j) std::swap(order[j], order[j - 1]);
+    tannic_tensor_t source = *t, dense = *t;
+    int64_t pitch = 1;
+    for (int i = rank - 1; i >= 0; --i) {
+        source.shape.sizes[i] = dense.shape.sizes[i] = t->shape.sizes[order[i]];
+        source.strides.sizes[i] = t->strides.sizes[order[i]];
+        dense.strides.sizes[i] = pitch;
+        pitch *= static_cast<int64_t>(dense.shape.sizes[i]);
+    }
+    source.layout = TANNIC_STRIDED;
+    if (scratch_acquire(&held, elements * dtype_size(dtype), as_stream(stream)) != TANNIC_SUCCESS) return TANNIC_ERROR;
+    dense.address = held;
+    dense.dtype = static_cast<tannic_type>(dtype);
+    dense.layout = TANNIC_CONTIGUOUS;
+    dense.size = elements;
+    const int status = tannic_hip_cast(&source, &dense, stream);
+    if (status != TANNIC_SUCCESS) {
+        scratch_release(held, as_stream(stream));
+        held = nullptr;
+        return status;
+    }
+    out = *t;
+    out.address = held;
+    out.dtype = static_cast<tannic_type>(dtype);
+    out.layout = TANNIC_STRIDED;
+    for (int i = 0; i < rank; ++i) out.strides.sizes[order[i]] = dense.strides.sizes[i];
+    return TANNIC_SUCCESS;
+}
+
 int gemm_entry(const tannic_tensor_t* a, const tannic_tensor_t* b, tannic_tensor_t* dst, tannic_stream_t stream, const GemmWorkspace* workspace) {
     if (!a || !b || !dst) return TANNIC_ERROR;
     if (!have_storage(a, b, dst)) return TANNIC_ERROR;
@@ -269,6 +317,29 @@ int gemm_entry(const tannic_tensor_t* a, const tannic_tensor_t* b, tannic_tensor
                 GemmProblem p;
                 status = describe_gemm(a, b, dst, p);
                 if (status != TANNIC_SUCCESS) return;
+                if constexpr (!std::is_same_v<A, B> && (std::is_same_v<D, float> || std::is_same_v<D, double>)) {
+                    // A product of two different types whose result is fp32 or float64 multiplies static_cast<D>(a) by
+                    // static_cast<D>(b) (src/cpu/matmul.cpp:36): the same numbers as the product of the operands converted
+                    // to D first, which runs on the matrix pipe where this pair has the scalar kernel only.  Worth the
+                    // copies from a few million multiply-adds on; never on the path that must not allocate.
+                    // (with few rows the scalar kernels stream the large operand once as it is: converting it first would
+                    // read and write it once more - fp32 x bf16, 16 rows over 4096 x 4096: 37 against 39 us, float64 x fp32 67 against 114)
+                    const bool few_rows_stream = p.M <= 16 && p.a_cs == 1 && p.b_rs == 1 && p.K >= 256 && !std::is_same_v<B, D>;
+                    if (workspace == nullptr && !few_rows_stream && static_cast<double>(p.M) * p.N * p.K * p.batches >= static_cast<double>(1 << 24)) {
+                        tannic_tensor_t a2 = *a, b2 = *b;
+                        void* held[2] = {nullptr, nullptr};
+                        int copied = TANNIC_SUCCESS;
+                        if (!std::is_same_v<A, D>) copied = dense_copy_as(a, dtype_code<D>(), a2, held[0], stream);
+                        if (copied == TANNIC_SUCCESS && !std::is_same_v<B, D>) copied = dense_copy_as(b, dtype_code<D>(), b2, held[1], stream);
+                        if (copied == TANNIC_SUCCESS) copied = gemm_entry(&a2, &b2, dst, stream, workspace);
+                        for (void* h : held)
+                            if (h) scratch_release(h, s);
+                        if (copied != TANNIC_UNSUPPORTED_DTYPE) {
+                            status = copied;
+                            return;
+                        }
+                    }
+                }
                 const void *first = a->address, *second = b->address;
                 if constexpr (std::is_same_v<A, B>) {
                     // A matrix times a column, y = A . v: the same numbers are v^T . A^T, one row times a matrix whose "rows of

@@ -100,6 +100,8 @@ LAYOUTS = {
     "thousand_square_tt": ((200, 1000), (1010, 200), [("transpose", (-1, -2))], [("transpose", (-1, -2))]),
     "thousand_square_short_k_nt": ((1000, 100), (1010, 100), [], [("transpose", (-1, -2))]),
     "thousand_square_short_k_nn": ((1000, 100), (100, 1010), [], []),
+    "rank4_rank2_nt_large": ((2, 3, 200, 320), (480, 320), [], [("transpose", (-1, -2))]),
+    "stream_49_rows_long_k_wide": ((49, 2048), (400, 2048), [], [("transpose", (-1, -2))]),
 }
 
 
@@ -215,6 +217,20 @@ def test_mixed_gemm(device, pair):
     want, got = ops.matmul(*host), ops.matmul(*dev)
     assert got.dtype is want.dtype
     support.assert_close(got.numpy(), want.numpy(), 1e-5, k * 9 * 2.0 ** -24, f"gemm {pair}")
+
+
+@pytest.mark.parametrize("layout", ["thousand_square_nt", "thousand_square_tn", "nn_large_tiles_batched", "rank4_rank2_nt_large", "stream_49_rows_long_k_wide"])
+@pytest.mark.parametrize("pair", [(ta.int32, ta.float32), (ta.float64, ta.float32), (ta.float16, ta.float32), (ta.float32, ta.bfloat16), (ta.bfloat16, ta.float64),
+                                  (ta.int64, ta.float16), (ta.int32, ta.bfloat16)], ids=lambda p: f"{p[0]}-{p[1]}")
+def test_large_mixed_gemm_multiplies_converted_copies(device, pair, layout):
+    """Pairs of different types with an fp32 / float64 result, large enough that the operands are converted to the result
+    type first (in the order of their own strides) and multiplied on the matrix pipe: the same numbers as
+    static_cast<D>(a) * static_cast<D>(b) summed (src/cpu/matmul.cpp:36), in a different order."""
+    host, dev, k = operands(pair, layout, device, -3, 3)
+    want, got = ops.matmul(*host), ops.matmul(*dev)
+    assert got.dtype is want.dtype and got.shape == want.shape
+    eps = 2.0 ** -53 if want.dtype is ta.float64 else 2.0 ** -24
+    support.assert_close(got.numpy(), want.numpy(), 1e-13 if want.dtype is ta.float64 else 1e-5, k * 9 * eps, f"gemm {pair} {layout}")
 
 
 def test_operand_with_fewer_batch_dims_steps_by_its_own_batch_stride(device):
