@@ -485,6 +485,10 @@ int gemm_mfma_int8(const GemmProblem& p, const void* a, const void* b, void* c, 
     if (reinterpret_cast<uintptr_t>(a) % 16 || reinterpret_cast<uintptr_t>(b) % 16 || p.a_rs % 16 || p.b_cs % 16) return TANNIC_UNSUPPORTED_DTYPE;
     for (int d = 0; d < p.batch_rank; ++d)
         if (p.a_bs[d] % 16 || p.b_bs[d] % 16) return TANNIC_UNSUPPORTED_DTYPE;
+    if (p.M <= 32) {
+        const int status = gemm_skinny_int8(p, a, b, c, stream);
+        if (status != TANNIC_UNSUPPORTED_DTYPE) return status;
+    }
     auto tiles = [&](uint64_t bm, uint64_t bn) { return ((p.M + bm - 1) / bm) * ((p.N + bn - 1) / bn) * p.batches; };
     if (p.M > 192 && tiles(256, 256) >= 200) return gemm16_dtl<int8_t>(p, 256, 256, a, b, c, stream);
     if (p.M > 192 && tiles(256, 128) >= 128) return gemm16_dtl<int8_t>(p, 256, 128, a, b, c, stream);

@@ -43,6 +43,21 @@ template <> __device__ inline float4y skinny_mfma<float>(uint4y a, uint4y b, flo
     return c;
 }
 
+// int8: 16 bytes are sixteen k of the lane's row, one v_mfma_i32_16x16x64_i8 per four chunks; sums and results are int32
+typedef int int4y __attribute__((ext_vector_type(4)));
+template <class T> struct SkinnyTypes { using Acc = float4y; using Out = T; };
+template <> struct SkinnyTypes<int8_t> { using Acc = int4y; using Out = int32_t; };
+template <class T> __device__ inline typename SkinnyTypes<T>::Acc skinny_step(uint4y a, uint4y b, typename SkinnyTypes<T>::Acc c) {
+    if constexpr (std::is_same_v<T, int8_t>) {
+        int4y x, y;
+        __builtin_memcpy(&x, &a, 16);
+        __builtin_memcpy(&y, &b, 16);
+        return __builtin_amdgcn_mfma_i32_16x16x64_i8(x, y, c, 0, 0, 0);
+    } else {
+        return skinny_mfma<T>(a, b, c);
+    }
+}
+
 constexpr int kSkinnyWaves = 8;
 constexpr int kSkinnyUnroll = 8;   // K steps of 32 whose loads are issued together
 
@@ -147,8 +162,11 @@ constexpr int kStreamWaves = 4;
 constexpr int kStreamBytesPerWave = 32 * 1024;
 
 template <class T, int MB, int NB>
-__global__ __launch_bounds__(64 * kStreamWaves) void gemm_skinny_stream_kernel(const T* x, const T* w, T* c, GemmProblem p, uint32_t windows_per_wave) {
+__global__ __launch_bounds__(64 * kStreamWaves) void gemm_skinny_stream_kernel(const T* x, const T* w, typename SkinnyTypes<T>::Out* c, GemmProblem p,
+                                                                               uint32_t windows_per_wave) {
 #if defined(__HIP_DEVICE_COMPILE__)
+    using Acc = typename SkinnyTypes<T>::Acc;
+    using Out = typename SkinnyTypes<T>::Out;
     constexpr int BLOCKS = MB + NB;                       // 16-row blocks per window: W's, then x's
     constexpr int STAGE_BYTES = BLOCKS * 2048, STAGES = kStreamBytesPerWave / STAGE_BYTES, LOADS = 2 * BLOCKS;
     static_assert(STAGES >= 3, "a ring of at least three windows");
@@ -186,11 +204,11 @@ __global__ __launch_bounds__(64 * kStreamWaves) void gemm_skinny_stream_kernel(c
     const uint32_t first = wave * windows_per_wave;
     const uint32_t count = first >= all ? 0 : (all - first < windows_per_wave ? all - first : windows_per_wave);
 
-    float4y acc[MB][NB];
+    Acc acc[MB][NB];
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb)
 #pragma unroll
-        for (int nb = 0; nb < NB; ++nb) acc[mb][nb] = float4y{0.0f, 0.0f, 0.0f, 0.0f};
+        for (int nb = 0; nb < NB; ++nb) acc[mb][nb] = Acc{0, 0, 0, 0};
 #pragma unroll
     for (int t = 0; t < STAGES - 1; ++t)
         if (static_cast<uint32_t>(t) < count) issue(first + t, t);
@@ -216,35 +234,38 @@ __global__ __launch_bounds__(64 * kStreamWaves) void gemm_skinny_stream_kernel(c
 #pragma unroll
             for (int mb = 0; mb < MB; ++mb)
 #pragma unroll
-                for (int nb = 0; nb < NB; ++nb) acc[mb][nb] = skinny_mfma<T>(fw[half][nb], fx[half][mb], acc[mb][nb]);
+                for (int nb = 0; nb < NB; ++nb) acc[mb][nb] = skinny_step<T>(fw[half][nb], fx[half][mb], acc[mb][nb]);
         stage = stage + 1 == STAGES ? 0 : stage + 1;
         fill = fill + 1 == STAGES ? 0 : fill + 1;
     }
     // the wavefronts' tiles meet in LDS (every wavefront's ring has been read: its own MFMAs needed the data)
     __syncthreads();
-    float4y* partial = reinterpret_cast<float4y*>(skinny_lds);     // [wave][tile][lane]
+    Acc* partial = reinterpret_cast<Acc*>(skinny_lds);     // [wave][tile][lane]
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb)
 #pragma unroll
         for (int nb = 0; nb < NB; ++nb) partial[(wave * MB * NB + mb * NB + nb) * 64 + lane] = acc[mb][nb];
     __syncthreads();
     // accumulator: lane -> row of x (m) lane % 16; value v -> column n0 + 4 * (lane / 16) + v; wavefront t adds up tile t, t + 4, ..
-    T* cb = c + oc;
-    const bool vector_ok = p.c_rs % 4 == 0 && p.N % 4 == 0 && reinterpret_cast<uintptr_t>(cb) % (4 * sizeof(T)) == 0;
+    Out* cb = c + oc;
+    const bool vector_ok = p.c_rs % 4 == 0 && p.N % 4 == 0 && reinterpret_cast<uintptr_t>(cb) % (4 * sizeof(Out)) == 0;
     for (int t = wave; t < MB * NB; t += kStreamWaves) {
         const int mb = t / NB, nb = t % NB;
-        float4y sum = partial[t * 64 + lane];
+        Acc sum = partial[t * 64 + lane];
 #pragma unroll
         for (int v = 1; v < kStreamWaves; ++v) sum += partial[(v * MB * NB + t) * 64 + lane];
         const uint32_t m = mb * 16 + r, col = n0 + nb * 16 + 4 * kc;
         if (m >= p.M) continue;
-        T out[4];
+        Out out[4];
 #pragma unroll
-        for (int e = 0; e < 4; ++e) out[e] = narrow_result<T>(sum[e]);
-        T* dst = cb + static_cast<int64_t>(m) * p.c_rs + col;
+        for (int e = 0; e < 4; ++e) {
+            if constexpr (std::is_same_v<T, int8_t>) out[e] = sum[e];
+            else out[e] = narrow_result<T>(sum[e]);
+        }
+        Out* dst = cb + static_cast<int64_t>(m) * p.c_rs + col;
         if (vector_ok) {
             if (col < p.N) {
-                using Quad = std::conditional_t<sizeof(T) == 2, uint2, uint4>;
+                using Quad = std::conditional_t<sizeof(Out) == 2, uint2, uint4>;
                 Quad bits;
                 __builtin_memcpy(&bits, out, sizeof(Quad));
                 *reinterpret_cast<Quad*>(dst) = bits;
@@ -266,7 +287,7 @@ static int launch_stream(const GemmProblem& p, const void* a, const void* b, voi
     if (int rc = raise_lds_limit(reinterpret_cast<const void*>(kernel), lds, configured)) return rc;
     const uint32_t windows = p.K / kBKof<T>, per_wave = (windows + kStreamWaves - 1) / kStreamWaves;
     hipLaunchKernelGGL(kernel, dim3((p.N + 16 * NB - 1) / (16 * NB), p.batches), dim3(64 * kStreamWaves), lds, stream, static_cast<const T*>(a), static_cast<const T*>(b),
-                       static_cast<T*>(c), p, per_wave);
+                       static_cast<typename SkinnyTypes<T>::Out*>(c), p, per_wave);
     return launch_status("gemm_skinny_stream_kernel");
 }
 
@@ -291,8 +312,9 @@ int run_skinny(const GemmProblem& p, const void* a, const void* b, void* c, hipS
         const bool two = static_cast<uint64_t>((p.N + 31) / 32) * p.batches >= 400;
         if (p.M <= 16) return two ? launch_stream<T, 1, 2>(p, a, b, c, stream) : launch_stream<T, 1, 1>(p, a, b, c, stream);
         if (p.M <= 32) return two ? launch_stream<T, 2, 2>(p, a, b, c, stream) : launch_stream<T, 2, 1>(p, a, b, c, stream);
-        // (fp32 stops here: with more row blocks its MFMAs, a sixteenth as fast, take longer than W takes to arrive)
-        if constexpr (sizeof(T) == 4) {
+        // (fp32 stops here: with more row blocks its MFMAs, a sixteenth as fast, take longer than W takes to arrive; int8
+        // beyond 32 rows has its tiles)
+        if constexpr (sizeof(T) != 2) {
             return TANNIC_UNSUPPORTED_DTYPE;
         } else {
             // Up to 64 rows: every wavefront still brings its own windows of x, three or four 16-row blocks next to one of W, so
@@ -306,7 +328,7 @@ int run_skinny(const GemmProblem& p, const void* a, const void* b, void* c, hipS
             return launch_stream<T, 4, 1>(p, a, b, c, stream);
         }
     }
-    if constexpr (sizeof(T) == 4) {
+    if constexpr (sizeof(T) != 2) {
         return TANNIC_UNSUPPORTED_DTYPE;   // the kernel for other K is written for 16-bit fragments
     } else {
         if (p.M > 32) return TANNIC_UNSUPPORTED_DTYPE;
@@ -333,6 +355,9 @@ int run_skinny(const GemmProblem& p, const void* a, const void* b, void* c, hipS
 }
 
 int gemm_skinny_f32(const GemmProblem& p, const float* a, const float* b, float* c, hipStream_t stream) { return run_skinny<float>(p, a, b, c, stream); }
+
+// int8 x int8 -> int32, at most 32 rows over whole windows of 128 k: W goes by once where the 128-row tiles walk it at their own pace
+int gemm_skinny_int8(const GemmProblem& p, const void* a, const void* b, void* c, hipStream_t stream) { return run_skinny<int8_t>(p, a, b, c, stream); }
 
 int gemm_skinny_16bit(const GemmProblem& p, int dtype, const void* a, const void* b, void* c, hipStream_t stream) {
     if (dtype == TANNIC_FLOAT16) return run_skinny<f16>(p, a, b, c, stream);

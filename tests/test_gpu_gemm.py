@@ -152,12 +152,16 @@ def test_integer_gemm_bit_exact(device, pair, layout):
 
 @pytest.mark.parametrize("shape", [((300, 256), (520, 256)), ((16, 300, 128), (16, 520, 128)), ((50, 264, 128), (50, 264, 128)), ((2, 3, 70, 384), (136, 384)),
                                    ((4096, 512), (1024, 512)), ((1, 512), (1024, 512)), ((16, 256), (130, 256)), ((3, 5, 128), (3, 70, 128)),
-                                   ((130, 384), (1001, 384)), ((70, 200), (333, 200)), ((300, 1000), (77, 1000))],
+                                   ((130, 384), (1001, 384)), ((70, 200), (333, 200)), ((300, 1000), (77, 1000)),
+                                   # at most 32 rows over whole windows of 128 k: streamed (one and two row blocks, one and two column
+                                   # blocks per wavefront, ragged columns, a K the four wavefronts do not share evenly, batches)
+                                   ((32, 128), (12840, 128)), ((17, 1280), (200, 1280)), ((5, 640), (12816, 640)), ((4, 9, 384), (4, 90, 384)),
+                                   ((2, 3, 20, 256), (48, 256))],
                          ids=lambda s: "x".join(map(str, s[0])) + "." + "x".join(map(str, s[1])) + "T")
 def test_int8_gemm_on_matrix_cores_is_bit_exact(device, shape):
     """int8 x int8 -> int32 with both operands K-contiguous and K a multiple of 128: the tiled kernels on
     v_mfma_i32_16x16x64_i8 in each tile size (128 x 128, 256 x 128, 256 x 256; ragged rows and columns, batches, a
-    broadcast second operand; one, five and sixteen rows in a 128-row tile; a number of columns no quad divides; K that is
+    broadcast second operand; few rows, which stream W once; a number of columns no quad divides; K that is
     not a multiple of 128, which goes through zero-padded copies of both operands).  Integer sums are exact, so the checker's sequential loop and numpy agree bit for bit."""
     sa, sb = shape
     a = support.integers(SEED, 31, sa, -128, 128).astype(np.int8)
