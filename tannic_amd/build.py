@@ -44,6 +44,7 @@ UNITS = [
     ("gemm_skinny.hip", "gemm_skinny.o", []),
     ("gemm_small.hip", "gemm_small.o", []),
     ("gemm_f64.hip", "gemm_f64.o", []),
+    ("gemm_rows_nn.hip", "gemm_rows_nn.o", []),
     ("gemm_repack.hip", "gemm_repack.o", []),
     ("gemm_dtl.hip", "gemm_dtl.o", ["-DTH_DTL_PART=0"]),
     ("gemm_dtl.hip", "gemm_dtl_krows_f16.o", ["-DTH_DTL_PART=1"]),

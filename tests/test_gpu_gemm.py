@@ -100,6 +100,13 @@ LAYOUTS = {
     "thousand_square_tt": ((200, 1000), (1010, 200), [("transpose", (-1, -2))], [("transpose", (-1, -2))]),
     "thousand_square_short_k_nt": ((1000, 100), (1010, 100), [], [("transpose", (-1, -2))]),
     "thousand_square_short_k_nn": ((1000, 100), (100, 1010), [], []),
+    # at most eight rows times a matrix lying row by row (fp32: W read once along its rows, K shared between workgroups):
+    # one row, a K no eight divides under columns that end inside a wavefront, x transposed, W a slice of a wider matrix
+    "rows_nn_1_row": ((1, 1024), (1024, 512), [], []),
+    "rows_nn_5_rows_ragged": ((5, 1003), (1003, 520), [], []),
+    "rows_nn_8_rows_x_transposed": ((700, 8), (700, 1024), [("transpose", (-1, -2))], []),
+    "rows_nn_3_rows_slice_of_w": ((3, 512), (512, 1100), [], [("index", (slice(None), slice(4, 1028)))]),
+    "rows_nn_2_rows_long_k": ((2, 20000), (20000, 256), [], []),
     "rank4_rank2_nt_large": ((2, 3, 200, 320), (480, 320), [], [("transpose", (-1, -2))]),
     "stream_49_rows_long_k_wide": ((49, 2048), (400, 2048), [], [("transpose", (-1, -2))]),
 }
