@@ -133,8 +133,23 @@ def test_every_operator_family_replays(device):
     img7 = ta.tensor(support.normal(13, 17, (8, 128, 7, 7), 1.0), f16, device)
     ker7 = ta.tensor(support.normal(13, 18, (64, 128, 3, 3), 0.05), f16, device)
 
+    # products that convert an operand of another type first, float64 on its matrix kernel, a float64 convolution through
+    # the unfolded batch, a few fp32 rows times a row-major matrix (partial sums of workgroups that share K), int8 few rows
+    wide32 = ta.tensor(support.normal(13, 19, (200, 1024), 1.0), f32, device)
+    w_bf16 = ta.tensor(support.normal(13, 20, (512, 1024), 0.05), ta.bfloat16, device)
+    a64 = ta.tensor(support.normal(13, 21, (300, 260), 1.0), ta.float64, device)
+    b64 = ta.tensor(support.normal(13, 22, (260, 200), 1.0), ta.float64, device)
+    img64 = ta.tensor(support.normal(13, 23, (2, 8, 12, 12), 1.0), ta.float64, device)
+    ker64 = ta.tensor(support.normal(13, 24, (16, 8, 3, 3), 0.3), ta.float64, device)
+    few32 = ta.tensor(support.normal(13, 25, (3, 2048), 1.0), f32, device)
+    w32 = ta.tensor(support.normal(13, 26, (2048, 1024), 0.05), f32, device)
+    few8 = ta.tensor(support.integers(13, 27, (4, 512), -100, 100), ta.int8, device)
+    w8 = ta.tensor(support.integers(13, 28, (640, 512), -100, 100), ta.int8, device)
+
     def everything():
         return [
+            ops.matmul(wide32, w_bf16.transpose()), ops.matmul(a64, b64), ops.convolve2d(img64, ker64, None, 1, 1),
+            ops.matmul(few32, w32), ops.matmul(few8, w8.transpose()),
             ops.convolve2d(img16, ker16, None, 1, 1),
             ops.convolve2d(img32, ker32, bias32, 2, 1),
             ops.sum(big, 1), ops.mean(big, 0), ops.argmax(big, 1), ops.max(big, 2),
