@@ -108,19 +108,22 @@ __global__ __launch_bounds__(64 * kRowsNnWaves) void gemm_rows_nn_kernel(const T
     }
 }
 
-// c[m][n] = sum over the shares of partial[share][m][n], rounded once; four columns per thread
+// c[m][n] = sum over the shares of partial[share][m][n], rounded once.  A workgroup owns 64 quads of columns; its four
+// wavefronts each add up every fourth share (eight loads in flight) and meet in LDS.
 template <class T>
 __global__ __launch_bounds__(256) void gemm_rows_nn_finish_kernel(const float* partial, T* c, uint32_t M, uint32_t N, int64_t c_rs, uint32_t shares, uint32_t total) {
-    const uint32_t idx = blockIdx.x * 256 + threadIdx.x;
-    if (idx >= total) return;
-    const uint32_t quads = N / 4, m = idx / quads, col = (idx % quads) * 4;
+    __shared__ float4 part[3][64];
+    const uint32_t lane = threadIdx.x % 64, wave = threadIdx.x / 64;
+    const uint32_t idx = blockIdx.x * 64 + lane;
+    const bool live = idx < total;
+    const uint32_t quads = N / 4, m = live ? idx / quads : 0, col = live ? (idx % quads) * 4 : 0;
     const float* src = partial + static_cast<size_t>(m) * N + col;
     const size_t step = static_cast<size_t>(M) * N;
     float4 sum = float4{0.0f, 0.0f, 0.0f, 0.0f};
-    for (uint32_t s0 = 0; s0 < shares; s0 += 8) {
+    for (uint32_t s0 = wave; s0 < shares; s0 += 32) {
         float4 v[8];
 #pragma unroll
-        for (int u = 0; u < 8; ++u) v[u] = s0 + u < shares ? *reinterpret_cast<const float4*>(src + (s0 + u) * step) : float4{0.0f, 0.0f, 0.0f, 0.0f};
+        for (int u = 0; u < 8; ++u) v[u] = (live && s0 + 4 * u < shares) ? *reinterpret_cast<const float4*>(src + (s0 + 4 * u) * step) : float4{0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
         for (int u = 0; u < 8; ++u) {
             sum.x += v[u].x;
@@ -128,6 +131,16 @@ __global__ __launch_bounds__(256) void gemm_rows_nn_finish_kernel(const float* p
             sum.z += v[u].z;
             sum.w += v[u].w;
         }
+    }
+    if (wave != 0) part[wave - 1][lane] = sum;
+    __syncthreads();
+    if (wave != 0 || !live) return;
+#pragma unroll
+    for (int w = 0; w < 3; ++w) {
+        sum.x += part[w][lane].x;
+        sum.y += part[w][lane].y;
+        sum.z += part[w][lane].z;
+        sum.w += part[w][lane].w;
     }
     T* dst = c + static_cast<int64_t>(m) * c_rs + col;
     dst[0] = narrow_result<T>(sum.x);
@@ -144,6 +157,7 @@ static int launch_rows_nn(const GemmProblem& p, const T* x, const T* w, T* c, hi
     uint32_t shares = wanted / groups ? wanted / groups : 1;
     const uint32_t most = (p.K + 8 * kRowsNnWaves - 1) / (8 * kRowsNnWaves);   // at least eight rows of W per wavefront
     if (shares > most) shares = most;
+    if (shares > 128) shares = 128;   // (every share is a row of partial sums the second pass has to add)
     uint32_t chunk = (p.K + shares * kRowsNnWaves - 1) / (shares * kRowsNnWaves);
     chunk = (chunk + 7) / 8 * 8;
     // the staged rows of x must fit (kRowsNnWaves * chunk * MR floats): more shares of K where they would not
@@ -157,7 +171,7 @@ static int launch_rows_nn(const GemmProblem& p, const T* x, const T* w, T* c, hi
     if (partial) {
         if (status == TANNIC_SUCCESS) {
             const uint32_t total = p.M * (p.N / 4);
-            hipLaunchKernelGGL((gemm_rows_nn_finish_kernel<T>), dim3((total + 255) / 256), dim3(256), 0, stream, partial, c, p.M, p.N, p.c_rs, shares, total);
+            hipLaunchKernelGGL((gemm_rows_nn_finish_kernel<T>), dim3((total + 63) / 64), dim3(256), 0, stream, partial, c, p.M, p.N, p.c_rs, shares, total);
             status = launch_status("gemm_rows_nn_finish_kernel");
         }
         scratch_release(partial, stream);
