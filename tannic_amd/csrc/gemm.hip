@@ -403,7 +403,7 @@ int gemm_entry(const tannic_tensor_t* a, const tannic_tensor_t* b, tannic_tensor
                         if (status != TANNIC_UNSUPPORTED_DTYPE) return;   // (refused after all: on with the product as it is)
                     }
                 }
-                if constexpr (std::is_same_v<A, float> && std::is_same_v<B, float>) {
+                if constexpr (std::is_same_v<A, B> && (is_16bit<A>::value || std::is_same_v<A, float>)) {
                     // at most eight rows times a matrix that lies row by row (x . W as written): W is read once, along its rows
                     if (workspace == nullptr) {
                         status = gemm_rows_nn(p, a->dtype, first, second, dst->address, s);

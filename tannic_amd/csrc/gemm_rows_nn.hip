@@ -1,4 +1,4 @@
-// At most eight fp32 rows times a matrix that is contiguous along its columns: y[m][n] = sum over k of x[m][k] * W[k][n] with W[K,N]
+// At most eight rows (fp32; fp16 / bf16 where the tiles do badly) times a matrix that is contiguous along its columns: y[m][n] = sum over k of x[m][k] * W[k][n] with W[K,N]
 // lying row by row (x . W as written, where a linear layer stores W^T).  The work is reading W once, and W's rows are
 // the wrong way round for the matrix instructions (a fragment wants consecutive k of one column), so this is plain
 // fused multiply-adds: a lane owns four consecutive columns, a wavefront 256, and walks its share of K reading whole
@@ -187,6 +187,13 @@ static int run_rows_nn(const GemmProblem& p, const void* a, const void* b, void*
     // W contiguous along its columns and not along K, whole quads of columns, enough of it that reading it is the work
     if (p.b_cs != 1 || p.b_rs == 1 || p.N % 4 != 0 || p.N < 256 || p.K < 64 || static_cast<uint64_t>(p.N) * p.K < (1u << 18)) return TANNIC_UNSUPPORTED_DTYPE;
     if (static_cast<uint64_t>(p.M) * p.N >= (1ull << 31)) return TANNIC_UNSUPPORTED_DTYPE;
+    if constexpr (sizeof(T) == 2) {
+        // The 16-bit tiles that share K pass a wide W at this kernel's pace (fp16, one row over 4096 x 4096: 12 us either
+        // way; 32000 x 512: 8 against 12 here).  What they do badly is a narrow W under a long K (512 x 16384: 16 against
+        // 11 us) and an x that lies column by column with a number of rows no 16 bytes divide, which sends both operands
+        // to the loaders for any alignment (four rows, 256 x 8192: 151 against 9 us).
+        if (!(p.N <= 1024 || (p.a_cs != 1 && p.M % 8 != 0))) return TANNIC_UNSUPPORTED_DTYPE;
+    }
     const T* x = static_cast<const T*>(a);
     const T* w = static_cast<const T*>(b);
     T* y = static_cast<T*>(c);
@@ -195,9 +202,9 @@ static int run_rows_nn(const GemmProblem& p, const void* a, const void* b, void*
 }
 
 int gemm_rows_nn(const GemmProblem& p, int dtype, const void* a, const void* b, void* c, hipStream_t stream) {
-    // fp32 only: the 16-bit tiles that share K already pass W at this kernel's pace (fp16, one row over 4096 x 4096: 12 us
-    // there, 14 here with the second pass), so the kernel's 16-bit instances are not built
     if (dtype == TANNIC_FLOAT32) return run_rows_nn<float>(p, a, b, c, stream);
+    if (dtype == TANNIC_FLOAT16) return run_rows_nn<f16>(p, a, b, c, stream);
+    if (dtype == TANNIC_BFLOAT16) return run_rows_nn<bf16>(p, a, b, c, stream);
     return TANNIC_UNSUPPORTED_DTYPE;
 }
 
