@@ -214,6 +214,73 @@ __global__ __launch_bounds__(256) void gemm_generic_few_rows_kernel(const A* a, 
         }
 }
 
+// Few results under a long K (a handful of dot products: 48 x 13 over K = 12000), any types and strides: a tile kernel has
+// one or two blocks that walk all of K alone.  Here a workgroup owns 4 x 4 results and its 256 lanes stride over K
+// together (consecutive lanes, consecutive k); the sums meet in a butterfly per wavefront and in LDS across the four.
+// Integer sums are exact in any order; floating sums are a tree, within rounding of the CPU path's sequence.
+template <class A, class B, class D>
+__global__ __launch_bounds__(256) void gemm_generic_few_results_kernel(const A* a, const B* b, D* c, GemmProblem p, uint32_t tiles_n) {
+    using Acc = std::conditional_t<is_16bit<D>::value, float, D>;
+    __shared__ Acc part[4][16];
+    int64_t oa, ob, oc;
+    batch_offsets(p, blockIdx.y, oa, ob, oc);
+    const uint32_t m0 = (blockIdx.x / tiles_n) * 4, n0 = (blockIdx.x % tiles_n) * 4;
+    const A* pa[4];
+    const B* pb[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        pa[i] = a + oa + static_cast<int64_t>(m0 + i < p.M ? m0 + i : m0) * p.a_rs + static_cast<int64_t>(threadIdx.x) * p.a_cs;
+        pb[i] = b + ob + static_cast<int64_t>(n0 + i < p.N ? n0 + i : n0) * p.b_cs + static_cast<int64_t>(threadIdx.x) * p.b_rs;
+    }
+    const int64_t step_a = 256 * p.a_cs, step_b = 256 * p.b_rs;
+    Acc acc[4][4] = {};
+#pragma unroll 2
+    for (uint32_t k = threadIdx.x; k < p.K; k += 256) {
+        Acc x[4], y[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            x[i] = static_cast<Acc>(widen(*pa[i]));
+            y[i] = static_cast<Acc>(widen(*pb[i]));
+            pa[i] += step_a;
+            pb[i] += step_b;
+        }
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) acc[i][j] += x[i] * y[j];
+    }
+    const uint32_t lane = threadIdx.x % 64, wave = threadIdx.x / 64;
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            Acc v = acc[i][j];
+#pragma unroll
+            for (int step = 32; step >= 1; step >>= 1) v += __shfl_xor(v, step, 64);
+            if (lane == 0) part[wave][i * 4 + j] = v;
+        }
+    __syncthreads();
+    if (threadIdx.x < 16) {
+        const uint32_t m = m0 + threadIdx.x / 4, n = n0 + threadIdx.x % 4;
+        const Acc v = part[0][threadIdx.x] + part[1][threadIdx.x] + part[2][threadIdx.x] + part[3][threadIdx.x];
+        if (m < p.M && n < p.N) c[oc + static_cast<int64_t>(m) * p.c_rs + n] = narrow<D>(v);
+    }
+}
+
+// Whether the kernel above is the one to run: few results (what a few 64 x 64 tiles hold) under a K of 256 or more.
+// (`most`: 8192 where tiles that share K exist for larger products, 32768 for the types that only have kernels whose blocks walk all of K)
+inline bool few_results_under_a_long_k(const GemmProblem& p, uint64_t most) {
+    return p.M != 0 && p.N != 0 && p.batches != 0 && p.batches <= 65535 && p.K >= 256 && static_cast<uint64_t>(p.M) * p.N * p.batches <= most;
+}
+
+template <class A, class B, class D>
+int run_few_results(const GemmProblem& p, const void* a, const void* b, void* c, hipStream_t stream) {
+    const uint32_t tiles_m = (p.M + 3) / 4, tiles_n = (p.N + 3) / 4;
+    hipLaunchKernelGGL((gemm_generic_few_results_kernel<A, B, D>), dim3(tiles_m * tiles_n, p.batches), dim3(256), 0, stream, static_cast<const A*>(a), static_cast<const B*>(b),
+                       static_cast<D*>(c), p, tiles_n);
+    return launch_status("gemm_generic_few_results_kernel");
+}
+
 // c[m * c_rs + n] = t[n * M + m]: the few rows of a transposed result back into the columns they belong to
 template <class U>
 __global__ __launch_bounds__(256) void gemm_columns_from_rows_kernel(const U* t, U* c, uint32_t M, uint32_t N, int64_t c_rs, uint32_t total) {
@@ -401,6 +468,24 @@ int gemm_entry(const tannic_tensor_t* a, const tannic_tensor_t* b, tannic_tensor
                         }
                         scratch_release(turned, s);
                         if (status != TANNIC_UNSUPPORTED_DTYPE) return;   // (refused after all: on with the product as it is)
+                    }
+                }
+                constexpr bool shares_k = std::is_same_v<A, B> && (is_16bit<A>::value || std::is_same_v<A, float> || std::is_same_v<A, int8_t>);
+                if (few_results_under_a_long_k(p, shares_k ? 8192 : 32768)) {
+                    // (not where the tiles share K or W is streamed: aligned K-contiguous operands of the 16-bit types and
+                    // fp32, of int8 up to 32 rows; nor the few rows that the row-major kernel below or the scalar kernel
+                    // for few rows streams)
+                    bool elsewhere = !shares_k && p.M <= 16 && p.a_cs == 1 && p.b_rs == 1;
+                    if constexpr (shares_k) {
+                        constexpr int64_t unit = 16 / sizeof(A);
+                        const bool aligned_nt = p.a_cs == 1 && p.b_rs == 1 && p.K % (std::is_same_v<A, int8_t> ? 128 : unit) == 0 && p.a_rs % unit == 0 && p.b_cs % unit == 0 &&
+                                                reinterpret_cast<uintptr_t>(first) % 16 == 0 && reinterpret_cast<uintptr_t>(second) % 16 == 0;
+                        if (aligned_nt && (!std::is_same_v<A, int8_t> || p.M <= 32)) elsewhere = true;
+                        if (!std::is_same_v<A, int8_t> && p.M <= 8 && p.b_cs == 1 && p.b_rs != 1 && p.N >= 256 && p.N % 4 == 0) elsewhere = true;   // gemm_rows_nn
+                    }
+                    if (!elsewhere) {
+                        status = run_few_results<A, B, D>(p, first, second, dst->address, s);
+                        return;
                     }
                 }
                 if constexpr (std::is_same_v<A, B> && (is_16bit<A>::value || std::is_same_v<A, float>)) {

@@ -107,6 +107,12 @@ LAYOUTS = {
     "rows_nn_8_rows_x_transposed": ((700, 8), (700, 1024), [("transpose", (-1, -2))], []),
     "rows_nn_3_rows_slice_of_w": ((3, 512), (512, 1100), [], [("index", (slice(None), slice(4, 1028)))]),
     "rows_nn_2_rows_long_k": ((2, 20000), (20000, 256), [], []),
+    # few results under a long K (a workgroup per 4 x 4 results, its lanes striding over K): every layout, odd extents, batches
+    "few_results_nt": ((48, 2047), (13, 2047), [], [("transpose", (-1, -2))]),
+    "few_results_nn": ((20, 1500), (1500, 9), [], []),
+    "few_results_tn": ((3000, 6), (3000, 8), [("transpose", (-1, -2))], []),
+    "few_results_tt": ((1024, 33), (50, 1024), [("transpose", (-1, -2))], [("transpose", (-1, -2))]),
+    "few_results_batched": ((5, 6, 1100), (5, 1100, 10), [], []),
     "rank4_rank2_nt_large": ((2, 3, 200, 320), (480, 320), [], [("transpose", (-1, -2))]),
     "stream_49_rows_long_k_wide": ((49, 2048), (400, 2048), [], [("transpose", (-1, -2))]),
 }
@@ -148,7 +154,7 @@ def test_16bit_gemm_fp32_accumulate(device, dtype, layout):
 
 @pytest.mark.parametrize("layout", ["nn", "nt_mid", "tn_mid", "batched", "batch_broadcast", "rank4_rank2_nt",
                                     "single_row", "sixteen_rows", "stream_16_rows_ragged_columns", "stream_batched_views", "matrix_vector",
-                                    "matrix_vector_batched"])
+                                    "matrix_vector_batched", "few_results_nt", "few_results_nn", "few_results_tt", "few_results_batched"])
 @pytest.mark.parametrize("pair", [(ta.int8, ta.int8), (ta.int16, ta.int32), (ta.int32, ta.int32), (ta.int64, ta.int8)], ids=lambda p: f"{p[0]}-{p[1]}")
 def test_integer_gemm_bit_exact(device, pair, layout):
     host, dev, _ = operands(pair, layout, device, -100, 100)
@@ -180,6 +186,24 @@ def test_int8_gemm_on_matrix_cores_is_bit_exact(device, shape):
     support.assert_bit_exact(got.storage(), want, f"int8 gemm {sa} x {sb}^T against numpy")
     if int(np.prod(sa)) * sb[-2] < 40_000_000:
         support.assert_bit_exact(got.storage(), ops.matmul(ha, hb.transpose()).storage(), f"int8 gemm {sa} x {sb}^T against the checker")
+
+
+@pytest.mark.parametrize("shape", [((6, 64, 300), (6, 337, 300), "nt"), ((5, 70, 260), (5, 260, 129), "nn"), ((4, 200, 64), (4, 49, 200), "tt"),
+                                   ((3, 40, 384), (1, 384, 72), "nn"), ((1, 33, 130), (7, 90, 130), "nt")], ids=lambda s: s[2] + "-" + "x".join(map(str, s[0])))
+def test_int8_batches_in_other_layouts_are_bit_exact(device, shape):
+    """A batch of int8 products along one dim whose operands are not K-contiguous, or whose K no 128 divides: every
+    product's operands are copied into K-contiguous zero-padded rows (an operand all products share, once) and the batch
+    runs on the matrix cores; bit for bit equal to numpy's int64 product."""
+    sa, sb, layout = shape
+    a = support.integers(SEED, 41, sa, -128, 128).astype(np.int8)
+    b = support.integers(SEED, 42, sb, -128, 128).astype(np.int8)
+    (ha, da), (hb, db) = support.both(a, ta.int8, device), support.both(b, ta.int8, device)
+    va, vb = (da.transpose() if layout[0] == "t" else da), (db.transpose() if layout[1] == "t" else db)
+    na, nb = (np.swapaxes(a, -1, -2) if layout[0] == "t" else a), (np.swapaxes(b, -1, -2) if layout[1] == "t" else b)
+    got = ops.matmul(va, vb)
+    want = np.matmul(na.astype(np.int64), nb.astype(np.int64)).astype(np.int32)
+    assert got.dtype is ta.int32 and got.shape == want.shape
+    support.assert_bit_exact(got.storage(), want, f"int8 batch {sa} x {sb} {layout}")
 
 
 @pytest.mark.parametrize("layout", ["nn", "tn", "tt"])
