@@ -64,10 +64,14 @@ static int run_unfold_batch(const ConvProblem& p, int dtype, const void* x, cons
     const bool few = pixels <= 100 ? K >= 512
                                    : (K >= 768 && (batch_pixels <= 2048 || (p.HO == 1 && batch_pixels <= 8192))) || (K >= 2304 && batch_pixels <= 4096) ||
                                          (K >= 4608 && batch_pixels <= 8192 && p.stride_h > 1 && p.stride_w > 1);
-    // (float64: the alternative is the scalar kernel, which sixteen output channels sharing an unfolded column already beat;
-    // its product reads single doubles and asks nothing of K or of where the weights lie)
+    // (float64: the alternative is the scalar kernel, one thread per result walking K alone.  Six output channels sharing an
+    // unfolded column already beat it at full occupancy, and with few results in all it is bound by that walk: 4 images
+    // 349 -> 8 channels 7x7 over 8 x 8, 32 results under a K of 17101, 2202 us.  The float64 product reads single doubles
+    // and asks nothing of K or of where the weights lie.)
+    // (A K that no 16 bytes divide leaves the rows of the weights misaligned: the product then runs on the tiles for
+    // operands at any address.)
     constexpr bool f64 = std::is_same_v<T, double>;
-    if (f64 ? (K < 16 || p.O < 16) : ((ANY_SIZE ? K < 320 : !few) || K % E != 0)) return TANNIC_UNSUPPORTED_DTYPE;
+    if (f64 ? (p.O < 6 && batch_pixels * p.O >= 65536) : (ANY_SIZE ? K < 320 : !few)) return TANNIC_UNSUPPORTED_DTYPE;
     if (K >= (1u << 24) || pixels >= (1u << 24)) return TANNIC_UNSUPPORTED_DTYPE;
     const uint32_t pitch = static_cast<uint32_t>((pixels + E - 1) / E * E);
     if (static_cast<uint64_t>(p.N) * pitch < (ANY_SIZE ? 16 : 256)) return TANNIC_UNSUPPORTED_DTYPE;
@@ -125,8 +129,9 @@ static int run_unfold_batch(const ConvProblem& p, int dtype, const void* x, cons
         if constexpr (f64) status = gemm_mfma_f64(g, static_cast<const double*>(w), reinterpret_cast<const double*>(col), static_cast<double*>(y_part), stream);
         else if constexpr (std::is_same_v<T, float>) status = gemm_mfma_f32(g, static_cast<const float*>(w), reinterpret_cast<const float*>(col), static_cast<float*>(y_part), stream);
         else status = gemm_mfma_16bit(g, dtype, w, col, y_part, stream);
-        if (status == TANNIC_UNSUPPORTED_DTYPE) {
-            set_error_text("conv2d: internal: the unfolded product refused a problem its caller had checked");
+        if (status == TANNIC_UNSUPPORTED_DTYPE && n0 != 0) {
+            // (the first run of images decides: a refusal there leaves the convolution to the next kernel, nothing stored yet)
+            set_error_text("conv2d: internal: the unfolded product refused a run of images after it had taken the first");
             status = TANNIC_ERROR;
         }
     }

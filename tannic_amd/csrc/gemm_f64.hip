@@ -178,8 +178,12 @@ static int launch_f64(const GemmProblem& p, const double* a, const double* b, do
 int gemm_mfma_f64(const GemmProblem& p, const double* a, const double* b, double* c, hipStream_t stream) {
     if (p.b_group_stride || (p.c_group && p.batches != 1)) return TANNIC_UNSUPPORTED_DTYPE;
     // (fewer than 17 rows under a long K stream through the kernels for few rows: they are bound by memory)
-    if (p.M < 8 || p.N < 8 || p.K < 16 || p.batches == 0 || p.batches > 65535) return TANNIC_UNSUPPORTED_DTYPE;
-    if (p.M <= 16 && p.a_cs == 1 && p.b_rs == 1 && p.K >= 256) return TANNIC_UNSUPPORTED_DTYPE;
+    if (p.M == 0 || p.N == 0 || p.K == 0 || p.batches == 0 || p.batches > 65535) return TANNIC_UNSUPPORTED_DTYPE;
+    // (a product with grouped columns is a convolution's: no other kernel stores those, and it is taken whatever its extents)
+    if (!p.c_group) {
+        if (p.M < 8 || p.N < 8 || p.K < 16) return TANNIC_UNSUPPORTED_DTYPE;
+        if (p.M <= 16 && p.a_cs == 1 && p.b_rs == 1 && p.K >= 256) return TANNIC_UNSUPPORTED_DTYPE;
+    }
     // The matrix pipe bounds every shape of workgroup alike: what a choice costs is the rounds of 256 workgroups it
     // takes times the area of one.  Equal costs go to the larger tile, and a wavefront of 4 x 4 tiles loads half as much
     // per MFMA as one of 2 x 2 (the loads, not the matrix pipe, are what these kernels wait for).

@@ -115,6 +115,11 @@ CASES = {
     "unfolded_few_pixels_in_batch": ((2, 96, 14, 14), (24, 96, 3, 3), (1, 1), (1, 1)),
     "unfolded_one_row_high": ((4, 128, 1, 200), (40, 128, 1, 7), (1, 2), (0, 3)),
     "unfolded_any_one_image_long_k": ((1, 160, 12, 12), (8, 160, 7, 7), (1, 1), (3, 3)),
+    # ... a K that no 16 bytes divide (the rows of the weights start anywhere: the product's tiles for misaligned operands),
+    # and few output channels over few results (float64: the unfolded product instead of one thread per result)
+    "unfolded_odd_k_few_pixels": ((3, 116, 8, 8), (40, 116, 5, 5), (2, 2), (2, 2)),
+    "unfolded_any_odd_k": ((4, 77, 20, 20), (24, 77, 3, 3), (1, 1), (1, 1)),
+    "unfolded_three_channels_out_long_k": ((4, 50, 8, 8), (3, 50, 7, 7), (2, 2), (0, 0)),
     # ... in runs of images when the whole batch unfolded would be large (13 images and 1; one image at a time), with a
     # K beyond what the general tiles keep a table of
     "unfolded_any_runs_of_images": ((14, 128, 40, 40), (4, 128, 7, 7), (1, 1), (3, 3)),
