@@ -526,7 +526,50 @@ int run_reduce(const tannic_tensor_t* src, tannic_tensor_t* dst, hipStream_t str
         set_error_text("reduce: reduced axis of 2^32 elements or more is not supported");
         return TANNIC_ERROR;
     }
-    if (src->layout != TANNIC_CONTIGUOUS) {
+    // A view that is a dense tensor with its dims in another order (a transposed matrix) is still [outer, R, inner] in
+    // memory when the dims that stay keep their order among themselves: the results then come out in the order the
+    // destination holds them.  (Summing a transposed [3589, 2141] along its rows is the column sum of the matrix as it lies.)
+    size_t outer = 1, inner = 1;
+    bool as_slab = src->layout == TANNIC_CONTIGUOUS;
+    if (as_slab) {
+        for (int d = 0; d < src->rank; ++d) {
+            if (d < axis) outer *= src->shape.sizes[d];
+            else if (d > axis) inner *= src->shape.sizes[d];
+        }
+    } else {
+        int order[TANNIC_DIMENSIONS];
+        int count = 0;
+        for (int d = 0; d < src->rank; ++d)
+            if (src->shape.sizes[d] != 1 || d == axis) order[count++] = d;
+        for (int i = 1; i < count; ++i)
+            for (int j = i; j > 0 && src->strides.sizes[order[j]] > src->strides.sizes[order[j - 1]]; --j) {
+                const int t = order[j];
+                order[j] = order[j - 1];
+                order[j - 1] = t;
+            }
+        bool dense = true, in_order = true;
+        int64_t expect = 1;
+        int last_kept = -1;
+        for (int i = count - 1; i >= 0; --i) {
+            if (src->shape.sizes[order[i]] != 1 && src->strides.sizes[order[i]] != expect) dense = false;
+            expect *= static_cast<int64_t>(src->shape.sizes[order[i]]);
+        }
+        for (int i = 0; i < count; ++i) {
+            if (order[i] == axis) continue;
+            if (order[i] < last_kept) in_order = false;
+            last_kept = order[i];
+        }
+        if (dense && in_order && R > 0) {
+            bool before = true;
+            for (int i = 0; i < count; ++i) {
+                if (order[i] == axis) before = false;
+                else if (before) outer *= src->shape.sizes[order[i]];
+                else inner *= src->shape.sizes[order[i]];
+            }
+            as_slab = true;
+        }
+    }
+    if (!as_slab) {
         StridedWalk w{};
         w.rank = src->rank;
         w.axis = axis;
@@ -543,11 +586,6 @@ int run_reduce(const tannic_tensor_t* src, tannic_tensor_t* dst, hipStream_t str
                            static_cast<uint32_t>(slots));
         return launch_status("reduce_strided_kernel");
     }
-    size_t outer = 1, inner = 1;
-    for (int d = 0; d < src->rank; ++d) {
-        if (d < axis) outer *= src->shape.sizes[d];
-        else if (d > axis) inner *= src->shape.sizes[d];
-    }
     const size_t slots = outer * inner;
     if (slots == 0) return TANNIC_SUCCESS;
     if (slots >= (1ull << 31) || outer >= (1ull << 31)) { set_error_text("reduce: too many outputs"); return TANNIC_ERROR; }
@@ -555,6 +593,15 @@ int run_reduce(const tannic_tensor_t* src, tannic_tensor_t* dst, hipStream_t str
     constexpr int VEC = sizeof(T) >= 16 ? 1 : static_cast<int>(16 / sizeof(T));
     const bool aligned = reinterpret_cast<uintptr_t>(ps) % 16 == 0;
 
+    if (inner == 1 && R <= 16) {
+        // rows of a few elements (of one, when the reduced dim has extent 1): a lane per row instead of a wavefront
+        StridedWalk w{};
+        w.rank = 2; w.axis = 1;
+        w.extent[0] = static_cast<uint32_t>(outer); w.extent[1] = static_cast<uint32_t>(R);
+        w.stride[0] = static_cast<int64_t>(R); w.stride[1] = 1;
+        hipLaunchKernelGGL((reduce_strided_kernel<Op>), dim3((slots + kThreads - 1) / kThreads), dim3(kThreads), 0, stream, ps, pd, w, static_cast<uint32_t>(slots));
+        return launch_status("reduce_strided_kernel");
+    }
     if (inner == 1) {
         const uint32_t rows = static_cast<uint32_t>(outer);
         const bool vec = VEC > 1 && aligned && R % VEC == 0;

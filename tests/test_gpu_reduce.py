@@ -201,6 +201,24 @@ def test_strided_sources(device, dtype):
                 support.assert_bit_exact(got.storage(), want.storage(), f"{op} {dtype} {spec} axis={axis}")  # integer-valued: sums exact
 
 
+@pytest.mark.parametrize("dtype", [ta.float32, ta.int32, ta.float16, ta.float64], ids=str)
+def test_views_that_are_dense_in_another_order_and_rows_of_a_few_elements(device, dtype):
+    """A transposed matrix summed along its rows is the column sum of the matrix as it lies: views whose dims are a
+    dense tensor's in another order reduce as [outer, R, inner] when the dims that stay keep their order (and element by
+    element otherwise); rows of up to 16 elements, of one when the reduced dim has extent 1, take a lane each."""
+    cases = [((700, 300), [("transpose", (0, 1))]), ((40, 300, 64), [("transpose", (1, 2))]), ((40, 64, 300), [("transpose", (0, 1))]),
+             ((12, 64, 300), [("permute", (2, 0, 1))]), ((9, 1, 300, 70), [("transpose", (2, 3))]), ((5000, 1), []), ((4000, 7), []), ((30, 40, 1), []),
+             ((3000, 16), []), ((1, 900), [("transpose", (0, 1))])]
+    for shape, spec in cases:
+        h, d = support.both(np.round(support.values_for(dtype, SEED, 9, shape, -3, 3).astype(np.float64)), dtype, device)
+        hv, dv = support.apply_view(h, spec), support.apply_view(d, spec)
+        for axis in range(len(shape)):
+            for op in ("sum", "argmax", "max"):
+                want, got = getattr(ops, op)(hv, axis), getattr(ops, op)(dv, axis)
+                assert got.shape == want.shape
+                support.assert_bit_exact(got.storage(), want.storage(), f"{op} {dtype} {shape} {spec} axis={axis}")  # integer-valued: sums exact
+
+
 def test_rms_norm_statistics(device):
     """mean(X*X, -1, keepdim) then rsqrt: the reduction pattern of an RMSNorm row (R = 4096)."""
     h, d = support.both(support.values_for(ta.bfloat16, SEED, 7, (1, 64, 4096)), ta.bfloat16, device)
