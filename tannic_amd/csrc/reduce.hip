@@ -509,6 +509,30 @@ __global__ __launch_bounds__(kThreads) void reduce_strided_kernel(const typename
     else dst[slot] = Op::finish(acc, R);
 }
 
+// Few results over a long reduced dim (a lane per result would walk it alone): a wavefront per result, its lanes
+// striding over R in increasing order, combined like the lanes of a row.
+template <class Op>
+__global__ __launch_bounds__(kThreads) void reduce_strided_wave_kernel(const typename Op::S* src, typename Op::Out* dst, StridedWalk w, uint32_t slots) {
+    const uint32_t slot = blockIdx.x * (kThreads / kWave) + threadIdx.x / kWave, lane = threadIdx.x % kWave;
+    if (slot >= slots) return;   // whole wavefronts; nothing below synchronises across them
+    uint32_t rem = slot;
+    int64_t base = 0;
+    for (int d = w.rank - 1; d >= 0; --d) {
+        if (d == w.axis) continue;
+        base += static_cast<int64_t>(rem % w.extent[d]) * w.stride[d];
+        rem /= w.extent[d];
+    }
+    const uint32_t R = w.extent[w.axis];
+    const int64_t step = w.stride[w.axis];
+    typename Op::A acc = Op::init();
+    for (uint32_t r = lane; r < R; r += kWave) acc = Op::step(acc, src[base + static_cast<int64_t>(r) * step], r);
+    acc = wave_reduce<Op>(acc);
+    if (lane != 0) return;
+    if constexpr (is_value_only<Op>::value) dst[slot] = (R != 0 && same(acc, Op::init())) ? src[base] : acc;
+    else if constexpr (Op::needs_source) dst[slot] = src[base + static_cast<int64_t>(acc.index) * step];
+    else dst[slot] = Op::finish(acc, R);
+}
+
 // ---- host side -------------------------------------------------------------------
 template <class Op>
 int run_reduce(const tannic_tensor_t* src, tannic_tensor_t* dst, hipStream_t stream, uint8_t axis) {
@@ -582,6 +606,12 @@ int run_reduce(const tannic_tensor_t* src, tannic_tensor_t* dst, hipStream_t str
         if (slots == 0) return TANNIC_SUCCESS;
         if (slots >= (1ull << 31)) { set_error_text("reduce: too many outputs"); return TANNIC_ERROR; }
         if (element_count(dst) != slots) { set_error_text("reduce: the destination does not hold one element per reduced slice"); return TANNIC_ERROR; }
+        if (R >= 256 && slots <= 65536) {
+            constexpr uint32_t per_block = kThreads / kWave;
+            hipLaunchKernelGGL((reduce_strided_wave_kernel<Op>), dim3((static_cast<uint32_t>(slots) + per_block - 1) / per_block), dim3(kThreads), 0, stream, ps, pd, w,
+                               static_cast<uint32_t>(slots));
+            return launch_status("reduce_strided_wave_kernel");
+        }
         hipLaunchKernelGGL((reduce_strided_kernel<Op>), dim3((slots + kThreads - 1) / kThreads), dim3(kThreads), 0, stream, ps, pd, w,
                            static_cast<uint32_t>(slots));
         return launch_status("reduce_strided_kernel");

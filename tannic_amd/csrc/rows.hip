@@ -200,6 +200,38 @@ __global__ __launch_bounds__(kRowBlock) void softmax_wave_kernel(const T* x, con
         if (lane + 64 * e < L) y[base + lane + 64 * e] = narrow<T>(s[e] * inv);
 }
 
+// Many rows of at most 16 elements (of one: the softmax over a dim of extent 1): a lane per row, the row in its registers.
+template <class T, bool MASK>
+__global__ __launch_bounds__(kRowBlock) void softmax_lane_kernel(const T* x, const T* mask, T* y, uint32_t rows, uint32_t L, FastDiv q, float scale) {
+    using A = RowAcc<T>;
+    const uint32_t row = blockIdx.x * kRowBlock + threadIdx.x;
+    if (row >= rows) return;
+    const size_t base = static_cast<size_t>(row) * L;
+    uint32_t mrow = 0, quotient = 0;
+    if (MASK) q.divmod(row, quotient, mrow);
+    A s[16];
+    A top = -INFINITY;
+#pragma unroll
+    for (uint32_t i = 0; i < 16; ++i) {
+        s[i] = -INFINITY;
+        if (i < L) {
+            s[i] = static_cast<A>(widen(x[base + i])) * static_cast<A>(scale);
+            if (MASK) s[i] += static_cast<A>(widen(mask[static_cast<size_t>(mrow) * L + i]));
+        }
+        top = MaxOp::combine(top, s[i]);
+    }
+    A sum = 0;
+#pragma unroll
+    for (uint32_t i = 0; i < 16; ++i) {
+        s[i] = i < L ? fast_exp(s[i] - top, is_16bit<T>::value) : A(0);
+        sum += s[i];
+    }
+    const A inv = A(1) / sum;
+#pragma unroll
+    for (uint32_t i = 0; i < 16; ++i)
+        if (i < L) y[base + i] = narrow<T>(s[i] * inv);
+}
+
 // any length, any alignment: one block per row, the row read three times (from cache after the first), four elements of a
 // thread on their way at a time
 template <class T, bool MASK>
@@ -504,6 +536,12 @@ int run_softmax(const tannic_tensor_t* x, const tannic_tensor_t* mask, tannic_te
         }
         scratch_release(partial, stream);
         return status;
+    }
+    if (L <= 16 && rows >= 4096) {
+        const dim3 grid((rows + kRowBlock - 1) / kRowBlock);
+        if (pm) hipLaunchKernelGGL((softmax_lane_kernel<T, true>), grid, dim3(kRowBlock), 0, stream, px, pm, py, rows, L, FastDiv(Q), scale);
+        else hipLaunchKernelGGL((softmax_lane_kernel<T, false>), grid, dim3(kRowBlock), 0, stream, px, pm, py, rows, L, FastDiv(1), scale);
+        return launch_status("softmax_lane_kernel");
     }
     if (L <= 64 * 32 && rows >= 256) {
         // short rows that the vector kernel cannot take: a wavefront per row

@@ -230,7 +230,9 @@ def causal(n, dtype):
 SOFTMAX_SHAPES = [(4, 64), (3, 40, 512), (2, 4, 128, 128), (1300, 200), (5, 4096), (3, 37), (2, 1028), (2, 70000),
                   (300, 197), (2, 130, 511), (260, 1025), (257, 2047), (100, 197),
                   # a handful of very long rows shared by several blocks: odd and even lengths, one and many rows
-                  (1, 50257), (16, 50257), (3, 32768), (64, 16385)]
+                  (1, 50257), (16, 50257), (3, 32768), (64, 16385),
+                  # thousands of rows of at most 16 elements (of one element): a lane per row
+                  (5000, 1), (4100, 7), (70, 60, 16), (4200, 13)]
 
 
 @pytest.mark.parametrize("shape", SOFTMAX_SHAPES, ids=str)
@@ -259,6 +261,17 @@ def test_softmax_causal_mask(device, dtype, n):
     upper = np.triu(np.ones((n, n), dtype=bool), 1)
     assert (got[..., upper] == 0.0).all()                      # masked entries are exactly zero
     np.testing.assert_array_equal(got[..., 0, 0], 1.0)         # the first row attends to one entry
+
+
+@pytest.mark.parametrize("dtype", [ta.float16, ta.float32], ids=str)
+def test_softmax_causal_mask_over_many_short_rows(device, dtype):
+    """300 heads of 16 x 16 scores under a causal mask: rows of 16 elements, a lane each."""
+    x = values(dtype, 20, (300, 16, 16), -8.0, 8.0)
+    m = causal(16, dtype)
+    got = f64(ops.softmax(ta.tensor(x, dtype, device), ta.tensor(m, dtype, device), 0.5))
+    want = softmax_definition(x, m, 0.5)
+    check(got, want, dtype, f"softmax causal short rows {dtype}", {ta.float16: 1.5, ta.float32: 16.0}[dtype])
+    assert (got[..., np.triu(np.ones((16, 16), dtype=bool), 1)] == 0.0).all()
 
 
 def test_softmax_shift_invariance(device):

@@ -205,10 +205,14 @@ def test_strided_sources(device, dtype):
 def test_views_that_are_dense_in_another_order_and_rows_of_a_few_elements(device, dtype):
     """A transposed matrix summed along its rows is the column sum of the matrix as it lies: views whose dims are a
     dense tensor's in another order reduce as [outer, R, inner] when the dims that stay keep their order (and element by
-    element otherwise); rows of up to 16 elements, of one when the reduced dim has extent 1, take a lane each."""
+    element otherwise: a lane per result, or a wavefront when the results are few and the reduced dim long); rows of up
+    to 16 elements, of one when the reduced dim has extent 1, take a lane each."""
     cases = [((700, 300), [("transpose", (0, 1))]), ((40, 300, 64), [("transpose", (1, 2))]), ((40, 64, 300), [("transpose", (0, 1))]),
              ((12, 64, 300), [("permute", (2, 0, 1))]), ((9, 1, 300, 70), [("transpose", (2, 3))]), ((5000, 1), []), ((4000, 7), []), ((30, 40, 1), []),
-             ((3000, 16), []), ((1, 900), [("transpose", (0, 1))])]
+             ((3000, 16), []), ((1, 900), [("transpose", (0, 1))]),
+             # views that are not dense: few results over a long reduced dim take a wavefront each
+             ((40, 600, 6), [("index", (slice(0, 40, 2),))]), ((50, 2000), [("index", (slice(None), slice(1, 1999)))]),
+             ((6, 3, 1000), [("index", (slice(None), slice(None), slice(0, 1000, 3)))])]
     for shape, spec in cases:
         h, d = support.both(np.round(support.values_for(dtype, SEED, 9, shape, -3, 3).astype(np.float64)), dtype, device)
         hv, dv = support.apply_view(h, spec), support.apply_view(d, spec)
