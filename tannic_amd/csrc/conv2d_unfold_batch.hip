@@ -43,6 +43,21 @@ __global__ __launch_bounds__(256) void conv_unfold_batch_kernel(const T* x, T* c
     *reinterpret_cast<uint4*>(col + static_cast<size_t>(row) * pitch + group * E) = bits;
 }
 
+// dst[o][k] = k < K ? src[o][k] : 0 for rows of K and of Kp elements
+template <class T>
+__global__ __launch_bounds__(256) void conv_pad_rows_kernel(const T* src, T* dst, uint32_t K, uint32_t Kp, uint32_t total) {
+    const uint32_t idx = blockIdx.x * 256 + threadIdx.x;
+    if (idx >= total) return;
+    const uint32_t o = idx / Kp, k = idx % Kp;
+    dst[idx] = k < K ? src[static_cast<size_t>(o) * K + k] : T{};
+}
+
+template <class T>
+__global__ __launch_bounds__(256) void conv_zero_kernel(T* dst, uint32_t total) {
+    const uint32_t idx = blockIdx.x * 256 + threadIdx.x;
+    if (idx < total) dst[idx] = T{};
+}
+
 // ANY_SIZE: as the last kernel before the general ones, for whatever the specialised kernels have refused, as long as
 // the unfolded operand stays small enough to be worth writing out.
 template <class T, bool ANY_SIZE>
@@ -68,13 +83,13 @@ static int run_unfold_batch(const ConvProblem& p, int dtype, const void* x, cons
     // unfolded column already beat it at full occupancy, and with few results in all it is bound by that walk: 4 images
     // 349 -> 8 channels 7x7 over 8 x 8, 32 results under a K of 17101, 2202 us.  The float64 product reads single doubles
     // and asks nothing of K or of where the weights lie.)
-    // (A K that no 16 bytes divide leaves the rows of the weights misaligned: the product then runs on the tiles for
-    // operands at any address.)
     constexpr bool f64 = std::is_same_v<T, double>;
     if (f64 ? (p.O < 6 && batch_pixels * p.O >= 65536) : (ANY_SIZE ? K < 320 : !few)) return TANNIC_UNSUPPORTED_DTYPE;
     if (K >= (1u << 24) || pixels >= (1u << 24)) return TANNIC_UNSUPPORTED_DTYPE;
     const uint32_t pitch = static_cast<uint32_t>((pixels + E - 1) / E * E);
-    if (static_cast<uint64_t>(p.N) * pitch < (ANY_SIZE ? 16 : 256)) return TANNIC_UNSUPPORTED_DTYPE;
+    // (fewer columns than two tiles are wide stay with the patch kernels, unless the results are so few that the product
+    // runs a workgroup per 4 x 4 of them: one image 672 -> 8 4x4 over 8 x 8, 200 results under a K of 10752, 197 us on patches)
+    if (!ANY_SIZE && static_cast<uint64_t>(p.N) * pitch < 256 && static_cast<uint64_t>(p.O) * p.N * pitch > 8192) return TANNIC_UNSUPPORTED_DTYPE;
     // The unfolded operand is kept small: ANY_SIZE takes the images in runs whose unfolded operand stays within the
     // limit (one image's may reach four times that), one product per run, all through the same buffer.
     const uint64_t limit = (ANY_SIZE ? 256ull : 512ull) << 20, image_bytes = K * pitch * sizeof(T);
@@ -88,11 +103,30 @@ static int run_unfold_batch(const ConvProblem& p, int dtype, const void* x, cons
     if (columns >= (1ull << 31) || K * run * (pitch / E) >= (1ull << 31)) return TANNIC_UNSUPPORTED_DTYPE;
     // the kernel tensor as a K-contiguous O x K matrix, the result as pixel-contiguous rows
     if (p.ws[3] != 1 || p.ws[2] != static_cast<int64_t>(p.KW) || p.ws[1] != static_cast<int64_t>(p.KH) * p.KW || p.ws[0] != static_cast<int64_t>(K) ||
-        (!f64 && reinterpret_cast<uintptr_t>(w) % 16 != 0))
+        (!f64 && K % E == 0 && reinterpret_cast<uintptr_t>(w) % 16 != 0))
         return TANNIC_UNSUPPORTED_DTYPE;
     if (p.ys[3] != 1 || p.ys[2] != static_cast<int64_t>(p.WO)) return TANNIC_UNSUPPORTED_DTYPE;
+    // A K that no 16 bytes divide would leave the rows of the weights misaligned and the product on the tiles for operands
+    // at any address, which do not share K: the weights are copied into rows of Kp elements, zeros at their ends, and the
+    // unfolded operand gets Kp - K rows of zeros (fp32 405 -> 32 7x7 s3 over 126 x 126, K = 19845: 1523 us on those tiles).
+    const uint32_t Kp = f64 ? static_cast<uint32_t>(K) : static_cast<uint32_t>((K + E - 1) / E * E);
+    if (static_cast<uint64_t>(p.O) * Kp >= (1ull << 31) || static_cast<uint64_t>(Kp - K) * columns >= (1ull << 31)) return TANNIC_UNSUPPORTED_DTYPE;
+    T* padded = nullptr;
+    if (Kp != K) {
+        if (scratch_acquire(reinterpret_cast<void**>(&padded), static_cast<size_t>(p.O) * Kp * sizeof(T), stream) != TANNIC_SUCCESS) return TANNIC_ERROR;
+        const uint32_t total = p.O * Kp;
+        hipLaunchKernelGGL((conv_pad_rows_kernel<T>), dim3((total + 255) / 256), dim3(256), 0, stream, static_cast<const T*>(w), padded, static_cast<uint32_t>(K), Kp, total);
+        if (launch_status("conv_pad_rows_kernel") != TANNIC_SUCCESS) {
+            scratch_release(padded, stream);
+            return TANNIC_ERROR;
+        }
+    }
+    const void* weights = padded ? static_cast<const void*>(padded) : w;
     T* col = nullptr;
-    if (scratch_acquire(reinterpret_cast<void**>(&col), static_cast<size_t>(K) * columns * sizeof(T), stream) != TANNIC_SUCCESS) return TANNIC_ERROR;
+    if (scratch_acquire(reinterpret_cast<void**>(&col), static_cast<size_t>(Kp) * columns * sizeof(T), stream) != TANNIC_SUCCESS) {
+        if (padded) scratch_release(padded, stream);
+        return TANNIC_ERROR;
+    }
     int status = TANNIC_SUCCESS;
     for (uint32_t n0 = 0; n0 < p.N && status == TANNIC_SUCCESS; n0 += run) {
         ConvProblem part = p;
@@ -105,11 +139,17 @@ static int run_unfold_batch(const ConvProblem& p, int dtype, const void* x, cons
                            FastDiv(groups), FastDiv(part.N), FastDiv(p.WO), FastDiv(p.KH * p.KW), FastDiv(p.KW), total);
         status = launch_status("conv_unfold_batch_kernel");
         if (status != TANNIC_SUCCESS) break;
+        if (Kp != K) {
+            const uint32_t tail = static_cast<uint32_t>((Kp - K) * part_columns);
+            hipLaunchKernelGGL((conv_zero_kernel<T>), dim3((tail + 255) / 256), dim3(256), 0, stream, col + static_cast<size_t>(K) * part_columns, tail);
+            status = launch_status("conv_zero_kernel");
+            if (status != TANNIC_SUCCESS) break;
+        }
         GemmProblem g{};
         g.M = p.O;
         g.N = static_cast<uint32_t>(part_columns);
-        g.K = static_cast<uint32_t>(K);
-        g.a_rs = p.ws[0];
+        g.K = Kp;
+        g.a_rs = padded ? static_cast<int64_t>(Kp) : p.ws[0];
         g.a_cs = 1;
         g.b_rs = static_cast<int64_t>(part_columns);
         g.b_cs = 1;
@@ -126,9 +166,12 @@ static int run_unfold_batch(const ConvProblem& p, int dtype, const void* x, cons
             g.a_bs[d] = g.b_bs[d] = g.c_bs[d] = 0;
         }
         g.row_bias = bias;
-        if constexpr (f64) status = gemm_mfma_f64(g, static_cast<const double*>(w), reinterpret_cast<const double*>(col), static_cast<double*>(y_part), stream);
-        else if constexpr (std::is_same_v<T, float>) status = gemm_mfma_f32(g, static_cast<const float*>(w), reinterpret_cast<const float*>(col), static_cast<float*>(y_part), stream);
-        else status = gemm_mfma_16bit(g, dtype, w, col, y_part, stream);
+        // few results under a long K (a handful of pixels in all): a workgroup per 4 x 4 of them instead of one tile walking K
+        status = gemm_few_results(g, dtype, weights, col, y_part, stream);
+        if (status != TANNIC_UNSUPPORTED_DTYPE) continue;
+        if constexpr (f64) status = gemm_mfma_f64(g, static_cast<const double*>(weights), reinterpret_cast<const double*>(col), static_cast<double*>(y_part), stream);
+        else if constexpr (std::is_same_v<T, float>) status = gemm_mfma_f32(g, static_cast<const float*>(weights), reinterpret_cast<const float*>(col), static_cast<float*>(y_part), stream);
+        else status = gemm_mfma_16bit(g, dtype, weights, col, y_part, stream);
         if (status == TANNIC_UNSUPPORTED_DTYPE && n0 != 0) {
             // (the first run of images decides: a refusal there leaves the convolution to the next kernel, nothing stored yet)
             set_error_text("conv2d: internal: the unfolded product refused a run of images after it had taken the first");
@@ -136,6 +179,7 @@ static int run_unfold_batch(const ConvProblem& p, int dtype, const void* x, cons
         }
     }
     scratch_release(col, stream);
+    if (padded) scratch_release(padded, stream);
     return status;
 }
 
@@ -162,6 +206,8 @@ int conv2d_unfold_batch_any(const ConvProblem& p, int dtype, const void* x, cons
     if (p.KH == 1 && p.KW == 1) return TANNIC_UNSUPPORTED_DTYPE;
     if (dtype == TANNIC_FLOAT16) return run_unfold_batch<f16, true>(p, dtype, x, w, bias, y, stream);
     if (dtype == TANNIC_BFLOAT16) return run_unfold_batch<bf16, true>(p, dtype, x, w, bias, y, stream);
+    // (fp32 comes here after its gathering tiles and its own unfolding have refused: a K beyond the tiles' table)
+    if (dtype == TANNIC_FLOAT32) return run_unfold_batch<float, true>(p, dtype, x, w, bias, y, stream);
     return TANNIC_UNSUPPORTED_DTYPE;
 }
 

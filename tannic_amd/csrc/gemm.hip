@@ -262,8 +262,18 @@ __global__ __launch_bounds__(256) void gemm_generic_few_results_kernel(const A* 
     __syncthreads();
     if (threadIdx.x < 16) {
         const uint32_t m = m0 + threadIdx.x / 4, n = n0 + threadIdx.x % 4;
-        const Acc v = part[0][threadIdx.x] + part[1][threadIdx.x] + part[2][threadIdx.x] + part[3][threadIdx.x];
-        if (m < p.M && n < p.N) c[oc + static_cast<int64_t>(m) * p.c_rs + n] = narrow<D>(v);
+        Acc v = part[0][threadIdx.x] + part[1][threadIdx.x] + part[2][threadIdx.x] + part[3][threadIdx.x];
+        if (m >= p.M || n >= p.N) return;
+        // (a convolution's product: a per-row start value, columns in groups that go image by image)
+        if (p.row_bias) v += static_cast<Acc>(widen(static_cast<const D*>(p.row_bias)[m]));
+        int64_t at = oc + n;
+        if (p.c_group) {
+            uint32_t g, j;
+            p.c_group_div.divmod(n, g, j);
+            if (j >= p.c_group_live) return;
+            at = static_cast<int64_t>(g) * p.c_group_stride + j;
+        }
+        c[at + static_cast<int64_t>(m) * p.c_rs] = narrow<D>(v);
     }
 }
 
@@ -279,6 +289,18 @@ int run_few_results(const GemmProblem& p, const void* a, const void* b, void* c,
     hipLaunchKernelGGL((gemm_generic_few_results_kernel<A, B, D>), dim3(tiles_m * tiles_n, p.batches), dim3(256), 0, stream, static_cast<const A*>(a), static_cast<const B*>(b),
                        static_cast<D*>(c), p, tiles_n);
     return launch_status("gemm_generic_few_results_kernel");
+}
+
+// The same for a caller inside the library (the unfolded batch of a convolution): both operands and the result of one type.
+int gemm_few_results(const GemmProblem& p, int dtype, const void* a, const void* b, void* c, hipStream_t stream) {
+    if (!few_results_under_a_long_k(p, 8192)) return TANNIC_UNSUPPORTED_DTYPE;
+    switch (dtype) {
+        case TANNIC_FLOAT16: return run_few_results<f16, f16, f16>(p, a, b, c, stream);
+        case TANNIC_BFLOAT16: return run_few_results<bf16, bf16, bf16>(p, a, b, c, stream);
+        case TANNIC_FLOAT32: return run_few_results<float, float, float>(p, a, b, c, stream);
+        case TANNIC_FLOAT64: return run_few_results<double, double, double>(p, a, b, c, stream);
+        default: return TANNIC_UNSUPPORTED_DTYPE;
+    }
 }
 
 // c[m * c_rs + n] = t[n * M + m]: the few rows of a transposed result back into the columns they belong to

@@ -87,6 +87,7 @@ int gemm_skinny_16bit(const GemmProblem& p, int dtype, const void* a, const void
 int gemm_skinny_f32(const GemmProblem& p, const float* a, const float* b, float* c, hipStream_t stream);
 int gemm_skinny_int8(const GemmProblem& p, const void* a, const void* b, void* c, hipStream_t stream);
 int gemm_rows_nn(const GemmProblem& p, int dtype, const void* a, const void* b, void* c, hipStream_t stream);
+int gemm_few_results(const GemmProblem& p, int dtype, const void* a, const void* b, void* c, hipStream_t stream);
 int gemm_mfma_f64(const GemmProblem& p, const double* a, const double* b, double* c, hipStream_t stream);
 int gemm_mfma_16bit(const GemmProblem& p, int dtype, const void* a, const void* b, void* c, hipStream_t stream, const GemmWorkspace* workspace = nullptr);
 int gemm_mfma_f32(const GemmProblem& p, const float* a, const float* b, float* c, hipStream_t stream, const GemmWorkspace* workspace = nullptr);

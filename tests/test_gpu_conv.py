@@ -120,6 +120,11 @@ CASES = {
     "unfolded_odd_k_few_pixels": ((3, 116, 8, 8), (40, 116, 5, 5), (2, 2), (2, 2)),
     "unfolded_any_odd_k": ((4, 77, 20, 20), (24, 77, 3, 3), (1, 1), (1, 1)),
     "unfolded_three_channels_out_long_k": ((4, 50, 8, 8), (3, 50, 7, 7), (2, 2), (0, 0)),
+    # ... a handful of pixels in all (the product: a workgroup per 4 x 4 results), one pixel, a K padded with zeros to whole
+    # 16 bytes under many pixels (fp32: beyond the gathering tiles' table)
+    "unfolded_one_image_few_pixels": ((1, 96, 8, 8), (8, 96, 4, 4), (1, 1), (0, 0)),
+    "unfolded_one_pixel_an_image": ((2, 64, 3, 3), (43, 64, 3, 3), (3, 3), (1, 1)),
+    "unfolded_padded_k_many_pixels": ((1, 405, 30, 30), (8, 405, 5, 3), (1, 1), (2, 1)),
     # ... in runs of images when the whole batch unfolded would be large (13 images and 1; one image at a time), with a
     # K beyond what the general tiles keep a table of
     "unfolded_any_runs_of_images": ((14, 128, 40, 40), (4, 128, 7, 7), (1, 1), (3, 3)),
