@@ -612,6 +612,31 @@ int run_reduce(const tannic_tensor_t* src, tannic_tensor_t* dst, hipStream_t str
                                static_cast<uint32_t>(slots));
             return launch_status("reduce_strided_wave_kernel");
         }
+        // Neighbouring lanes are neighbouring results: the last dim that stays.  Where its stride is not 1 (a view with its
+        // outer dims swapped, reduced over the innermost) every lane reads a line of its own; a large view is then copied
+        // into a contiguous tensor first - one transposing pass - and reduced as a slab.
+        int last_kept = -1;
+        for (int d = src->rank - 1; d >= 0 && last_kept < 0; --d)
+            if (d != axis && src->shape.sizes[d] != 1) last_kept = d;
+        const size_t elements = slots * R;
+        if (last_kept >= 0 && src->strides.sizes[last_kept] != 1 && elements >= (1u << 18) && elements < (1ull << 31)) {
+            tannic_tensor_t dense = *src;
+            int64_t pitch = 1;
+            for (int d = src->rank - 1; d >= 0; --d) {
+                dense.strides.sizes[d] = pitch;
+                pitch *= static_cast<int64_t>(src->shape.sizes[d]);
+            }
+            dense.layout = TANNIC_CONTIGUOUS;
+            dense.size = elements;
+            void* copy = nullptr;
+            if (scratch_acquire(&copy, elements * sizeof(T), stream) != TANNIC_SUCCESS) return TANNIC_ERROR;
+            dense.address = copy;
+            tannic_stream_t on{reinterpret_cast<uintptr_t>(stream)};
+            int status = tannic_hip_repack(src, &dense, on);
+            if (status == TANNIC_SUCCESS) status = run_reduce<Op>(&dense, dst, stream, axis);
+            scratch_release(copy, stream);
+            return status;
+        }
         hipLaunchKernelGGL((reduce_strided_kernel<Op>), dim3((slots + kThreads - 1) / kThreads), dim3(kThreads), 0, stream, ps, pd, w,
                            static_cast<uint32_t>(slots));
         return launch_status("reduce_strided_kernel");

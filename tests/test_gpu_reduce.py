@@ -212,7 +212,9 @@ def test_views_that_are_dense_in_another_order_and_rows_of_a_few_elements(device
              ((3000, 16), []), ((1, 900), [("transpose", (0, 1))]),
              # views that are not dense: few results over a long reduced dim take a wavefront each
              ((40, 600, 6), [("index", (slice(0, 40, 2),))]), ((50, 2000), [("index", (slice(None), slice(1, 1999)))]),
-             ((6, 3, 1000), [("index", (slice(None), slice(None), slice(0, 1000, 3)))])]
+             ((6, 3, 1000), [("index", (slice(None), slice(None), slice(0, 1000, 3)))]),
+             # a large view whose neighbouring results lie far apart is copied into a contiguous tensor first
+             ((40, 50, 12, 20), [("transpose", (0, 1))]), ((300, 1100), [("index", (slice(None), slice(0, 1100, 2))), ("transpose", (0, 1))])]
     for shape, spec in cases:
         h, d = support.both(np.round(support.values_for(dtype, SEED, 9, shape, -3, 3).astype(np.float64)), dtype, device)
         hv, dv = support.apply_view(h, spec), support.apply_view(d, spec)
